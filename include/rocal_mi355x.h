@@ -1,0 +1,164 @@
+/*
+ * rocal_mi355x.h - C ABI of the MI355X (gfx950) augmentation hot path for rocAL.
+ *
+ * Every entry point is extern "C" and takes plain pointers, sizes and PODs only. The protocol
+ * follows rocAL's three phases for a node:
+ *
+ *   create   (Node::create_node, user thread, once)        -> rmx_create_<op>()
+ *   update   (Node::update_node, output thread, per batch) -> rmx_update_<op>()  [host arrays in]
+ *   process  (Graph::process = vxProcessGraph, per batch)  -> rmx_op_launch()    [device buffers]
+ *
+ * rmx_update_* packs the per-sample host arrays (the vx_arrays / ROI tensors of the reference)
+ * into one row of a per-batch parameter table and uploads it asynchronously on the context's
+ * stream; rmx_op_launch() enqueues ONE kernel that covers the whole ragged batch. Nothing
+ * blocks except rmx_ctx_sync(). All functions return 0 on success or an rmx_status code;
+ * rmx_last_error() returns the message of the calling thread's last failure.
+ *
+ * Image batches use rocAL's dense tensor model (rocAL/source/pipeline/tensor.cpp:116-137):
+ * [N, Hmax, Wmax, C] (NHWC) or [N, C, Hmax, Wmax] (NCHW), sample i valid inside its ROI.
+ */
+#ifndef ROCAL_MI355X_H
+#define ROCAL_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RMX_API __attribute__((visibility("default")))
+
+typedef struct rmx_ctx rmx_ctx;
+typedef struct rmx_op rmx_op;
+
+enum rmx_status {
+    RMX_OK = 0,
+    RMX_ERR_INVALID = 1,     /* bad argument (message says which) */
+    RMX_ERR_HIP = 2,         /* a HIP runtime call failed (message carries the numeric code) */
+    RMX_ERR_UNSUPPORTED = 3, /* combination outside the hot path (e.g. cubic interpolation) */
+    RMX_ERR_NOMEM = 4
+};
+
+/* rocAL/include/pipeline/commons.h:45-70,110-113 */
+enum { RMX_NHWC = 0, RMX_NCHW = 1 };
+enum { RMX_FP32 = 0, RMX_FP16 = 1, RMX_UINT8 = 2 };
+enum { RMX_ROI_LTRB = 0, RMX_ROI_XYWH = 1 };
+/* rocAL/include/api/rocal_api_types.h:347-366 */
+enum { RMX_INTERP_NEAREST = 0, RMX_INTERP_LINEAR = 1, RMX_INTERP_TRIANGULAR = 5 };
+
+/* flags for resize-family ops */
+enum {
+    RMX_F_QUANTIZE_U8 = 1u << 0 /* round the resampled value to u8 before normalising: reproduces the
+                                   two-node graph resize(u8) -> CropMirrorNormalize in one pass */
+};
+
+/* TensorInfo of one side of a node (rocAL/include/pipeline/tensor.h:65-309): padded maxima. */
+typedef struct rmx_tensor_desc {
+    uint32_t n, h, w, c;
+    int32_t layout; /* RMX_NHWC | RMX_NCHW */
+    int32_t dtype;  /* RMX_FP32 | RMX_FP16 | RMX_UINT8 */
+} rmx_tensor_desc;
+
+/* ---- context: one device + one stream (rocAL/source/device/device_manager_hip.cpp:53-77) ---- */
+/* own_stream != 0: the context creates (and later destroys) its own non-blocking stream and
+ * `stream` is ignored. own_stream == 0: `stream` is a hipStream_t to borrow (NULL = the device's
+ * default stream). */
+RMX_API int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out);
+RMX_API int rmx_ctx_destroy(rmx_ctx *ctx);
+RMX_API int rmx_ctx_sync(rmx_ctx *ctx);
+RMX_API void *rmx_ctx_stream(rmx_ctx *ctx);
+RMX_API const char *rmx_last_error(void);
+RMX_API const char *rmx_version(void);
+
+/* ---- process: replaces vxProcessGraph for one node (rocAL/source/pipeline/graph.cpp:96-103) ---- */
+/* src/dst are device pointers to the batch buffers, borrowed for the duration of the kernel
+ * (rocAL swaps them every batch, rocAL/source/pipeline/tensor.cpp:478-489). Asynchronous. */
+RMX_API int rmx_op_launch(rmx_op *op, const void *src, void *dst);
+RMX_API int rmx_op_destroy(rmx_op *op);
+/* Algorithmic bytes of the last update: sum of source-window bytes + destination bytes. */
+RMX_API uint64_t rmx_op_algorithmic_bytes(const rmx_op *op);
+/* Name of the kernel the op launches (as it appears in a rocprofv3 kernel trace). */
+RMX_API const char *rmx_op_kernel_name(const rmx_op *op);
+
+/* ---- CropMirrorNormalize: replaces vxExtRppCropMirrorNormalize
+ *      (rocAL/source/augmentations/geometry_augmentations/node_crop_mirror_normalize.cpp:87-88).
+ * out[n,c,y,x] = in[n, y1+y, x1+(mirror? cw-1-x : x), c] * scale[n*C+c] + bias[n*C+c] (one fp32 FMA).
+ * rocAL passes bias in its "multiplier" array and scale in its "offset" array (:56-61). */
+RMX_API int rmx_create_crop_mirror_normalize(rmx_ctx *ctx, const rmx_tensor_desc *src,
+                                             const rmx_tensor_desc *dst, int roi_type, rmx_op **out);
+RMX_API int rmx_update_crop_mirror_normalize(rmx_op *op, const uint32_t *crop_roi /*[N][4]*/,
+                                             const float *scale /*[N*C]*/, const float *bias /*[N*C]*/,
+                                             const uint32_t *mirror /*[N]*/);
+
+/* ---- Crop: replaces vxExtRppCrop (node_crop.cpp:47-48, node_random_crop.cpp:47) ---- */
+RMX_API int rmx_create_crop(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                            int roi_type, rmx_op **out);
+RMX_API int rmx_update_crop(rmx_op *op, const uint32_t *crop_roi);
+
+/* ---- Flip: replaces vxExtRppFlip (node_flip.cpp:44-45) ---- */
+RMX_API int rmx_create_flip(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                            int roi_type, rmx_op **out);
+RMX_API int rmx_update_flip(rmx_op *op, const uint32_t *src_roi, const uint32_t *horizontal,
+                            const uint32_t *vertical);
+
+/* ---- Resize family: replaces vxExtRppResize (node_resize.cpp:56-57, node_crop_resize.cpp:60-61),
+ *      vxExtRppResizeCropMirror (node_resize_crop_mirror.cpp:59-60) and
+ *      vxExtRppResizeMirrorNormalize (node_resize_mirror_normalize.cpp:90-92).
+ * mirror, mean, stddev may be NULL (=> no flip / no normalisation). mean/stddev are [N*C];
+ * the kernel computes fmaf(v, 1/std, -(mean*(1/std))). */
+RMX_API int rmx_create_resize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                              int interpolation, int roi_type, uint32_t flags, rmx_op **out);
+RMX_API int rmx_update_resize(rmx_op *op, const uint32_t *src_roi /*[N][4]*/, const uint32_t *dst_w /*[N]*/,
+                              const uint32_t *dst_h /*[N]*/, const uint32_t *mirror, const float *mean,
+                              const float *stddev);
+/* Fused chain resize -> CropMirrorNormalize (the RandomResizedCrop + CMN graph): the resize
+ * target is (dst_w,dst_h); the CMN crop window crop_roi[N][4] (x,y,w,h inside the resized image,
+ * NULL = whole image) selects what is written; scale/bias as in CropMirrorNormalize. */
+RMX_API int rmx_update_resize_cmn(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w,
+                                  const uint32_t *dst_h, const uint32_t *crop_roi, const float *scale,
+                                  const float *bias, const uint32_t *mirror);
+
+/* ---- Colour family (u8 NHWC -> u8 NHWC): replaces vxExtRppColorTwist (node_color_twist.cpp:48-49),
+ *      vxExtRppBrightness (node_brightness.cpp:44), vxExtRppContrast (node_contrast.cpp:44),
+ *      vxExtRppHue (node_hue.cpp:42), vxExtRppSaturation (node_saturation.cpp:42). ---- */
+RMX_API int rmx_create_color_twist(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                   int roi_type, rmx_op **out);
+RMX_API int rmx_update_color_twist(rmx_op *op, const uint32_t *src_roi, const float *alpha,
+                                   const float *beta, const float *hue_deg, const float *sat);
+RMX_API int rmx_create_brightness(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                  int roi_type, rmx_op **out);
+RMX_API int rmx_update_brightness(rmx_op *op, const uint32_t *src_roi, const float *alpha, const float *beta);
+RMX_API int rmx_create_contrast(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                int roi_type, rmx_op **out);
+RMX_API int rmx_update_contrast(rmx_op *op, const uint32_t *src_roi, const float *factor, const float *center);
+RMX_API int rmx_create_hue(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                           int roi_type, rmx_op **out);
+RMX_API int rmx_update_hue(rmx_op *op, const uint32_t *src_roi, const float *hue_deg);
+RMX_API int rmx_create_saturation(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                  int roi_type, rmx_op **out);
+RMX_API int rmx_update_saturation(rmx_op *op, const uint32_t *src_roi, const float *sat);
+
+/* ---- WarpAffine: replaces vxExtRppWarpAffine (node_warp_affine.cpp:61-62). affine is [N][6] in
+ *      rocAL's fill order x0,y0,x1,y1,o0,o1 (:43-48), read as M=[[x0,x1,o0],[y0,y1,o1]] mapping
+ *      destination to source about the ROI / output centres. Out-of-ROI samples give 0. ---- */
+RMX_API int rmx_create_warp_affine(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                   int interpolation, int roi_type, rmx_op **out);
+RMX_API int rmx_update_warp_affine(rmx_op *op, const uint32_t *src_roi, const float *affine /*[N][6]*/,
+                                   const uint32_t *dst_w, const uint32_t *dst_h);
+
+/* ---- Rotate: replaces vxExtRppRotate (node_rotate.cpp:43-44); angle in degrees, direction and
+ *      centre as rocAL/source/meta_data/meta_node_rotate.cpp:53-77. ---- */
+RMX_API int rmx_create_rotate(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                              int interpolation, int roi_type, rmx_op **out);
+RMX_API int rmx_update_rotate(rmx_op *op, const uint32_t *src_roi, const float *angle_deg /*[N]*/,
+                              const uint32_t *dst_w, const uint32_t *dst_h);
+
+/* ---- measurement helper: plain device-to-device streaming copy (nbytes, 16-byte multiples),
+ *      used to establish the copy ceiling of the box and the scale of rocprof's byte counters. */
+RMX_API int rmx_copy_bytes(rmx_ctx *ctx, const void *src, void *dst, size_t nbytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

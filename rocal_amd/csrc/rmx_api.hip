@@ -1,0 +1,689 @@
+// Host side of the C ABI: contexts, ops, the per-batch parameter table and kernel launches.
+// One op = one node of the reference graph (create_node / update_node / process phases).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "rmx_common.h"
+#include "rmx_launch.h"
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess)                                                                      \
+            return fail(RMX_ERR_HIP, "%s failed: %d (%s)", #expr, (int)e_, hipGetErrorString(e_)); \
+    } while (0)
+
+enum OpKind {
+    OP_CMN = 1, OP_CROP, OP_FLIP, OP_RESIZE, OP_COLOR_TWIST, OP_BRIGHTNESS, OP_CONTRAST, OP_HUE,
+    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE
+};
+
+constexpr int TABLE_RING = 4;  // updates in flight before the host has to wait on an old upload
+
+}  // namespace
+
+struct rmx_ctx {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool owns_stream = false;
+    int num_cus = 256;
+    int max_lds_per_block = 65536;
+};
+
+struct rmx_op {
+    rmx_ctx *ctx = nullptr;
+    int kind = 0;
+    rmx_tensor_desc src{}, dst{};
+    int interp = RMX_INTERP_LINEAR;
+    int roi_type = RMX_ROI_XYWH;
+    uint32_t flags = 0;
+    bool norm = false, quant = false;
+    int n = 0;
+
+    RmxSample *h_table[TABLE_RING] = {};  // pinned
+    RmxSample *d_table[TABLE_RING] = {};
+    hipEvent_t uploaded[TABLE_RING] = {};
+    int cur = -1;  // slot of the last update, -1 before the first
+
+    // launch plan of the last update
+    rmx::KernelFn fn = nullptr;
+    const char *kernel_name = "";
+    int strips = 1, strip_rows = 1, tile_w = 512, lds_per_wave = 0, waves_per_block = 4;
+    int aux0 = 0, aux1 = 0;
+    uint64_t algo_bytes = 0;
+};
+
+namespace {
+
+int check_desc(const rmx_tensor_desc *d, const char *what) {
+    if (!d) return fail(RMX_ERR_INVALID, "%s descriptor is NULL", what);
+    if (d->n == 0 || d->h == 0 || d->w == 0) return fail(RMX_ERR_INVALID, "%s descriptor has a zero dimension", what);
+    if (d->c != 3) return fail(RMX_ERR_UNSUPPORTED, "%s: only 3-channel (RGB) tensors are on the hot path (c=%u)", what, d->c);
+    if (d->layout != RMX_NHWC && d->layout != RMX_NCHW) return fail(RMX_ERR_UNSUPPORTED, "%s: layout %d not supported", what, d->layout);
+    if (d->dtype != RMX_FP32 && d->dtype != RMX_FP16 && d->dtype != RMX_UINT8) return fail(RMX_ERR_UNSUPPORTED, "%s: dtype %d not supported", what, d->dtype);
+    return RMX_OK;
+}
+
+int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    if (!ctx) return fail(RMX_ERR_INVALID, "context is NULL");
+    if (!out) return fail(RMX_ERR_INVALID, "output handle pointer is NULL");
+    *out = nullptr;
+    int rc;
+    if ((rc = check_desc(src, "source"))) return rc;
+    if ((rc = check_desc(dst, "destination"))) return rc;
+    if (src->dtype != RMX_UINT8 || src->layout != RMX_NHWC)
+        return fail(RMX_ERR_UNSUPPORTED, "source must be uint8 NHWC (decoded RGB batch)");
+    if (src->n != dst->n) return fail(RMX_ERR_INVALID, "batch size mismatch: source %u, destination %u", src->n, dst->n);
+    if (roi_type != RMX_ROI_LTRB && roi_type != RMX_ROI_XYWH) return fail(RMX_ERR_INVALID, "roi_type %d invalid", roi_type);
+    HIP_TRY(hipSetDevice(ctx->device));
+    rmx_op *op = new (std::nothrow) rmx_op();
+    if (!op) return fail(RMX_ERR_NOMEM, "out of host memory");
+    op->ctx = ctx;
+    op->kind = kind;
+    op->src = *src;
+    op->dst = *dst;
+    op->roi_type = roi_type;
+    op->n = (int)src->n;
+    size_t bytes = sizeof(RmxSample) * (size_t)op->n;
+    for (int i = 0; i < TABLE_RING; i++) {
+        hipError_t e = hipHostMalloc((void **)&op->h_table[i], bytes, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipMalloc((void **)&op->d_table[i], bytes);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&op->uploaded[i], hipEventDisableTiming);
+        if (e != hipSuccess) {
+            rmx_op_destroy(op);
+            return fail(RMX_ERR_HIP, "allocating the parameter table failed: %d (%s)", (int)e, hipGetErrorString(e));
+        }
+        memset(op->h_table[i], 0, bytes);
+    }
+    *out = op;
+    return RMX_OK;
+}
+
+// Next table slot; waits until the upload that last used it has completed.
+int next_slot(rmx_op *op, RmxSample **row) {
+    int slot = (op->cur + 1) % TABLE_RING;
+    HIP_TRY(hipSetDevice(op->ctx->device));
+    HIP_TRY(hipEventSynchronize(op->uploaded[slot]));
+    *row = op->h_table[slot];
+    return slot;
+}
+
+int commit_slot(rmx_op *op, int slot) {
+    HIP_TRY(hipMemcpyAsync(op->d_table[slot], op->h_table[slot], sizeof(RmxSample) * (size_t)op->n,
+                           hipMemcpyHostToDevice, op->ctx->stream));
+    HIP_TRY(hipEventRecord(op->uploaded[slot], op->ctx->stream));
+    op->cur = slot;
+    return RMX_OK;
+}
+
+// ROI in the caller's convention -> x,y,w,h clipped to the padded source tensor.
+int read_roi(const rmx_op *op, const uint32_t *roi, int i, int32_t *x, int32_t *y, int32_t *w, int32_t *h) {
+    if (!roi) {
+        *x = 0; *y = 0; *w = (int32_t)op->src.w; *h = (int32_t)op->src.h;
+        return RMX_OK;
+    }
+    uint32_t a = roi[i * 4], b = roi[i * 4 + 1], c = roi[i * 4 + 2], d = roi[i * 4 + 3];
+    if (op->roi_type == RMX_ROI_LTRB) {  // l,t,r,b with r,b exclusive bounds as rocAL's width/height users read them
+        if (c < a || d < b) return fail(RMX_ERR_INVALID, "sample %d: LTRB roi has r<l or b<t", i);
+        c -= a;
+        d -= b;
+    }
+    if (a >= op->src.w || b >= op->src.h) return fail(RMX_ERR_INVALID, "sample %d: roi origin (%u,%u) outside the %ux%u source", i, a, b, op->src.w, op->src.h);
+    if (c > op->src.w - a) c = op->src.w - a;
+    if (d > op->src.h - b) d = op->src.h - b;
+    *x = (int32_t)a; *y = (int32_t)b; *w = (int32_t)c; *h = (int32_t)d;
+    return RMX_OK;
+}
+
+size_t dtype_size(int dtype) { return dtype == RMX_FP32 ? 4 : dtype == RMX_FP16 ? 2 : 1; }
+
+void plan_streaming(rmx_op *op, int max_rows, int rows_per_strip) {
+    op->strip_rows = rows_per_strip;
+    op->strips = std::max(1, (max_rows + rows_per_strip - 1) / rows_per_strip);
+    op->aux0 = rows_per_strip;
+    op->lds_per_wave = 0;
+    op->waves_per_block = 4;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *rmx_last_error(void) { return g_err.c_str(); }
+const char *rmx_version(void) { return "rocal-mi355x 0.1 (gfx950)"; }
+
+int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
+    if (!out) return fail(RMX_ERR_INVALID, "output handle pointer is NULL");
+    *out = nullptr;
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if (device < 0 || device >= count) return fail(RMX_ERR_INVALID, "device %d out of range (have %d)", device, count);
+    HIP_TRY(hipSetDevice(device));
+    rmx_ctx *ctx = new (std::nothrow) rmx_ctx();
+    if (!ctx) return fail(RMX_ERR_NOMEM, "out of host memory");
+    ctx->device = device;
+    if (!own_stream) {
+        ctx->stream = (hipStream_t)stream;
+    } else {
+        hipError_t e = hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking);
+        if (e != hipSuccess) {
+            delete ctx;
+            return fail(RMX_ERR_HIP, "hipStreamCreateWithFlags failed: %d (%s)", (int)e, hipGetErrorString(e));
+        }
+        ctx->owns_stream = true;
+    }
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) == hipSuccess) {
+        ctx->num_cus = prop.multiProcessorCount;
+        ctx->max_lds_per_block = (int)prop.sharedMemPerBlock;
+    }
+    *out = ctx;
+    return RMX_OK;
+}
+
+int rmx_ctx_destroy(rmx_ctx *ctx) {
+    if (!ctx) return RMX_OK;
+    if (ctx->owns_stream) {
+        (void)hipStreamSynchronize(ctx->stream);
+        (void)hipStreamDestroy(ctx->stream);
+    }
+    delete ctx;
+    return RMX_OK;
+}
+
+int rmx_ctx_sync(rmx_ctx *ctx) {
+    if (!ctx) return fail(RMX_ERR_INVALID, "context is NULL");
+    HIP_TRY(hipStreamSynchronize(ctx->stream));
+    return RMX_OK;
+}
+
+void *rmx_ctx_stream(rmx_ctx *ctx) { return ctx ? (void *)ctx->stream : nullptr; }
+
+int rmx_op_destroy(rmx_op *op) {
+    if (!op) return RMX_OK;
+    (void)hipSetDevice(op->ctx->device);
+    (void)hipStreamSynchronize(op->ctx->stream);
+    for (int i = 0; i < TABLE_RING; i++) {
+        if (op->uploaded[i]) (void)hipEventDestroy(op->uploaded[i]);
+        if (op->h_table[i]) (void)hipHostFree(op->h_table[i]);
+        if (op->d_table[i]) (void)hipFree(op->d_table[i]);
+    }
+    delete op;
+    return RMX_OK;
+}
+
+uint64_t rmx_op_algorithmic_bytes(const rmx_op *op) { return op ? op->algo_bytes : 0; }
+const char *rmx_op_kernel_name(const rmx_op *op) { return op ? op->kernel_name : ""; }
+
+int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
+    if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
+    if (!src || !dst) return fail(RMX_ERR_INVALID, "source/destination buffer is NULL");
+    if (op->cur < 0 || !op->fn) return fail(RMX_ERR_INVALID, "op launched before its first update");
+    RmxKArgs a{};
+    a.src = (const uint8_t *)src;
+    a.dst = dst;
+    a.table = op->d_table[op->cur];
+    a.src_bytes = (uint64_t)op->src.n * op->src.h * op->src.w * op->src.c;
+    a.n = op->n;
+    a.src_h = (int)op->src.h;
+    a.src_w = (int)op->src.w;
+    a.dst_h = (int)op->dst.h;
+    a.dst_w = (int)op->dst.w;
+    a.strips = op->strips;
+    a.lds_bytes = op->lds_per_wave;
+    a.aux0 = op->aux0;
+    a.aux1 = op->aux1;
+    const uint64_t waves = (uint64_t)op->n * (uint64_t)op->strips;
+    const int wpb = op->waves_per_block;
+    const uint64_t blocks = (waves + wpb - 1) / wpb;
+    if (blocks == 0 || blocks > 0x7fffffffull) return fail(RMX_ERR_INVALID, "grid of %llu workgroups is out of range", (unsigned long long)blocks);
+    const size_t lds = (size_t)op->lds_per_wave * wpb;
+    if (lds > (size_t)op->ctx->max_lds_per_block) return fail(RMX_ERR_INVALID, "plan needs %zu bytes of LDS per workgroup (limit %d)", lds, op->ctx->max_lds_per_block);
+    HIP_TRY(hipSetDevice(op->ctx->device));
+    hipLaunchKernelGGL(op->fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
+    HIP_TRY(hipGetLastError());
+    return RMX_OK;
+}
+
+/* ------------------------------------------------------------------ K1 family */
+
+static int create_k1(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, bool norm, rmx_op **out) {
+    int rc = make_op(ctx, kind, src, dst, roi_type, out);
+    if (rc) return rc;
+    (*out)->norm = norm;
+    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, norm, &(*out)->kernel_name);
+    return RMX_OK;
+}
+
+static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const float *bias, const uint32_t *hflip, const uint32_t *vflip) {
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    uint64_t bytes = 0;
+    int max_rows = 1;
+    for (int i = 0; i < op->n; i++) {
+        RmxSample &s = t[i];
+        int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+        if (rc) return rc;
+        s.dst_w = std::min<int32_t>(s.src_w, (int32_t)op->dst.w);
+        s.dst_h = std::min<int32_t>(s.src_h, (int32_t)op->dst.h);
+        s.src_w = s.dst_w;
+        s.src_h = s.dst_h;
+        s.flags = ((hflip && hflip[i]) ? RMX_S_HFLIP : 0u) | ((vflip && vflip[i]) ? RMX_S_VFLIP : 0u);
+        for (int c = 0; c < 3; c++) {
+            s.scale[c] = scale ? scale[i * 3 + c] : 1.0f;
+            s.bias[c] = bias ? bias[i * 3 + c] : 0.0f;
+        }
+        bytes += (uint64_t)s.dst_w * s.dst_h * 3 * (1 + dtype_size(op->dst.dtype));
+        max_rows = std::max(max_rows, (int)s.dst_h);
+    }
+    op->algo_bytes = bytes;
+    plan_streaming(op, max_rows, 8);
+    return commit_slot(op, slot);
+}
+
+int rmx_create_crop_mirror_normalize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_k1(ctx, OP_CMN, src, dst, roi_type, true, out);
+}
+
+int rmx_update_crop_mirror_normalize(rmx_op *op, const uint32_t *crop_roi, const float *scale, const float *bias, const uint32_t *mirror) {
+    if (!op || op->kind != OP_CMN) return fail(RMX_ERR_INVALID, "op is not a CropMirrorNormalize node");
+    if (!crop_roi || !scale || !bias) return fail(RMX_ERR_INVALID, "crop_roi, scale and bias arrays are required");
+    return update_k1(op, crop_roi, scale, bias, mirror, nullptr);
+}
+
+int rmx_create_crop(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_k1(ctx, OP_CROP, src, dst, roi_type, false, out);
+}
+
+int rmx_update_crop(rmx_op *op, const uint32_t *crop_roi) {
+    if (!op || op->kind != OP_CROP) return fail(RMX_ERR_INVALID, "op is not a Crop node");
+    if (!crop_roi) return fail(RMX_ERR_INVALID, "crop_roi array is required");
+    return update_k1(op, crop_roi, nullptr, nullptr, nullptr, nullptr);
+}
+
+int rmx_create_flip(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_k1(ctx, OP_FLIP, src, dst, roi_type, false, out);
+}
+
+int rmx_update_flip(rmx_op *op, const uint32_t *src_roi, const uint32_t *horizontal, const uint32_t *vertical) {
+    if (!op || op->kind != OP_FLIP) return fail(RMX_ERR_INVALID, "op is not a Flip node");
+    return update_k1(op, src_roi, nullptr, nullptr, horizontal, vertical);
+}
+
+/* ------------------------------------------------------------------ K2 family */
+
+int rmx_create_resize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int interpolation, int roi_type, uint32_t flags, rmx_op **out) {
+    if (interpolation != RMX_INTERP_LINEAR && interpolation != RMX_INTERP_NEAREST && interpolation != RMX_INTERP_TRIANGULAR) {
+        if (out) *out = nullptr;
+        return fail(RMX_ERR_UNSUPPORTED, "interpolation %d is outside the hot path (nearest=0, linear=1, triangular=5)", interpolation);
+    }
+    int rc = make_op(ctx, OP_RESIZE, src, dst, roi_type, out);
+    if (rc) return rc;
+    (*out)->interp = interpolation;
+    (*out)->flags = flags;
+    return RMX_OK;
+}
+
+static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
+    const bool quant = (op->flags & RMX_F_QUANTIZE_U8) != 0;
+    // a quantised value that is not normalised is stored through an identity FMA
+    const bool knorm = norm || (quant && op->dst.dtype != RMX_UINT8);
+    op->norm = knorm;
+    op->quant = quant && knorm;
+    int max_dw = 1, max_dh = 1;
+    for (int i = 0; i < op->n; i++) {
+        max_dw = std::max(max_dw, (int)t[i].dst_w);
+        max_dh = std::max(max_dh, (int)t[i].dst_h);
+    }
+    if (op->interp == RMX_INTERP_TRIANGULAR) {
+        op->fn = rmx::select_resize_tri_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
+        if (!op->fn) return fail(RMX_ERR_UNSUPPORTED, "triangular resize kernel not available");
+        // 128 output columns per wave (two per lane); ring of horizontally filtered rows per wave
+        const int tile_w = 128;
+        float max_ry = 1.0f, max_rx = 1.0f;
+        for (int i = 0; i < op->n; i++) {
+            if (t[i].dst_w <= 0 || t[i].dst_h <= 0) continue;
+            max_rx = std::max(max_rx, t[i].rx);
+            max_ry = std::max(max_ry, t[i].ry);
+        }
+        const int ky = (int)std::ceil(2.0f * max_ry);
+        const int kx_cap = (int)std::ceil(2.0f * max_rx);
+        int ring_rows = 2;
+        while (ring_rows < ky + 1) ring_rows *= 2;
+        const int src_cols = std::min<int>((int)op->src.w, (int)std::ceil(tile_w * (double)max_rx) + kx_cap + 4);
+        const int src_pitch = ((src_cols + 3) / 4) * 4 + 8;
+        // LDS slice: coef[kx_cap][128] | ring[ring_rows][3][128] | srcrow[src_pitch]
+        size_t words = (size_t)kx_cap * tile_w + (size_t)ring_rows * 3 * tile_w + src_pitch;
+        op->lds_per_wave = (int)((words * 4 + 15) / 16 * 16);
+        if (op->lds_per_wave > op->ctx->max_lds_per_block || kx_cap > 0xffff)
+            return fail(RMX_ERR_UNSUPPORTED, "triangular resize with scale %.1f x %.1f needs %d bytes of LDS per wave", max_rx, max_ry, op->lds_per_wave);
+        op->waves_per_block = std::max(1, std::min(4, op->ctx->max_lds_per_block / op->lds_per_wave));
+        op->tile_w = tile_w;
+        const int xtiles = (max_dw + tile_w - 1) / tile_w;
+        op->aux1 = xtiles;
+        op->strip_rows = 12;
+        op->aux0 = op->strip_rows;
+        const int ystrips = (max_dh + op->strip_rows - 1) / op->strip_rows;
+        op->strips = xtiles * ystrips;
+        for (int i = 0; i < op->n; i++) t[i].strip_rows = (ring_rows << 16) | kx_cap;
+        return RMX_OK;
+    }
+    const char *nm = nullptr;
+    op->fn = (op->interp == RMX_INTERP_NEAREST)
+                 ? rmx::select_resize_nearest_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm)
+                 : rmx::select_resize_linear_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm);
+    op->kernel_name = nm;
+    // x-tile: up to 64 lanes x 8 px; LDS per wave = rows x (staged columns + pads) dwords
+    int tile_w = std::min(((max_dw + 7) / 8) * 8, 512);
+    const int budget = 24 * 1024;
+    int lds = 0;
+    for (;;) {
+        lds = 0;
+        for (int i = 0; i < op->n; i++) {
+            const RmxSample &s = t[i];
+            if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+            for (int pass = 0; pass < 2; pass++) {
+                int tw = pass == 0 ? std::min<int>(tile_w, s.dst_w) : (s.dst_w % tile_w);
+                if (tw <= 0) continue;
+                int L = (tw + 7) / 8, G = 64 / L;
+                int rows = (int)std::ceil((G - 1) * (double)s.ry) + 4;
+                int cols = std::min<int>(s.src_w, (int)std::ceil(tw * (double)s.rx) + 3);
+                int pitch = 4 + ((cols + 3) / 4) * 4 + 4;
+                lds = std::max(lds, rows * pitch * 4);
+            }
+        }
+        if (lds <= budget || tile_w <= 64) break;
+        tile_w = std::max(64, (tile_w / 2 + 7) / 8 * 8);
+    }
+    op->lds_per_wave = (lds + 15) / 16 * 16;
+    if (op->lds_per_wave > op->ctx->max_lds_per_block)
+        return fail(RMX_ERR_UNSUPPORTED, "resize plan needs %d bytes of LDS per wave", op->lds_per_wave);
+    op->waves_per_block = std::max(1, std::min(4, op->ctx->max_lds_per_block / std::max(1, op->lds_per_wave)));
+    op->tile_w = tile_w;
+    op->aux1 = tile_w;
+    op->strip_rows = 8;
+    op->aux0 = op->strip_rows;
+    op->strips = std::max(1, (max_dh + op->strip_rows - 1) / op->strip_rows);
+    return RMX_OK;
+}
+
+static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                                const uint32_t *crop_roi, const float *scale, const float *bias,
+                                const float *mean, const float *stddev, const uint32_t *mirror) {
+    if (!op || op->kind != OP_RESIZE) return fail(RMX_ERR_INVALID, "op is not a Resize node");
+    if (!dst_w || !dst_h) return fail(RMX_ERR_INVALID, "dst_w and dst_h arrays are required");
+    if ((mean == nullptr) != (stddev == nullptr)) return fail(RMX_ERR_INVALID, "mean and stddev must be given together");
+    if ((scale == nullptr) != (bias == nullptr)) return fail(RMX_ERR_INVALID, "scale and bias must be given together");
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    uint64_t bytes = 0;
+    for (int i = 0; i < op->n; i++) {
+        RmxSample &s = t[i];
+        int rc = read_roi(op, src_roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+        if (rc) return rc;
+        s.rs_w = (int32_t)dst_w[i];
+        s.rs_h = (int32_t)dst_h[i];
+        if (s.rs_w < 0 || s.rs_h < 0) return fail(RMX_ERR_INVALID, "sample %d: destination size out of range", i);
+        if (crop_roi) {
+            uint32_t cx = crop_roi[i * 4], cy = crop_roi[i * 4 + 1], cw = crop_roi[i * 4 + 2], chh = crop_roi[i * 4 + 3];
+            if (cx > (uint32_t)s.rs_w || cy > (uint32_t)s.rs_h) return fail(RMX_ERR_INVALID, "sample %d: crop origin outside the resized image", i);
+            s.pc_x = (int32_t)cx;
+            s.pc_y = (int32_t)cy;
+            s.dst_w = (int32_t)std::min<uint32_t>(cw, (uint32_t)s.rs_w - cx);
+            s.dst_h = (int32_t)std::min<uint32_t>(chh, (uint32_t)s.rs_h - cy);
+        } else {
+            s.pc_x = s.pc_y = 0;
+            s.dst_w = s.rs_w;
+            s.dst_h = s.rs_h;
+        }
+        s.dst_w = std::min<int32_t>(s.dst_w, (int32_t)op->dst.w);
+        s.dst_h = std::min<int32_t>(s.dst_h, (int32_t)op->dst.h);
+        if (s.src_w <= 0 || s.src_h <= 0 || s.rs_w <= 0 || s.rs_h <= 0) s.dst_w = s.dst_h = 0;
+        s.flags = (mirror && mirror[i]) ? RMX_S_HFLIP : 0u;
+        if (s.dst_w > 0) {
+            s.rx = (float)s.src_w / (float)s.rs_w;
+            s.ry = (float)s.src_h / (float)s.rs_h;
+            s.fsx = s.rx > 1.0f ? 1 / s.rx : 1.0f;
+            s.fsy = s.ry > 1.0f ? 1 / s.ry : 1.0f;
+        } else {
+            s.rx = s.ry = s.fsx = s.fsy = 1.0f;
+        }
+        for (int c = 0; c < 3; c++) {
+            if (scale) {
+                s.scale[c] = scale[i * 3 + c];
+                s.bias[c] = bias[i * 3 + c];
+            } else if (mean) {
+                if (stddev[i * 3 + c] == 0.0f) return fail(RMX_ERR_INVALID, "sample %d: standard deviation of channel %d is 0", i, c);
+                float inv = 1 / stddev[i * 3 + c];
+                s.scale[c] = inv;
+                s.bias[c] = -(mean[i * 3 + c] * inv);
+            } else {
+                s.scale[c] = 1.0f;
+                s.bias[c] = 0.0f;
+            }
+        }
+        // bytes of the source window actually mapped by the written window
+        double fx = s.rs_w > 0 ? (double)s.dst_w / s.rs_w : 0, fy = s.rs_h > 0 ? (double)s.dst_h / s.rs_h : 0;
+        bytes += (uint64_t)std::llround((double)s.src_w * s.src_h * fx * fy) * 3 +
+                 (uint64_t)s.dst_w * s.dst_h * 3 * dtype_size(op->dst.dtype);
+    }
+    op->algo_bytes = bytes;
+    int rc = plan_resize(op, t, scale != nullptr || mean != nullptr);
+    if (rc) return rc;
+    return commit_slot(op, slot);
+}
+
+int rmx_update_resize(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                      const uint32_t *mirror, const float *mean, const float *stddev) {
+    return update_resize_common(op, src_roi, dst_w, dst_h, nullptr, nullptr, nullptr, mean, stddev, mirror);
+}
+
+int rmx_update_resize_cmn(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                          const uint32_t *crop_roi, const float *scale, const float *bias, const uint32_t *mirror) {
+    if (!scale || !bias) return fail(RMX_ERR_INVALID, "scale and bias arrays are required");
+    return update_resize_common(op, src_roi, dst_w, dst_h, crop_roi, scale, bias, nullptr, nullptr, mirror);
+}
+
+/* ------------------------------------------------------------------ K3 family */
+
+static int create_color(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    int rc = make_op(ctx, kind, src, dst, roi_type, out);
+    if (rc) return rc;
+    const bool twist = (kind == OP_COLOR_TWIST || kind == OP_HUE || kind == OP_SATURATION);
+    (*out)->fn = rmx::select_color_kernel(twist ? 1 : 0, dst->dtype, dst->layout, &(*out)->kernel_name);
+    return RMX_OK;
+}
+
+// hue in degrees -> shift in sextants reduced to [0,6]
+static float hue_to_sextants(float hue_deg) {
+    float s = std::fmod(hue_deg, 360.0f);
+    if (s < 0.0f) s += 360.0f;
+    return s / 60.0f;
+}
+
+static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const float *p1, const float *p2, const float *p3,
+                        float d0, float d1, float d2, float d3, bool hue_in_p2) {
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    uint64_t bytes = 0;
+    int max_rows = 1;
+    for (int i = 0; i < op->n; i++) {
+        RmxSample &s = t[i];
+        int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+        if (rc) return rc;
+        s.dst_w = std::min<int32_t>(s.src_w, (int32_t)op->dst.w);
+        s.dst_h = std::min<int32_t>(s.src_h, (int32_t)op->dst.h);
+        s.flags = 0;
+        s.color[0] = p0 ? p0[i] : d0;
+        s.color[1] = p1 ? p1[i] : d1;
+        s.color[2] = p2 ? (hue_in_p2 ? hue_to_sextants(p2[i]) : p2[i]) : d2;
+        s.color[3] = p3 ? p3[i] : d3;
+        bytes += (uint64_t)s.dst_w * s.dst_h * 3 * (1 + dtype_size(op->dst.dtype));
+        max_rows = std::max(max_rows, (int)s.dst_h);
+    }
+    op->algo_bytes = bytes;
+    plan_streaming(op, max_rows, 8);
+    return commit_slot(op, slot);
+}
+
+int rmx_create_color_twist(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_color(ctx, OP_COLOR_TWIST, src, dst, roi_type, out);
+}
+int rmx_update_color_twist(rmx_op *op, const uint32_t *src_roi, const float *alpha, const float *beta, const float *hue_deg, const float *sat) {
+    if (!op || op->kind != OP_COLOR_TWIST) return fail(RMX_ERR_INVALID, "op is not a ColorTwist node");
+    if (!alpha || !beta || !hue_deg || !sat) return fail(RMX_ERR_INVALID, "alpha, beta, hue and sat arrays are required");
+    return update_color(op, src_roi, alpha, beta, hue_deg, sat, 1, 0, 0, 1, true);
+}
+int rmx_create_brightness(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_color(ctx, OP_BRIGHTNESS, src, dst, roi_type, out);
+}
+int rmx_update_brightness(rmx_op *op, const uint32_t *src_roi, const float *alpha, const float *beta) {
+    if (!op || op->kind != OP_BRIGHTNESS) return fail(RMX_ERR_INVALID, "op is not a Brightness node");
+    if (!alpha || !beta) return fail(RMX_ERR_INVALID, "alpha and beta arrays are required");
+    return update_color(op, src_roi, alpha, beta, nullptr, nullptr, 1, 0, 0, 0, false);
+}
+int rmx_create_contrast(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_color(ctx, OP_CONTRAST, src, dst, roi_type, out);
+}
+int rmx_update_contrast(rmx_op *op, const uint32_t *src_roi, const float *factor, const float *center) {
+    if (!op || op->kind != OP_CONTRAST) return fail(RMX_ERR_INVALID, "op is not a Contrast node");
+    if (!factor || !center) return fail(RMX_ERR_INVALID, "factor and center arrays are required");
+    // out = fma(x - center, factor, center)
+    return update_color(op, src_roi, factor, center, center, nullptr, 1, 0, 0, 0, false);
+}
+int rmx_create_hue(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_color(ctx, OP_HUE, src, dst, roi_type, out);
+}
+int rmx_update_hue(rmx_op *op, const uint32_t *src_roi, const float *hue_deg) {
+    if (!op || op->kind != OP_HUE) return fail(RMX_ERR_INVALID, "op is not a Hue node");
+    if (!hue_deg) return fail(RMX_ERR_INVALID, "hue array is required");
+    return update_color(op, src_roi, nullptr, nullptr, hue_deg, nullptr, 1, 0, 0, 1, true);
+}
+int rmx_create_saturation(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_color(ctx, OP_SATURATION, src, dst, roi_type, out);
+}
+int rmx_update_saturation(rmx_op *op, const uint32_t *src_roi, const float *sat) {
+    if (!op || op->kind != OP_SATURATION) return fail(RMX_ERR_INVALID, "op is not a Saturation node");
+    if (!sat) return fail(RMX_ERR_INVALID, "sat array is required");
+    return update_color(op, src_roi, nullptr, nullptr, nullptr, sat, 1, 0, 0, 1, true);
+}
+
+/* ------------------------------------------------------------------ K4 family */
+
+static int create_warp(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int interpolation, int roi_type, rmx_op **out) {
+    if (interpolation != RMX_INTERP_LINEAR && interpolation != RMX_INTERP_NEAREST) {
+        if (out) *out = nullptr;
+        return fail(RMX_ERR_UNSUPPORTED, "warp interpolation %d is outside the hot path (nearest=0, linear=1)", interpolation);
+    }
+    int rc = make_op(ctx, kind, src, dst, roi_type, out);
+    if (rc) return rc;
+    (*out)->interp = interpolation;
+    (*out)->fn = rmx::select_warp_kernel(interpolation, dst->dtype, dst->layout, &(*out)->kernel_name);
+    return RMX_OK;
+}
+
+static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, const float *angle, const uint32_t *dst_w, const uint32_t *dst_h) {
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    uint64_t bytes = 0;
+    int max_dw = 1, max_dh = 1;
+    double worst_box = 0;
+    for (int i = 0; i < op->n; i++) {
+        RmxSample &s = t[i];
+        int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+        if (rc) return rc;
+        s.dst_w = std::min<int32_t>(dst_w ? (int32_t)dst_w[i] : s.src_w, (int32_t)op->dst.w);
+        s.dst_h = std::min<int32_t>(dst_h ? (int32_t)dst_h[i] : s.src_h, (int32_t)op->dst.h);
+        if (s.src_w <= 0 || s.src_h <= 0) s.dst_w = s.dst_h = 0;
+        s.flags = 0;
+        if (affine) {
+            // rocAL's fill order x0,y0,x1,y1,o0,o1 -> M = [[x0,x1,o0],[y0,y1,o1]]
+            const float *a = affine + i * 6;
+            s.m[0] = a[0]; s.m[1] = a[2]; s.m[2] = a[4];
+            s.m[3] = a[1]; s.m[4] = a[3]; s.m[5] = a[5];
+        } else {
+            float rad = angle[i] * 0.017453292519943295f;
+            float c = std::cos(rad), sn = std::sin(rad);
+            s.m[0] = c;  s.m[1] = -sn; s.m[2] = 0.0f;
+            s.m[3] = sn; s.m[4] = c;   s.m[5] = 0.0f;
+        }
+        bytes += (uint64_t)s.src_w * s.src_h * 3 + (uint64_t)s.dst_w * s.dst_h * 3 * dtype_size(op->dst.dtype);
+        max_dw = std::max(max_dw, (int)s.dst_w);
+        max_dh = std::max(max_dh, (int)s.dst_h);
+        // LDS need of a 32x16 destination tile: bounding box of its image under M, plus margins
+        double bw = 32.0 * std::fabs(s.m[0]) + 16.0 * std::fabs(s.m[1]) + 5.0;
+        double bh = 32.0 * std::fabs(s.m[3]) + 16.0 * std::fabs(s.m[4]) + 5.0;
+        if (std::isfinite(bw) && std::isfinite(bh)) {
+            bw = std::min(bw, (double)s.src_w);
+            bh = std::min(bh, (double)s.src_h);
+            worst_box = std::max(worst_box, (std::ceil(bw / 4) * 4 + 4) * bh);
+        }
+    }
+    op->algo_bytes = bytes;
+    const int cap = 16 * 1024;  // per wave; bigger boxes fall back to global gathers inside the kernel
+    int need = (int)std::min<double>(worst_box * 4, (double)cap);
+    op->lds_per_wave = std::max(256, (need + 15) / 16 * 16);
+    op->waves_per_block = 4;
+    const int tiles_x = (max_dw + 31) / 32, tiles_y = (max_dh + 15) / 16;
+    op->strips = tiles_x * tiles_y;
+    op->aux0 = tiles_x;
+    op->aux1 = tiles_y;
+    return commit_slot(op, slot);
+}
+
+int rmx_create_warp_affine(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int interpolation, int roi_type, rmx_op **out) {
+    return create_warp(ctx, OP_WARP_AFFINE, src, dst, interpolation, roi_type, out);
+}
+int rmx_update_warp_affine(rmx_op *op, const uint32_t *src_roi, const float *affine, const uint32_t *dst_w, const uint32_t *dst_h) {
+    if (!op || op->kind != OP_WARP_AFFINE) return fail(RMX_ERR_INVALID, "op is not a WarpAffine node");
+    if (!affine) return fail(RMX_ERR_INVALID, "affine array is required");
+    return update_warp(op, src_roi, affine, nullptr, dst_w, dst_h);
+}
+int rmx_create_rotate(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int interpolation, int roi_type, rmx_op **out) {
+    return create_warp(ctx, OP_ROTATE, src, dst, interpolation, roi_type, out);
+}
+int rmx_update_rotate(rmx_op *op, const uint32_t *src_roi, const float *angle_deg, const uint32_t *dst_w, const uint32_t *dst_h) {
+    if (!op || op->kind != OP_ROTATE) return fail(RMX_ERR_INVALID, "op is not a Rotate node");
+    if (!angle_deg) return fail(RMX_ERR_INVALID, "angle array is required");
+    return update_warp(op, src_roi, nullptr, angle_deg, dst_w, dst_h);
+}
+
+/* ------------------------------------------------------------------ measurement helper */
+
+int rmx_copy_bytes(rmx_ctx *ctx, const void *src, void *dst, size_t nbytes) {
+    if (!ctx || !src || !dst) return fail(RMX_ERR_INVALID, "context/source/destination is NULL");
+    if (nbytes % 16 != 0) return fail(RMX_ERR_INVALID, "nbytes must be a multiple of 16");
+    if ((((uintptr_t)src) | ((uintptr_t)dst)) & 15u) return fail(RMX_ERR_INVALID, "buffers must be 16-byte aligned");
+    HIP_TRY(hipSetDevice(ctx->device));
+    rmx::launch_copy(ctx->stream, src, dst, nbytes, ctx->num_cus);
+    HIP_TRY(hipGetLastError());
+    return RMX_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,42 @@
+// Shared host/device definitions of the MI355X augmentation library: the per-sample row of
+// the per-batch parameter table, kernel launch arguments and host-side bookkeeping.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include "../../include/rocal_mi355x.h"
+
+// One row per sample; the whole batch's table is uploaded once per update and every
+// workgroup reads its sample's row with scalar loads (the row index is wave-uniform).
+struct __attribute__((aligned(16))) RmxSample {
+    int32_t src_x, src_y, src_w, src_h;  // source window in pixels (ROI or crop), XYWH
+    int32_t dst_w, dst_h;                // valid output size written for this sample
+    int32_t pc_x, pc_y;                  // offset of the written window inside the virtual resized image
+    int32_t rs_w, rs_h;                  // virtual resized size (== dst when there is no post-crop)
+    uint32_t flags;                      // RMX_S_*
+    int32_t strip_rows;                  // output rows per wave strip for this sample
+    float rx, ry;                        // src_len / rs_len (IEEE division done on the host)
+    float fsx, fsy;                      // triangular: ratio > 1 ? 1/ratio : 1
+    float scale[3], bias[3];             // normalisation: out = v*scale + bias
+    float color[4];                      // colour twist: alpha, beta, hue shift in sextants [0,6], saturation
+    float m[6];                          // warp: destination -> source affine about the centres
+};
+static_assert(sizeof(RmxSample) == 128, "parameter table row must stay 128 bytes");
+
+enum : uint32_t { RMX_S_HFLIP = 1u, RMX_S_VFLIP = 2u };
+
+struct RmxKArgs {
+    const uint8_t *src;      // batch base, u8 NHWC
+    void *dst;               // batch base
+    const RmxSample *table;  // device table, n rows
+    uint64_t src_bytes;      // total bytes of the source batch (bounds the wide loads)
+    int32_t n;
+    int32_t src_h, src_w;    // padded source dims (pixels); row stride = src_w*3
+    int32_t dst_h, dst_w;    // padded destination dims
+    int32_t strips;          // wave strips per sample (grid = n*strips waves)
+    int32_t lds_bytes;       // dynamic LDS per wave
+    int32_t aux0, aux1;
+};
+
+#define RMX_WAVE 64

@@ -1,0 +1,199 @@
+// Device-side building blocks shared by every kernel: realigned wide loads of packed RGB,
+// the rounding rules, and the typed/layout-aware group stores.
+#pragma once
+#include "rmx_common.h"
+
+#define RMX_DEV __device__ __forceinline__
+
+namespace rmx {
+
+constexpr int PX = 8;  // output pixels per lane group (8 x fp16 = one 128-bit store per channel)
+
+// multi-dword vectors that only promise dword alignment (global memory accepts that)
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x3_a4 __attribute__((ext_vector_type(3), aligned(4)));
+
+RMX_DEV float ubyte0(uint32_t v) { return (float)(v & 0xffu); }
+RMX_DEV float ubyte1(uint32_t v) { return (float)((v >> 8) & 0xffu); }
+RMX_DEV float ubyte2(uint32_t v) { return (float)((v >> 16) & 0xffu); }
+RMX_DEV float ubyte3(uint32_t v) { return (float)(v >> 24); }
+
+// u8 store rule: round-to-nearest-even, then saturate.
+RMX_DEV float round_u8(float v) {
+    v = __builtin_rintf(v);
+    return __builtin_fminf(__builtin_fmaxf(v, 0.0f), 255.0f);
+}
+
+// Order LDS traffic between the lanes of one wavefront. A wave's DS instructions execute in
+// issue order, so no hardware barrier is needed: this only stops the compiler from moving
+// LDS reads above the writes they depend on.
+RMX_DEV void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup -> XCD placement: hardware deals consecutive workgroup ids round-robin over the
+// 8 XCDs (each with its own L2). Remap so that consecutive logical ids land on one XCD, which
+// keeps all strips of a sample (and their shared halo rows) in a single L2.
+RMX_DEV uint32_t xcd_swizzle(uint32_t b, uint32_t nblocks) {
+    constexpr uint32_t XCDS = 8;
+    uint32_t per = nblocks / XCDS;
+    uint32_t body = per * XCDS;
+    if (b >= body) return b;  // ragged tail keeps its id
+    return (b % XCDS) * per + (b / XCDS);
+}
+
+// ---------------------------------------------------------------- source loads
+
+// Load `ND` consecutive dwords starting at the 4-byte-aligned address that contains byte
+// `p`, and realign them so that byte 0 of out[0] is *p. out has ND-1 dwords. Reads never go
+// past the dword that holds the last byte of the batch buffer.
+template <int ND>
+RMX_DEV void load_realigned(const uint8_t *p, const uint8_t *buf_end, uint32_t (&out)[ND - 1]) {
+    uintptr_t a = (uintptr_t)p;
+    uint32_t phase = (uint32_t)(a & 3u);
+    const uint32_t *q = (const uint32_t *)(a & ~(uintptr_t)3);
+    uint32_t d[ND];
+    if ((const uint8_t *)(q + ND) <= buf_end) {
+        if constexpr (ND == 4) {
+            u32x4_a4 t = *reinterpret_cast<const u32x4_a4 *>(q);  // global_load_dwordx4 at dword alignment
+            d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+        } else if constexpr (ND == 7) {
+            u32x4_a4 t = *reinterpret_cast<const u32x4_a4 *>(q);
+            u32x3_a4 u = *reinterpret_cast<const u32x3_a4 *>(q + 4);
+            d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w; d[4] = u.x; d[5] = u.y; d[6] = u.z;
+        } else {
+#pragma unroll
+            for (int i = 0; i < ND; i++) d[i] = q[i];
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < ND; i++) d[i] = ((const uint8_t *)(q + i) < buf_end) ? q[i] : 0u;
+    }
+#pragma unroll
+    for (int i = 0; i < ND - 1; i++) out[i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], phase);
+}
+
+// 8 packed RGB pixels (24 bytes = 6 dwords, byte 0 = R of pixel 0) -> v[c][k]
+RMX_DEV void unpack8(const uint32_t (&w)[6], float (&v)[3][PX]) {
+    v[0][0] = ubyte0(w[0]); v[1][0] = ubyte1(w[0]); v[2][0] = ubyte2(w[0]);
+    v[0][1] = ubyte3(w[0]); v[1][1] = ubyte0(w[1]); v[2][1] = ubyte1(w[1]);
+    v[0][2] = ubyte2(w[1]); v[1][2] = ubyte3(w[1]); v[2][2] = ubyte0(w[2]);
+    v[0][3] = ubyte1(w[2]); v[1][3] = ubyte2(w[2]); v[2][3] = ubyte3(w[2]);
+    v[0][4] = ubyte0(w[3]); v[1][4] = ubyte1(w[3]); v[2][4] = ubyte2(w[3]);
+    v[0][5] = ubyte3(w[3]); v[1][5] = ubyte0(w[4]); v[2][5] = ubyte1(w[4]);
+    v[0][6] = ubyte2(w[4]); v[1][6] = ubyte3(w[4]); v[2][6] = ubyte0(w[5]);
+    v[0][7] = ubyte1(w[5]); v[1][7] = ubyte2(w[5]); v[2][7] = ubyte3(w[5]);
+}
+
+// ---------------------------------------------------------------- typed stores
+
+template <typename T> struct OutCvt;
+template <> struct OutCvt<float> {
+    static RMX_DEV float cvt(float v) { return v; }
+};
+template <> struct OutCvt<__half> {
+    static RMX_DEV __half cvt(float v) { return __float2half_rn(v); }
+};
+template <> struct OutCvt<uint8_t> {
+    static RMX_DEV uint8_t cvt(float v) { return (uint8_t)round_u8(v); }
+};
+
+// Store `cnt` (<= N) consecutive elements; one or more 128/64/32-bit stores when the run is
+// full and the address allows it, element-wise otherwise.
+template <typename T, int N>
+RMX_DEV void store_run(T *p, const T (&e)[N], int cnt) {
+    constexpr int BYTES = N * (int)sizeof(T);
+    uintptr_t a = (uintptr_t)p;
+    if (cnt == N) {
+        if constexpr (BYTES % 16 == 0) {
+            if ((a & 15u) == 0) {
+                uint4 t[BYTES / 16];
+                __builtin_memcpy(t, e, BYTES);
+#pragma unroll
+                for (int i = 0; i < BYTES / 16; i++) reinterpret_cast<uint4 *>(p)[i] = t[i];
+                return;
+            }
+        }
+        if constexpr (BYTES % 8 == 0) {
+            if ((a & 7u) == 0) {
+                uint2 t[BYTES / 8];
+                __builtin_memcpy(t, e, BYTES);
+#pragma unroll
+                for (int i = 0; i < BYTES / 8; i++) reinterpret_cast<uint2 *>(p)[i] = t[i];
+                return;
+            }
+        }
+        if constexpr (BYTES % 4 == 0) {
+            if ((a & 3u) == 0) {
+                uint32_t t[BYTES / 4];
+                __builtin_memcpy(t, e, BYTES);
+#pragma unroll
+                for (int i = 0; i < BYTES / 4; i++) reinterpret_cast<uint32_t *>(p)[i] = t[i];
+                return;
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < N; i++)
+        if (i < cnt) p[i] = e[i];
+}
+
+// Write one lane's group of N horizontally adjacent pixels (v[c][k], k-th pixel of the group)
+// to output row y starting at column x0. `cnt` pixels are valid. When `rev` the group is
+// written in reversed pixel order (horizontal mirror): pixel k goes to column x0 + cnt-1-k.
+template <typename T, int LAYOUT, int N = PX>
+RMX_DEV void store_group(T *sample, int H, int W, int y, int x0, int cnt, const float (&v)[3][N], bool rev) {
+    if (cnt <= 0) return;
+    if constexpr (LAYOUT == RMX_NCHW) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            T e[N];
+            if (rev && cnt == N) {
+#pragma unroll
+                for (int k = 0; k < N; k++) e[k] = OutCvt<T>::cvt(v[c][N - 1 - k]);
+            } else if (rev) {
+#pragma unroll
+                for (int k = 0; k < N; k++) {
+                    float s = v[c][0];
+#pragma unroll
+                    for (int j = 1; j < N; j++) s = (j == cnt - 1 - k) ? v[c][j] : s;
+                    e[k] = OutCvt<T>::cvt(s);
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < N; k++) e[k] = OutCvt<T>::cvt(v[c][k]);
+            }
+            T *p = sample + ((size_t)c * H + y) * W + x0;
+            store_run<T, N>(p, e, cnt);
+        }
+    } else {
+        T e[N * 3];
+        if (rev && cnt == N) {
+#pragma unroll
+            for (int k = 0; k < N; k++)
+#pragma unroll
+                for (int c = 0; c < 3; c++) e[k * 3 + c] = OutCvt<T>::cvt(v[c][N - 1 - k]);
+        } else if (rev) {
+#pragma unroll
+            for (int k = 0; k < N; k++)
+#pragma unroll
+                for (int c = 0; c < 3; c++) {
+                    float s = v[c][0];
+#pragma unroll
+                    for (int j = 1; j < N; j++) s = (j == cnt - 1 - k) ? v[c][j] : s;
+                    e[k * 3 + c] = OutCvt<T>::cvt(s);
+                }
+        } else {
+#pragma unroll
+            for (int k = 0; k < N; k++)
+#pragma unroll
+                for (int c = 0; c < 3; c++) e[k * 3 + c] = OutCvt<T>::cvt(v[c][k]);
+        }
+        T *p = sample + ((size_t)y * W + x0) * 3;
+        store_run<T, N * 3>(p, e, cnt * 3);
+    }
+}
+
+}  // namespace rmx

@@ -1,0 +1,234 @@
+// K2t: triangular (antialiased) resize, separable, both passes staged through LDS, with the
+// same epilogue as the bilinear kernel ([u8 quantise] -> [mirror] -> [normalise] -> layout -> cast).
+//
+// A wavefront owns an x-tile of 128 output columns (two per lane) and a strip of output rows
+// and walks down the strip with a ring of horizontally filtered source rows in its private LDS
+// slice:
+//   horizontal pass  one source row at a time: stage the row segment (dword per pixel), then
+//                    every lane accumulates its two columns over the kx taps in tap order
+//                    (coefficients come from a per-tile LDS table built once per strip);
+//   vertical pass    per output row: accumulate the ky ring rows in tap order, normalise by
+//                    1/(rowsum*colsum), epilogue, store.
+// Source rows enter the ring exactly once per strip; the intermediate never touches HBM.
+#include "rmx_device.h"
+#include "rmx_launch.h"
+
+namespace rmx {
+
+extern __shared__ uint32_t rmx_lds_tri[];
+
+constexpr int TTW = 128;  // output columns per wave tile
+constexpr int TPX = 2;    // columns per lane
+
+struct TriAxis {
+    float ratio, radius, fscale, offset;
+    int ksize;
+};
+
+RMX_DEV TriAxis tri_axis(float ratio, float fscale) {
+    TriAxis t;
+    t.ratio = ratio;
+    t.radius = ratio > 1.0f ? ratio : 1.0f;
+    t.fscale = fscale;
+    t.offset = (ratio - 1) * 0.5f - t.radius;
+    t.ksize = (int)ceilf(t.radius * 2);
+    return t;
+}
+
+RMX_DEV void tri_loc(const TriAxis &t, int d, float lo, int &loc, float &w0) {
+    float raw = (float)d * t.ratio;
+    raw = raw + t.offset;
+    raw = raw + lo;
+    loc = (int)ceilf(raw);
+    w0 = (float)loc - raw;
+}
+
+RMX_DEV float tri_coeff(float w0, float radius, int k, float fscale) {
+    float c = 1 - fabsf((w0 - radius + (float)k) * fscale);
+    return c < 0 ? 0 : c;
+}
+
+template <typename T, int LAYOUT, bool NORM, bool QUANT>
+__global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
+    const int lane = threadIdx.x & (RMX_WAVE - 1);
+    const int wib = threadIdx.x / RMX_WAVE;
+    const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
+    uint32_t wave = xcd_swizzle(blockIdx.x, gridDim.x) * (blockDim.x / RMX_WAVE) + wib;
+    wave = __builtin_amdgcn_readfirstlane(wave);
+    if (wave >= nwaves) return;
+    const int s = (int)(wave / (uint32_t)a.strips);
+    const int part = (int)(wave % (uint32_t)a.strips);
+    const int tiles_x = a.aux1;
+    const int strip = part / tiles_x, tx = part - strip * tiles_x;
+    const RmxSample &P = a.table[s];
+
+    const int dw = P.dst_w, dh = P.dst_h;
+    const int srows = a.aux0;
+    const int r0 = strip * srows, xt = tx * TTW;
+    if (r0 >= dh || xt >= dw) return;
+    const int r1 = min(r0 + srows, dh);
+    const int tw = min(TTW, dw - xt);
+    const bool hf = (P.flags & RMX_S_HFLIP) != 0;
+    const int xlo = P.src_x, ylo = P.src_y;
+    const int xhi = xlo + P.src_w - 1, yhi = ylo + P.src_h - 1;
+    const int pcx = P.pc_x, pcy = P.pc_y;
+    const TriAxis ax = tri_axis(P.rx, P.fsx), ay = tri_axis(P.ry, P.fsy);
+    const int kx = ax.ksize, ky = ay.ksize;
+    const int ring_rows = P.strip_rows >> 16;      // power of two
+    const int kx_cap = P.strip_rows & 0xffff;
+    const int ring_mask = ring_rows - 1;
+
+    const size_t row_stride = (size_t)a.src_w * 3;
+    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    const uint8_t *buf_end = a.src + a.src_bytes;
+    T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
+
+    // LDS slice: coef[kx_cap][TTW] | ring[ring_rows][3][TTW] | srcrow[...]
+    uint32_t *base = rmx_lds_tri + (size_t)wib * (a.lds_bytes >> 2);
+    float *coef = reinterpret_cast<float *>(base);
+    float *ring = coef + kx_cap * TTW;
+    uint32_t *srcrow = reinterpret_cast<uint32_t *>(ring + ring_rows * 3 * TTW);
+
+    float sc[3], bi[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        sc[c] = P.scale[c];
+        bi[c] = P.bias[c];
+    }
+
+    // ---- per-lane column taps (two columns), coefficient table, column sums
+    const int t0 = xt + lane * TPX;
+    const int cnt = max(0, min(TPX, dw - t0));
+    int locx[TPX];
+    float colsum[TPX];
+#pragma unroll
+    for (int i = 0; i < TPX; i++) {
+        int u = pcx + min(t0 + i, dw - 1);
+        float w0;
+        tri_loc(ax, u, (float)xlo, locx[i], w0);
+        float sum = 0.0f;
+        for (int k = 0; k < kx; k++) {
+            float c = tri_coeff(w0, ax.radius, k, ax.fscale);
+            coef[k * TTW + lane * TPX + i] = c;
+            sum += c;
+        }
+        colsum[i] = (sum == 0.0f) ? 1.0f : sum;
+    }
+    // tile-wide staged source column range (wave-uniform)
+    int l_first, l_last;
+    {
+        float w0;
+        tri_loc(ax, pcx + xt, (float)xlo, l_first, w0);
+        tri_loc(ax, pcx + xt + tw - 1, (float)xlo, l_last, w0);
+    }
+    const int cs = max(min(l_first, xhi), xlo);
+    const int ce = max(min(l_last + kx - 1, xhi), xlo);
+    const int items = (ce - cs + 4) >> 2;
+    wave_sync();
+
+    int next_row;
+    {
+        int loc;
+        float w0;
+        tri_loc(ay, pcy + r0, (float)ylo, loc, w0);
+        next_row = max(min(loc, yhi), ylo);
+    }
+
+    for (int r = r0; r < r1; r++) {
+        int locy;
+        float w0y;
+        tri_loc(ay, pcy + r, (float)ylo, locy, w0y);
+        const int rb = max(min(locy + ky - 1, yhi), ylo);
+        // ---- horizontal pass for the source rows that enter the window
+        for (; next_row <= rb; next_row++) {
+            for (int j = lane; j < items; j += RMX_WAVE) {
+                const uint8_t *p = simg + (size_t)next_row * row_stride + (size_t)(cs + 4 * j) * 3;
+                uint32_t w[3];
+                load_realigned<4>(p, buf_end, w);
+                uint4 px;
+                px.x = w[0];
+                px.y = __builtin_amdgcn_alignbyte(w[1], w[0], 3);
+                px.z = __builtin_amdgcn_alignbyte(w[2], w[1], 2);
+                px.w = w[2] >> 8;
+                *reinterpret_cast<uint4 *>(srcrow + 4 * j) = px;
+            }
+            wave_sync();
+            float *slot = ring + (next_row & ring_mask) * 3 * TTW;
+#pragma unroll
+            for (int i = 0; i < TPX; i++) {
+                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+                for (int k = 0; k < kx; k++) {
+                    const int ci = max(min(locx[i] + k, xhi), xlo) - cs;
+                    const uint32_t p = srcrow[ci];
+                    const float c = coef[k * TTW + lane * TPX + i];
+                    a0 = __builtin_fmaf(ubyte0(p), c, a0);
+                    a1 = __builtin_fmaf(ubyte1(p), c, a1);
+                    a2 = __builtin_fmaf(ubyte2(p), c, a2);
+                }
+                slot[0 * TTW + lane * TPX + i] = a0;
+                slot[1 * TTW + lane * TPX + i] = a1;
+                slot[2 * TTW + lane * TPX + i] = a2;
+            }
+            wave_sync();
+        }
+        // ---- vertical pass (each lane reads only ring entries it wrote itself)
+        if (cnt > 0) {
+            float rsum = 0.0f;
+            for (int j = 0; j < ky; j++) rsum += tri_coeff(w0y, ay.radius, j, ay.fscale);
+            rsum = (rsum == 0.0f) ? 1.0f : rsum;
+            float v[3][TPX];
+#pragma unroll
+            for (int i = 0; i < TPX; i++) {
+                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+                for (int j = 0; j < ky; j++) {
+                    const int rr = max(min(locy + j, yhi), ylo);
+                    const float *slot = ring + (rr & ring_mask) * 3 * TTW + lane * TPX + i;
+                    const float c = tri_coeff(w0y, ay.radius, j, ay.fscale);
+                    a0 = __builtin_fmaf(slot[0 * TTW], c, a0);
+                    a1 = __builtin_fmaf(slot[1 * TTW], c, a1);
+                    a2 = __builtin_fmaf(slot[2 * TTW], c, a2);
+                }
+                const float inv = 1 / (rsum * colsum[i]);
+                v[0][i] = a0 * inv;
+                v[1][i] = a1 * inv;
+                v[2][i] = a2 * inv;
+            }
+#pragma unroll
+            for (int c = 0; c < 3; c++)
+#pragma unroll
+                for (int i = 0; i < TPX; i++) {
+                    float t = v[c][i];
+                    if constexpr (QUANT) t = round_u8(t);
+                    if constexpr (NORM) t = __builtin_fmaf(t, sc[c], bi[c]);
+                    v[c][i] = t;
+                }
+            const int x0 = hf ? (dw - t0 - cnt) : t0;
+            store_group<T, LAYOUT, TPX>(dimg, a.dst_h, a.dst_w, r, x0, cnt, v, hf);
+        }
+    }
+}
+
+template <typename T, int LAYOUT>
+static KernelFn pick3(bool norm, bool quant) {
+    if (norm && quant) return (KernelFn)rmx_resize_tri_kernel<T, LAYOUT, true, true>;
+    if (norm) return (KernelFn)rmx_resize_tri_kernel<T, LAYOUT, true, false>;
+    return (KernelFn)rmx_resize_tri_kernel<T, LAYOUT, false, false>;
+}
+
+KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
+    *name = "rmx_resize_tri_kernel";
+    if (layout == RMX_NCHW) {
+        switch (dtype) {
+            case RMX_FP32: return pick3<float, RMX_NCHW>(norm, quant);
+            case RMX_FP16: return pick3<__half, RMX_NCHW>(norm, quant);
+            default: return pick3<uint8_t, RMX_NCHW>(norm, quant);
+        }
+    }
+    switch (dtype) {
+        case RMX_FP32: return pick3<float, RMX_NHWC>(norm, quant);
+        case RMX_FP16: return pick3<__half, RMX_NHWC>(norm, quant);
+        default: return pick3<uint8_t, RMX_NHWC>(norm, quant);
+    }
+}
+
+}  // namespace rmx

@@ -1,0 +1,16 @@
+// Host-side kernel selection: each kernel family exports a selector that maps the static
+// node configuration to one template instantiation.
+#pragma once
+#include "rmx_common.h"
+
+namespace rmx {
+typedef void (*KernelFn)(RmxKArgs);
+
+KernelFn select_cmn_kernel(int dtype, int layout, bool norm, const char **name);
+KernelFn select_resize_linear_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
+KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
+KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
+KernelFn select_color_kernel(int kind, int dtype, int layout, const char **name);
+KernelFn select_warp_kernel(int interp, int dtype, int layout, const char **name);
+void launch_copy(hipStream_t stream, const void *src, void *dst, size_t nbytes, int num_cus);
+}  // namespace rmx

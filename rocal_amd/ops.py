@@ -1,0 +1,231 @@
+"""Thin Python doorway onto the C ABI (include/rocal_mi355x.h): contexts and per-node ops.
+
+torch is used only for device memory and streams; every pixel is produced by the HIP kernels
+in librocal_mi355x.so. Parameter arrays are numpy (host) arrays, as rocAL's vx_arrays are.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import TensorDesc, check
+
+NHWC, NCHW = 0, 1
+FP32, FP16, UINT8 = 0, 1, 2
+ROI_LTRB, ROI_XYWH = 0, 1
+NEAREST, LINEAR, TRIANGULAR = 0, 1, 5
+F_QUANTIZE_U8 = 1
+
+
+def _torch():
+    import torch
+    return torch
+
+
+def torch_dtype(dtype):
+    t = _torch()
+    return {FP32: t.float32, FP16: t.float16, UINT8: t.uint8}[dtype]
+
+
+def _arr(a, dt):
+    if a is None:
+        return None, None
+    a = np.ascontiguousarray(a, dtype=dt)
+    return a, a.ctypes.data_as(C.c_void_p)
+
+
+class Context:
+    """One device + one stream (rmx_ctx). stream="torch" borrows torch's current stream,
+    stream="own" lets the context create its own, an integer is a hipStream_t to borrow."""
+
+    def __init__(self, device=0, stream="torch"):
+        self._h = C.c_void_p()
+        sp, own = None, 0
+        if stream == "torch":
+            t = _torch()
+            sp = C.c_void_p(t.cuda.current_stream(device).cuda_stream)
+        elif stream == "own":
+            own = 1
+        elif stream is not None:
+            sp = C.c_void_p(int(stream))
+        check(_lib.lib().rmx_ctx_create(int(device), sp, own, C.byref(self._h)))
+        self.device = device
+
+    def sync(self):
+        check(_lib.lib().rmx_ctx_sync(self._h))
+
+    @property
+    def stream(self):
+        return _lib.lib().rmx_ctx_stream(self._h)
+
+    def copy_bytes(self, src, dst, nbytes):
+        check(_lib.lib().rmx_copy_bytes(self._h, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), nbytes))
+
+    def close(self):
+        if self._h:
+            _lib.lib().rmx_ctx_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def desc(n, h, w, layout, dtype, c=3):
+    return TensorDesc(n, h, w, c, layout, dtype)
+
+
+class Op:
+    """One node (rmx_op). Subclasses bind create/update of a specific reference node."""
+
+    _create = None
+
+    def __init__(self, ctx, src_desc, dst_desc, *extra, roi_type=ROI_XYWH):
+        self.ctx = ctx
+        self.src_desc, self.dst_desc = src_desc, dst_desc
+        self._h = C.c_void_p()
+        fn = getattr(_lib.lib(), self._create)
+        check(fn(ctx._h, C.byref(src_desc), C.byref(dst_desc), *extra[:self._n_pre], int(roi_type),
+                 *extra[self._n_pre:], C.byref(self._h)))
+
+    _n_pre = 0
+
+    def _update(self, name, *arrays_and_types):
+        keep, ptrs = [], []
+        for a, dt in arrays_and_types:
+            arr, p = _arr(a, dt)
+            keep.append(arr)
+            ptrs.append(p)
+        check(getattr(_lib.lib(), name)(self._h, *ptrs))
+
+    def launch(self, src, dst):
+        """src/dst: torch CUDA tensors (the batch buffers). Asynchronous on the context's stream."""
+        assert src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()
+        sd, dd = self.src_desc, self.dst_desc
+        assert src.numel() * src.element_size() >= sd.n * sd.h * sd.w * sd.c, "source buffer smaller than its descriptor"
+        esz = {FP32: 4, FP16: 2, UINT8: 1}[dd.dtype]
+        assert dst.numel() * dst.element_size() >= dd.n * dd.h * dd.w * dd.c * esz, "destination buffer smaller than its descriptor"
+        check(_lib.lib().rmx_op_launch(self._h, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())))
+
+    def alloc_output(self, fill=0):
+        t = _torch()
+        d = self.dst_desc
+        shape = (d.n, d.c, d.h, d.w) if d.layout == NCHW else (d.n, d.h, d.w, d.c)
+        return t.full(shape, fill, dtype=torch_dtype(d.dtype), device="cuda:%d" % self.ctx.device)
+
+    @property
+    def algorithmic_bytes(self):
+        return int(_lib.lib().rmx_op_algorithmic_bytes(self._h))
+
+    @property
+    def kernel_name(self):
+        return _lib.lib().rmx_op_kernel_name(self._h).decode()
+
+    def close(self):
+        if self._h:
+            _lib.lib().rmx_op_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+_U, _F = np.uint32, np.float32
+
+
+class CropMirrorNormalize(Op):
+    _create = "rmx_create_crop_mirror_normalize"
+
+    def update(self, crop_roi, scale, bias, mirror=None):
+        self._update("rmx_update_crop_mirror_normalize", (crop_roi, _U), (scale, _F), (bias, _F), (mirror, _U))
+
+
+class Crop(Op):
+    _create = "rmx_create_crop"
+
+    def update(self, crop_roi):
+        self._update("rmx_update_crop", (crop_roi, _U))
+
+
+class Flip(Op):
+    _create = "rmx_create_flip"
+
+    def update(self, src_roi, horizontal, vertical):
+        self._update("rmx_update_flip", (src_roi, _U), (horizontal, _U), (vertical, _U))
+
+
+class Resize(Op):
+    _create = "rmx_create_resize"
+    _n_pre = 1
+
+    def __init__(self, ctx, src_desc, dst_desc, interpolation=LINEAR, flags=0, roi_type=ROI_XYWH):
+        super().__init__(ctx, src_desc, dst_desc, int(interpolation), C.c_uint32(flags), roi_type=roi_type)
+
+    def update(self, src_roi, dst_w, dst_h, mirror=None, mean=None, stddev=None):
+        self._update("rmx_update_resize", (src_roi, _U), (dst_w, _U), (dst_h, _U), (mirror, _U), (mean, _F), (stddev, _F))
+
+    def update_cmn(self, src_roi, dst_w, dst_h, scale, bias, mirror=None, crop_roi=None):
+        self._update("rmx_update_resize_cmn", (src_roi, _U), (dst_w, _U), (dst_h, _U), (crop_roi, _U), (scale, _F),
+                     (bias, _F), (mirror, _U))
+
+
+class ColorTwist(Op):
+    _create = "rmx_create_color_twist"
+
+    def update(self, src_roi, alpha, beta, hue, sat):
+        self._update("rmx_update_color_twist", (src_roi, _U), (alpha, _F), (beta, _F), (hue, _F), (sat, _F))
+
+
+class Brightness(Op):
+    _create = "rmx_create_brightness"
+
+    def update(self, src_roi, alpha, beta):
+        self._update("rmx_update_brightness", (src_roi, _U), (alpha, _F), (beta, _F))
+
+
+class Contrast(Op):
+    _create = "rmx_create_contrast"
+
+    def update(self, src_roi, factor, center):
+        self._update("rmx_update_contrast", (src_roi, _U), (factor, _F), (center, _F))
+
+
+class Hue(Op):
+    _create = "rmx_create_hue"
+
+    def update(self, src_roi, hue):
+        self._update("rmx_update_hue", (src_roi, _U), (hue, _F))
+
+
+class Saturation(Op):
+    _create = "rmx_create_saturation"
+
+    def update(self, src_roi, sat):
+        self._update("rmx_update_saturation", (src_roi, _U), (sat, _F))
+
+
+class WarpAffine(Op):
+    _create = "rmx_create_warp_affine"
+    _n_pre = 1
+
+    def __init__(self, ctx, src_desc, dst_desc, interpolation=LINEAR, roi_type=ROI_XYWH):
+        super().__init__(ctx, src_desc, dst_desc, int(interpolation), roi_type=roi_type)
+
+    def update(self, src_roi, affine, dst_w, dst_h):
+        self._update("rmx_update_warp_affine", (src_roi, _U), (affine, _F), (dst_w, _U), (dst_h, _U))
+
+
+class Rotate(Op):
+    _create = "rmx_create_rotate"
+    _n_pre = 1
+
+    def __init__(self, ctx, src_desc, dst_desc, interpolation=LINEAR, roi_type=ROI_XYWH):
+        super().__init__(ctx, src_desc, dst_desc, int(interpolation), roi_type=roi_type)
+
+    def update(self, src_roi, angle, dst_w, dst_h):
+        self._update("rmx_update_rotate", (src_roi, _U), (angle, _F), (dst_w, _U), (dst_h, _U))

@@ -1,0 +1,350 @@
+"""GPU parity: every kernel family through the C ABI against the CPU oracle on the same seeded
+inputs. Bars (stated where they are checked): bit-exact for crop/flip/layout work and for u8
+outputs of integer-only stages; <=1 LSB for u8 resize/warp/colour; <=1e-5 relative (fp32) and
+<=1e-3 (fp16) for normalised outputs. The kernels are written to reproduce the oracle's fp32
+operation order, so most cases are additionally checked for exact equality."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from rocal_amd import ops, workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {ops.FP32: 1e-5, ops.FP16: 1e-3}
+
+
+def _gpu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _cpu(t, ctx):
+    ctx.sync()
+    return t.cpu().numpy()
+
+
+def _check(got, exp, dtype, exact=True, what=""):
+    assert got.shape == exp.shape, (got.shape, exp.shape)
+    if dtype == ops.UINT8:
+        d = np.abs(got.astype(np.int32) - exp.astype(np.int32))
+        assert d.max() <= 1, "%s: u8 output differs by %d" % (what, d.max())
+        if exact:
+            assert d.max() == 0, "%s: %d u8 values differ by 1" % (what, int((d > 0).sum()))
+        return
+    g, e = got.astype(np.float64), exp.astype(np.float64)
+    # relative bar with an absolute floor of one tolerance unit at |value| = 1 (outputs cross zero)
+    tol = RTOL[dtype]
+    err = np.abs(g - e) / np.maximum(np.abs(e), 1.0)
+    assert err.max() <= tol, "%s: max relative error %g > %g" % (what, err.max(), tol)
+    if exact:
+        nbad = int((got != exp).sum())
+        assert nbad == 0, "%s: %d of %d values not bit-identical" % (what, nbad, got.size)
+
+
+def _mean_std(n):
+    return orc.cmn_scale_bias(wl.MEAN, wl.STD, n)
+
+
+# ------------------------------------------------------------------ K1: CMN / crop / flip
+
+@pytest.mark.parametrize("dtype", [ops.FP32, ops.FP16, ops.UINT8])
+@pytest.mark.parametrize("layout", [ops.NCHW, ops.NHWC])
+def test_cmn_config0_small(ctx, dtype, layout):
+    c = wl.config0(n=8)
+    n = 8
+    scale, bias = _mean_std(n)
+    if dtype == ops.UINT8:  # the reference's own u8 CMN case: mean 128, std 1.2 (unit_tests.cpp:730-735)
+        scale, bias = orc.cmn_scale_bias([128, 128, 128], [1.2, 1.2, 1.2], n)
+    exp = orc.crop_mirror_normalize(c["img"], c["crop"], scale, bias, c["mirror"], 224, 224, layout, dtype)
+    op = ops.CropMirrorNormalize(ctx, ops.desc(n, 256, 256, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, layout, dtype))
+    op.update(c["crop"], scale, bias, c["mirror"])
+    out = op.alloc_output()
+    op.launch(_gpu(c["img"]), out)
+    _check(_cpu(out, ctx), exp, dtype, exact=True, what="cmn")
+
+
+def test_cmn_ragged_unaligned(ctx):
+    """Odd widths, odd offsets, crops larger than some ROIs, output padded beyond the crop."""
+    rng = np.random.default_rng(7)
+    n, H, W = 6, 37, 53
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    crop = np.array([[0, 0, 53, 37], [1, 2, 50, 30], [7, 0, 13, 37], [52, 36, 1, 1], [3, 3, 9, 8], [5, 1, 47, 35]], np.uint32)
+    mirror = np.array([1, 0, 1, 1, 0, 1], np.uint32)
+    scale, bias = _mean_std(n)
+    for layout in (ops.NCHW, ops.NHWC):
+        for dtype in (ops.FP32, ops.FP16, ops.UINT8):
+            exp = orc.crop_mirror_normalize(img, crop, scale, bias, mirror, 40, 56, layout, dtype)
+            op = ops.CropMirrorNormalize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 40, 56, layout, dtype))
+            op.update(crop, scale, bias, mirror)
+            out = op.alloc_output()
+            op.launch(_gpu(img), out)
+            _check(_cpu(out, ctx), exp, dtype, exact=True, what="cmn ragged %d %d" % (layout, dtype))
+
+
+def test_crop_and_flip_bit_exact(ctx):
+    rng = np.random.default_rng(8)
+    n, H, W = 5, 64, 96
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    crop = np.array([[0, 0, 96, 64], [10, 5, 40, 50], [95, 63, 1, 1], [3, 0, 77, 64], [8, 8, 16, 16]], np.uint32)
+    op = ops.Crop(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, H, W, ops.NHWC, ops.UINT8))
+    op.update(crop)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    exp = orc.crop_mirror_normalize(img, crop, None, None, None, H, W, ops.NHWC, ops.UINT8)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="crop")
+    # flip: all four (h,v) combinations + involution
+    roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
+    hflag = np.array([0, 1, 0, 1, 1], np.uint32)
+    vflag = np.array([0, 0, 1, 1, 0], np.uint32)
+    fop = ops.Flip(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, H, W, ops.NHWC, ops.UINT8))
+    fop.update(roi, hflag, vflag)
+    out1 = fop.alloc_output()
+    gi = _gpu(img)
+    fop.launch(gi, out1)
+    exp = orc.crop_mirror_normalize(img, roi, None, None, hflag, H, W, ops.NHWC, ops.UINT8, vflip=vflag)
+    got = _cpu(out1, ctx)
+    _check(got, exp, ops.UINT8, exact=True, what="flip")
+    for i in range(n):
+        ref = img[i]
+        if hflag[i]:
+            ref = ref[:, ::-1]
+        if vflag[i]:
+            ref = ref[::-1]
+        assert np.array_equal(got[i], ref)
+    out2 = fop.alloc_output()
+    fop.launch(out1, out2)
+    assert np.array_equal(_cpu(out2, ctx), img), "flip twice must be the identity"
+
+
+# ------------------------------------------------------------------ K2: resize family
+
+@pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST, ops.TRIANGULAR])
+def test_resize_u8_ragged(ctx, interp):
+    rng = np.random.default_rng(9)
+    n, H, W = 6, 70, 90
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.5)
+    roi = np.array([[0, 0, 90, 70], [5, 3, 60, 61], [0, 0, 33, 70], [11, 13, 64, 40], [0, 0, 90, 70], [1, 1, 8, 9]], np.uint32)
+    dw = np.array([64, 120, 17, 64, 45, 100], np.uint32)
+    dh = np.array([48, 80, 100, 20, 35, 90], np.uint32)
+    exp = orc.resize(img, roi, dw, dh, 100, 120, interp=interp)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 100, 120, ops.NHWC, ops.UINT8), interp)
+    op.update(roi, dw, dh)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="resize u8 interp %d" % interp)
+
+
+@pytest.mark.parametrize("interp", [ops.LINEAR, ops.TRIANGULAR])
+@pytest.mark.parametrize("dtype,layout", [(ops.FP16, ops.NCHW), (ops.FP32, ops.NCHW), (ops.FP32, ops.NHWC), (ops.UINT8, ops.NCHW)])
+def test_resize_mirror_normalize(ctx, interp, dtype, layout):
+    rng = np.random.default_rng(10)
+    n, H, W = 4, 120, 160
+    img = wl.smooth_noise(rng, n, H, W, sigma=2.0)
+    roi = np.array([[0, 0, 160, 120], [8, 8, 100, 100], [0, 0, 97, 51], [30, 20, 130, 100]], np.uint32)
+    dw = np.array([64, 64, 64, 56], np.uint32)
+    dh = np.array([48, 48, 40, 48], np.uint32)
+    mirror = np.array([1, 0, 1, 1], np.uint32)
+    mean = np.tile(wl.MEAN, n)
+    std = np.tile(wl.STD, n)
+    scale, bias = _mean_std(n)
+    exp = orc.resize(img, roi, dw, dh, 48, 64, interp=interp, mirror=mirror, scale=scale, bias=bias, layout=layout, dtype=dtype)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 48, 64, layout, dtype), interp)
+    op.update(roi, dw, dh, mirror, mean, std)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, dtype, exact=True, what="rmn")
+
+
+def test_rrc_cmn_fused_config1_small(ctx):
+    """Configuration 1 at reduced batch: ragged sources, RandomResizedCrop windows, bilinear to
+    224x224, u8 quantisation between the two reference nodes, mirror, normalise, fp16 NCHW."""
+    n = 12
+    c = wl.config1(n=n, hw_range=(240, 640))
+    scale, bias = _mean_std(n)
+    dw = np.full(n, 224, np.uint32)
+    dh = np.full(n, 224, np.uint32)
+    exp = orc.resize(c["img"], c["roi"], dw, dh, 224, 224, interp=orc.LINEAR, mirror=c["mirror"], scale=scale, bias=bias,
+                     layout=ops.NCHW, dtype=ops.FP16, flags=orc.F_QUANTIZE_U8)
+    op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR,
+                    flags=ops.F_QUANTIZE_U8)
+    op.update_cmn(c["roi"], dw, dh, scale, bias, c["mirror"])
+    out = op.alloc_output()
+    op.launch(_gpu(c["img"]), out)
+    _check(_cpu(out, ctx), exp, ops.FP16, exact=True, what="rrc+cmn")
+    # the fused pass equals the two-node graph: resize to u8, then CropMirrorNormalize
+    mid = orc.resize(c["img"], c["roi"], dw, dh, 224, 224, interp=orc.LINEAR)
+    full = np.tile(np.array([0, 0, 224, 224], np.uint32), (n, 1))
+    two = orc.crop_mirror_normalize(mid, full, scale, bias, c["mirror"], 224, 224, ops.NCHW, ops.FP16)
+    assert np.array_equal(two.view(np.uint16), exp.view(np.uint16))
+
+
+def test_resize_then_center_crop_fused(ctx):
+    """resize(256) -> CMN centre crop 224 as one launch (post-crop window inside the resized image)."""
+    rng = np.random.default_rng(11)
+    n, H, W = 3, 300, 280
+    img = wl.smooth_noise(rng, n, H, W, sigma=2.0)
+    roi = np.array([[0, 0, 280, 300], [0, 0, 200, 300], [10, 10, 260, 200]], np.uint32)
+    dw = np.full(n, 256, np.uint32)
+    dh = np.full(n, 256, np.uint32)
+    crop = np.tile(np.array([16, 16, 224, 224], np.uint32), (n, 1))
+    mirror = np.array([0, 1, 1], np.uint32)
+    scale, bias = _mean_std(n)
+    mid = orc.resize(img, roi, dw, dh, 256, 256, interp=orc.LINEAR)
+    exp = orc.crop_mirror_normalize(mid, crop, scale, bias, mirror, 224, 224, ops.NCHW, ops.FP32)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP32), ops.LINEAR,
+                    flags=ops.F_QUANTIZE_U8)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror, crop_roi=crop)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, ops.FP32, exact=True, what="resize+centre crop")
+
+
+def test_triangular_config4_small(ctx):
+    n = 2
+    c = wl.config4(n=n, src_hw=(270, 480), dst_hw=(90, 160))
+    scale, bias = _mean_std(n)
+    dw = np.full(n, 160, np.uint32)
+    dh = np.full(n, 90, np.uint32)
+    exp = orc.resize(c["img"], c["roi"], dw, dh, 90, 160, interp=orc.TRIANGULAR, mirror=c["mirror"], scale=scale, bias=bias,
+                     layout=ops.NCHW, dtype=ops.FP16)
+    op = ops.Resize(ctx, ops.desc(n, 270, 480, ops.NHWC, ops.UINT8), ops.desc(n, 90, 160, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+    op.update(c["roi"], dw, dh, c["mirror"], np.tile(wl.MEAN, n), np.tile(wl.STD, n))
+    out = op.alloc_output()
+    op.launch(_gpu(c["img"]), out)
+    _check(_cpu(out, ctx), exp, ops.FP16, exact=True, what="triangular")
+
+
+# ------------------------------------------------------------------ K3: colour family
+
+def test_color_twist_config2_small(ctx):
+    n = 8
+    c = wl.config2(n=n)
+    exp = orc.color_twist(c["img"], c["roi"], c["alpha"], c["beta"], c["hue"], c["sat"])
+    op = ops.ColorTwist(ctx, ops.desc(n, 224, 224, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NHWC, ops.UINT8))
+    op.update(c["roi"], c["alpha"], c["beta"], c["hue"], c["sat"])
+    out = op.alloc_output()
+    op.launch(_gpu(c["img"]), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="color twist")
+
+
+def test_color_family_fixed_params(ctx):
+    """The fixed parameters of the reference's own unit tests (tests/cpp_api/unit_tests/unit_tests.cpp:
+    755,763,812,816,820)."""
+    rng = np.random.default_rng(12)
+    n, H, W = 2, 50, 75
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
+    gi = _gpu(img)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    one = lambda v: np.full(n, v, np.float32)
+
+    def run(op, *args):
+        op.update(roi, *args)
+        out = op.alloc_output()
+        op.launch(gi, out)
+        return _cpu(out, ctx)
+
+    _check(run(ops.Brightness(ctx, sd, sd), one(1.9), one(20.0)), orc.brightness(img, roi, one(1.9), one(20.0)), ops.UINT8, what="brightness")
+    _check(run(ops.Contrast(ctx, sd, sd), one(30.0), one(80.0)), orc.contrast(img, roi, one(30.0), one(80.0)), ops.UINT8, what="contrast")
+    _check(run(ops.Hue(ctx, sd, sd), one(150.0)), orc.color_twist(img, roi, one(1), one(0), one(150.0), one(1)), ops.UINT8, what="hue")
+    _check(run(ops.Saturation(ctx, sd, sd), one(0.3)), orc.color_twist(img, roi, one(1), one(0), one(0), one(0.3)), ops.UINT8, what="sat")
+    _check(run(ops.ColorTwist(ctx, sd, sd), one(0.2), one(10.0), one(100.0), one(0.25)),
+           orc.color_twist(img, roi, one(0.2), one(10.0), one(100.0), one(0.25)), ops.UINT8, what="twist fixed")
+
+
+def test_color_twist_all_rgb_values(ctx):
+    """Every (r,g,b) triple on a 64-step lattice plus the extremes, several parameter sets."""
+    v = np.unique(np.concatenate([np.arange(0, 256, 5), [1, 2, 254, 255]])).astype(np.uint8)
+    r, g, b = np.meshgrid(v, v, v, indexing="ij")
+    px = np.stack([r.ravel(), g.ravel(), b.ravel()], -1)
+    W = 256
+    H = (len(px) + W - 1) // W
+    n = 4
+    img = np.zeros((n, H, W, 3), np.uint8)
+    img.reshape(n, -1, 3)[:, :len(px)] = px
+    roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
+    alpha = np.array([1.0, 0.7, 1.3, 1.95], np.float32)
+    beta = np.array([0.0, 12.5, -7.25, 25.0], np.float32)
+    hue = np.array([0.0, -18.0, 127.3, 359.9], np.float32)
+    sat = np.array([1.0, 0.0, 1.4, 0.37], np.float32)
+    exp = orc.color_twist(img, roi, alpha, beta, hue, sat)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    op = ops.ColorTwist(ctx, sd, sd)
+    op.update(roi, alpha, beta, hue, sat)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="twist lattice")
+
+
+# ------------------------------------------------------------------ K4: warp / rotate
+
+@pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST])
+def test_warp_affine_config3_small(ctx, interp):
+    n = 6
+    c = wl.config3(n=n, size=160)
+    dw = np.full(n, 160, np.uint32)
+    dh = np.full(n, 160, np.uint32)
+    m = np.stack([orc.affine_from_rocal(a) for a in c["affine"]])
+    exp = orc.warp_affine(c["img"], c["roi"], m, dw, dh, 160, 160, interp=interp)
+    sd = ops.desc(n, 160, 160, ops.NHWC, ops.UINT8)
+    op = ops.WarpAffine(ctx, sd, sd, interp)
+    op.update(c["roi"], c["affine"], dw, dh)
+    out = op.alloc_output()
+    op.launch(_gpu(c["img"]), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="warp")
+
+
+def test_rotate_and_odd_shapes(ctx):
+    rng = np.random.default_rng(13)
+    n, H, W = 5, 75, 101
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.5)
+    roi = np.array([[0, 0, 101, 75], [3, 2, 90, 70], [0, 0, 50, 75], [0, 0, 101, 75], [7, 7, 64, 64]], np.uint32)
+    angle = np.array([45.0, -30.0, 90.0, 0.0, 179.0], np.float32)
+    dw = np.array([101, 90, 80, 101, 64], np.uint32)
+    dh = np.array([75, 70, 75, 75, 64], np.uint32)
+    m = np.stack([orc.rotate_matrix(a) for a in angle])
+    exp = orc.warp_affine(img, roi, m, dw, dh, H, W, interp=orc.LINEAR)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    op = ops.Rotate(ctx, sd, sd, ops.LINEAR)
+    op.update(roi, angle, dw, dh)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="rotate")
+
+
+def test_warp_minification_falls_back_to_global_gather(ctx):
+    """Scale 6x: the source box of a tile exceeds the LDS slice, the kernel gathers from global memory."""
+    rng = np.random.default_rng(14)
+    n, H, W = 2, 400, 400
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.5)
+    roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
+    affine = np.array([[6.0, 0.3, -0.2, 5.5, 3.0, -2.0], [0.2, 7.0, -6.5, 0.1, 0.0, 0.0]], np.float32)
+    dw = np.full(n, 64, np.uint32)
+    dh = np.full(n, 64, np.uint32)
+    m = np.stack([orc.affine_from_rocal(a) for a in affine])
+    exp = orc.warp_affine(img, roi, m, dw, dh, 64, 64, interp=orc.LINEAR)
+    op = ops.WarpAffine(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 64, 64, ops.NHWC, ops.UINT8), ops.LINEAR)
+    op.update(roi, affine, dw, dh)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="warp minify")
+
+
+# ------------------------------------------------------------------ error behaviour
+
+def test_errors_are_loud(ctx):
+    sd = ops.desc(2, 8, 8, ops.NHWC, ops.UINT8)
+    with pytest.raises(RuntimeError, match="interpolation"):
+        ops.Resize(ctx, sd, sd, 2)  # cubic is outside the hot path
+    with pytest.raises(RuntimeError, match="uint8 NHWC"):
+        ops.Crop(ctx, ops.desc(2, 8, 8, ops.NCHW, ops.FP32), sd)
+    with pytest.raises(RuntimeError, match="batch size"):
+        ops.Crop(ctx, sd, ops.desc(3, 8, 8, ops.NHWC, ops.UINT8))
+    op = ops.Resize(ctx, sd, sd, ops.LINEAR)
+    import torch
+    with pytest.raises(RuntimeError, match="before its first update"):
+        op.launch(torch.zeros(2, 8, 8, 3, dtype=torch.uint8, device="cuda"), op.alloc_output())
+    roi = np.tile(np.array([0, 0, 8, 8], np.uint32), (2, 1))
+    with pytest.raises(RuntimeError, match="standard deviation"):
+        op.update(roi, [4, 4], [4, 4], None, np.zeros(6, np.float32), np.zeros(6, np.float32))
