@@ -1,0 +1,219 @@
+#!/usr/bin/env python3
+"""Benchmark of the augmentation hot path on one MI355X.
+
+A step is one pass of the hot path over one batch: the launch that replaces vxProcessGraph for
+the fused node (what rocAL's own process timer brackets). Inputs and the per-batch parameter
+table are resident in HBM when the timed region starts. Prints ONE JSON line on stdout.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--all] [--no-cpu]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published
+
+WORKLOADS = {
+    0: "C0 CropMirrorNormalize 256x256->224x224 fp32 NCHW batch 128 (configs[0])",
+    1: "C1 RandomResizedCrop+CropMirrorNormalize ragged[240..640]->224x224 fp16 NCHW batch 256 (configs[1])",
+    2: "C2 ColorTwist 224x224 u8->u8 NHWC batch 256 (configs[2])",
+    3: "C3 WarpAffine 512x512 u8->u8 NHWC batch 128 (configs[3])",
+    4: "C4 triangular 1920x1080->640x360 +normalize fp16 NCHW batch 32 (configs[4])",
+}
+
+
+def build_case(cfg, ctx, n=None):
+    """Returns (op, src_tensor, dst_tensor, n_images, cpu_fn) for a configuration; cpu_fn(k) runs the
+    CPU checker on the first k images of the same batch."""
+    import torch
+    from rocal_amd import ops, workloads as wl
+
+    def scale_bias(k):
+        inv = (1 / wl.STD).astype(np.float32)
+        return np.tile(inv, k), np.tile(-(wl.MEAN * inv), k)
+
+    if cfg == 0:
+        n = n or 128
+        c = wl.config0(n)
+        scale, bias = scale_bias(n)
+        op = ops.CropMirrorNormalize(ctx, ops.desc(n, 256, 256, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP32))
+        op.update(c["crop"], scale, bias, c["mirror"])
+
+        def cpu(k):
+            from oracle import orc
+            return orc.crop_mirror_normalize(c["img"][:k], c["crop"][:k], scale[:3 * k], bias[:3 * k], c["mirror"][:k], 224, 224, orc.NCHW, orc.FP32)
+    elif cfg == 1:
+        n = n or 256
+        c = wl.config1(n)
+        scale, bias = scale_bias(n)
+        dw = np.full(n, 224, np.uint32)
+        op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+        op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
+
+        def cpu(k):
+            from oracle import orc
+            return orc.resize(c["img"][:k], c["roi"][:k], dw[:k], dw[:k], 224, 224, interp=orc.LINEAR, mirror=c["mirror"][:k],
+                              scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16, flags=orc.F_QUANTIZE_U8)
+    elif cfg == 2:
+        n = n or 256
+        c = wl.config2(n)
+        sd = ops.desc(n, 224, 224, ops.NHWC, ops.UINT8)
+        op = ops.ColorTwist(ctx, sd, sd)
+        op.update(c["roi"], c["alpha"], c["beta"], c["hue"], c["sat"])
+
+        def cpu(k):
+            from oracle import orc
+            return orc.color_twist(c["img"][:k], c["roi"][:k], c["alpha"][:k], c["beta"][:k], c["hue"][:k], c["sat"][:k])
+    elif cfg == 3:
+        n = n or 128
+        c = wl.config3(n)
+        sd = ops.desc(n, 512, 512, ops.NHWC, ops.UINT8)
+        dw = np.full(n, 512, np.uint32)
+        op = ops.WarpAffine(ctx, sd, sd, ops.LINEAR)
+        op.update(c["roi"], c["affine"], dw, dw)
+
+        def cpu(k):
+            from oracle import orc
+            m = np.stack([orc.affine_from_rocal(a) for a in c["affine"][:k]])
+            return orc.warp_affine(c["img"][:k], c["roi"][:k], m, dw[:k], dw[:k], 512, 512)
+    elif cfg == 4:
+        n = n or 32
+        c = wl.config4(n)
+        dw = np.full(n, 640, np.uint32)
+        dh = np.full(n, 360, np.uint32)
+        op = ops.Resize(ctx, ops.desc(n, 1080, 1920, ops.NHWC, ops.UINT8), ops.desc(n, 360, 640, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+        op.update(c["roi"], dw, dh, c["mirror"], np.tile(wl.MEAN, n), np.tile(wl.STD, n))
+        scale, bias = scale_bias(n)
+
+        def cpu(k):
+            from oracle import orc
+            return orc.resize(c["img"][:k], c["roi"][:k], dw[:k], dh[:k], 360, 640, interp=orc.TRIANGULAR, mirror=c["mirror"][:k],
+                              scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16)
+    else:
+        raise SystemExit("unknown config %r" % cfg)
+    src = torch.from_numpy(c["img"]).cuda()
+    dst = op.alloc_output()
+    return op, src, dst, n, cpu
+
+
+def time_launches(op, src, dst, steps, warmup):
+    """K launches between two HIP events recorded on the stream the kernel runs on."""
+    import torch
+    for _ in range(warmup):
+        op.launch(src, dst)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        op.launch(src, dst)
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return e0.elapsed_time(e1) / steps, wall * 1e3 / steps  # ms per launch (device), ms per step (host clock)
+
+
+def copy_ceiling(ctx, nbytes=1 << 30, reps=20):
+    import torch
+    a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    a.zero_()
+    for _ in range(3):
+        ctx.copy_bytes(a, b, nbytes)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        ctx.copy_bytes(a, b, nbytes)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / reps
+    return 2.0 * nbytes / (ms * 1e-3) / 1e9  # read + write
+
+
+def cpu_baseline(cpu_fn, n, budget_s=12.0):
+    """Times the CPU checker (a port of the reference semantics, OpenMP over samples) on a bounded
+    sample of the same batch."""
+    from oracle import orc
+    k = min(n, 16)
+    t0 = time.perf_counter()
+    cpu_fn(k)
+    dt = time.perf_counter() - t0
+    per_img = dt / k
+    k2 = int(max(k, min(n, budget_s / max(per_img, 1e-9))))
+    reps = max(1, int(budget_s / max(per_img * k2, 1e-9)))
+    reps = min(reps, 50)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        cpu_fn(k2)
+    dt = time.perf_counter() - t0
+    return {"value": round(k2 * reps / dt, 1), "unit": "images/s", "cores": orc.num_threads(), "kind": "port",
+            "sample": "%d images of the same batch x %d passes (%.1f s)" % (k2, reps, dt)}
+
+
+def run_config(cfg, ctx, steps, warmup, with_cpu):
+    import torch
+    op, src, dst, n, cpu_fn = build_case(cfg, ctx)
+    ms_kernel, ms_step = time_launches(op, src, dst, steps, warmup)
+    algo = op.algorithmic_bytes
+    achieved = algo / (ms_kernel * 1e-3) / 1e9
+    out = {
+        "metric": "images/s", "value": round(n / (ms_kernel * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": round(ms_kernel, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": WORKLOADS[cfg], "batch": n, "kernel": op.kernel_name, "algorithmic_bytes_per_launch": algo,
+                   "host_ms_per_step": round(ms_step, 6)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},
+    }
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline(cpu_fn, n)
+    del op, src, dst
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=1)
+    ap.add_argument("--all", action="store_true", help="also measure the other configurations (written to gpurun_out/bench_all.json)")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build measures ONE GPU (the path shards trivially by sample; no multi-GPU figure is produced). "
+                         "Run with --gpus 1.")
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    from rocal_amd import ops
+    ctx = ops.Context(0)
+    ceiling = copy_ceiling(ctx)
+    res = run_config(args.config, ctx, args.steps, args.warmup, not args.no_cpu)
+    res["metric"] = "images/s + HBM GB/s (% peak), RandomResizedCrop+CMN 224^2 fp16, batch 256" if args.config == 1 else "images/s"
+    res["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
+    res["roofline"]["frac_of_copy_ceiling"] = round(res["roofline"]["achieved"] / ceiling, 4)
+    if args.all:
+        allres = {args.config: res}
+        for cfg in range(5):
+            if cfg != args.config:
+                allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu)
+                allres[cfg]["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
+                print("config %d: %s" % (cfg, json.dumps(allres[cfg])), file=sys.stderr)
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_all.json"), "w") as f:
+            json.dump(allres, f, indent=1)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()
