@@ -168,7 +168,7 @@ def run_config(cfg, ctx, steps, warmup, with_cpu):
         "metric": "images/s", "value": round(n / (ms_kernel * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps,
         "warmup": warmup, "ms_per_step": round(ms_kernel, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": WORKLOADS[cfg], "batch": n, "kernel": op.kernel_name, "algorithmic_bytes_per_launch": algo,
+        "config": {"workload": WORKLOADS[cfg], "batch": n, "kernel": op.kernel_name, "algorithmic_bytes_per_launch": algo, "plan": op.plan,
                    "host_ms_per_step": round(ms_step, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None},

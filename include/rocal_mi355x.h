@@ -78,6 +78,8 @@ RMX_API int rmx_op_launch(rmx_op *op, const void *src, void *dst);
 RMX_API int rmx_op_destroy(rmx_op *op);
 /* Algorithmic bytes of the last update: sum of source-window bytes + destination bytes. */
 RMX_API uint64_t rmx_op_algorithmic_bytes(const rmx_op *op);
+/* Launch plan of the last update as text (waves, strips, LDS per wave ...), for logs and benchmarks. */
+RMX_API const char *rmx_op_plan(const rmx_op *op);
 /* Name of the kernel the op launches (as it appears in a rocprofv3 kernel trace). */
 RMX_API const char *rmx_op_kernel_name(const rmx_op *op);
 

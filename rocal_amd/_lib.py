@@ -6,7 +6,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "librocal_mi355x.so")
+LIB_PATH = os.environ.get("RMX_LIB", os.path.join(_HERE, "lib", "librocal_mi355x.so"))
 
 
 class TensorDesc(C.Structure):
@@ -36,6 +36,7 @@ _SIGS = {
     "rmx_op_destroy": [_vp],
     "rmx_op_algorithmic_bytes": [_vp],
     "rmx_op_kernel_name": [_vp],
+    "rmx_op_plan": [_vp],
     "rmx_create_crop_mirror_normalize": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
     "rmx_update_crop_mirror_normalize": [_vp, _vp, _vp, _vp, _vp],
     "rmx_create_crop": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
@@ -62,7 +63,7 @@ _SIGS = {
     "rmx_copy_bytes": [_vp, _vp, _vp, C.c_size_t],
 }
 _RESTYPES = {"rmx_last_error": C.c_char_p, "rmx_version": C.c_char_p, "rmx_ctx_stream": _vp,
-             "rmx_op_algorithmic_bytes": C.c_uint64, "rmx_op_kernel_name": C.c_char_p}
+             "rmx_op_algorithmic_bytes": C.c_uint64, "rmx_op_kernel_name": C.c_char_p, "rmx_op_plan": C.c_char_p}
 
 EXPORTS = tuple(_SIGS)
 

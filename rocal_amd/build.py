@@ -9,7 +9,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(HERE, "lib", "obj")
-LIB = os.path.join(LIBDIR, "librocal_mi355x.so")
+LIB = os.path.join(LIBDIR, os.environ.get("RMX_LIB_NAME", "librocal_mi355x.so"))  # override: experiment builds
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # -ffp-contract=off: the kernels spell every fused multiply-add out (bit-exact parity with the
@@ -21,7 +21,7 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 
 def _compile(src):
     obj = os.path.join(OBJDIR, os.path.basename(src) + ".o")
-    cmd = [HIPCC] + FLAGS + ["-c", src, "-o", obj]
+    cmd = [HIPCC] + FLAGS + os.environ.get("RMX_EXTRA_FLAGS", "").split() + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature name: that warning is expected
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

@@ -70,6 +70,8 @@ struct rmx_op {
     // launch plan of the last update
     rmx::KernelFn fn = nullptr;
     const char *kernel_name = "";
+    rmx::KernelFn fn_fast = nullptr;  // specialisation usable when the destination base is 16-byte aligned
+    const char *fast_name = "";
     int strips = 1, strip_rows = 1, tile_w = 512, lds_per_wave = 0, waves_per_block = 4;
     int aux0 = 0, aux1 = 0;
     uint64_t algo_bytes = 0;
@@ -235,7 +237,15 @@ int rmx_op_destroy(rmx_op *op) {
 }
 
 uint64_t rmx_op_algorithmic_bytes(const rmx_op *op) { return op ? op->algo_bytes : 0; }
-const char *rmx_op_kernel_name(const rmx_op *op) { return op ? op->kernel_name : ""; }
+
+const char *rmx_op_plan(const rmx_op *op) {
+    static thread_local char buf[256];
+    if (!op) return "";
+    snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=%d",
+             (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block, op->fn_fast != nullptr);
+    return buf;
+}
+const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : op->kernel_name) : ""; }
 
 int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
@@ -255,6 +265,8 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.lds_bytes = op->lds_per_wave;
     a.aux0 = op->aux0;
     a.aux1 = op->aux1;
+    a.dbg = nullptr;
+    if (const char *e = getenv("RMX_EXP_DBGPTR")) a.dbg = (uint64_t *)strtoull(e, nullptr, 0);
     const uint64_t waves = (uint64_t)op->n * (uint64_t)op->strips;
     const int wpb = op->waves_per_block;
     const uint64_t blocks = (waves + wpb - 1) / wpb;
@@ -262,7 +274,8 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     const size_t lds = (size_t)op->lds_per_wave * wpb;
     if (lds > (size_t)op->ctx->max_lds_per_block) return fail(RMX_ERR_INVALID, "plan needs %zu bytes of LDS per workgroup (limit %d)", lds, op->ctx->max_lds_per_block);
     HIP_TRY(hipSetDevice(op->ctx->device));
-    hipLaunchKernelGGL(op->fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
+    rmx::KernelFn fn = (op->fn_fast && (((uintptr_t)dst) & 15u) == 0) ? op->fn_fast : op->fn;
+    hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
     HIP_TRY(hipGetLastError());
     return RMX_OK;
 }
@@ -347,6 +360,14 @@ int rmx_create_resize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor
     return RMX_OK;
 }
 
+// the kernels' source-coordinate law, evaluated on the host in the same fp32 operation order
+static inline float src_coord_h(int u, float ratio, float off, float lo) {
+    float s = (float)u * ratio;
+    s = s + off;
+    s = s + lo;
+    return s;
+}
+
 static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     const bool quant = (op->flags & RMX_F_QUANTIZE_U8) != 0;
     // a quantised value that is not normalised is stored through an identity FMA
@@ -396,24 +417,48 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                  ? rmx::select_resize_nearest_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm)
                  : rmx::select_resize_linear_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm);
     op->kernel_name = nm;
-    // x-tile: up to 64 lanes x 8 px; LDS per wave = rows x (staged columns + pads) dwords
+    // x-tile: up to 64 lanes x 8 px. Each wave keeps a ring of R staged source rows in LDS;
+    // R and the row pitch are computed per sample with the kernel's own float formulas.
     int tile_w = std::min(((max_dw + 7) / 8) * 8, 512);
-    const int budget = 24 * 1024;
+    const int budget = 16 * 1024;
     int lds = 0;
     for (;;) {
         lds = 0;
         for (int i = 0; i < op->n; i++) {
-            const RmxSample &s = t[i];
-            if (s.dst_w <= 0 || s.dst_h <= 0) continue;
-            for (int pass = 0; pass < 2; pass++) {
-                int tw = pass == 0 ? std::min<int>(tile_w, s.dst_w) : (s.dst_w % tile_w);
-                if (tw <= 0) continue;
-                int L = (tw + 7) / 8, G = 64 / L;
-                int rows = (int)std::ceil((G - 1) * (double)s.ry) + 4;
-                int cols = std::min<int>(s.src_w, (int)std::ceil(tw * (double)s.rx) + 3);
-                int pitch = 4 + ((cols + 3) / 4) * 4 + 4;
-                lds = std::max(lds, rows * pitch * 4);
+            RmxSample &s = t[i];
+            if (s.dst_w <= 0 || s.dst_h <= 0) {
+                s.strip_rows = 1;
+                continue;
             }
+            const float offx = (s.rx - 1.0f) * 0.5f, offy = (s.ry - 1.0f) * 0.5f;
+            const int xlo = s.src_x, xhi = s.src_x + s.src_w - 1;
+            int ring = 1, pitch_max = 0, maxnew = 0;
+            for (int xt = 0; xt < s.dst_w; xt += tile_w) {
+                const int tw = std::min<int>(s.dst_w - xt, tile_w);
+                const int L = (tw + 7) / 8, G = 64 / L;
+                const int ixmin = (int)std::floor(src_coord_h(s.pc_x + xt, s.rx, offx, (float)xlo));
+                const int ixmax = (int)std::floor(src_coord_h(s.pc_x + xt + tw - 1, s.rx, offx, (float)xlo));
+                const int cs = std::max(std::min(ixmin, xhi), xlo), ce = std::max(std::min(ixmax + 1, xhi), xlo);
+                const int items = (ce - cs + 1 + 3) >> 2;
+                pitch_max = std::max(pitch_max, 4 + items * 4 + 4);
+                if (xt == 0 || tw != tile_w) {  // G only changes on the last, narrower tile
+                    for (int r = 0; r < s.dst_h; r++) {
+                        const int re = std::min(r + G - 1, s.dst_h - 1);
+                        const int a_k = (int)std::floor(src_coord_h(s.pc_y + r, s.ry, offy, (float)s.src_y));
+                        const int b_k = (int)std::floor(src_coord_h(s.pc_y + re, s.ry, offy, (float)s.src_y)) + 1;
+                        ring = std::max(ring, b_k - a_k + 1);
+                        if (r + G < s.dst_h) {  // rows that enter the window when the step after this one is staged
+                            const int rn = std::min(r + 2 * G - 1, s.dst_h - 1);
+                            const int a_n = (int)std::floor(src_coord_h(s.pc_y + r + G, s.ry, offy, (float)s.src_y));
+                            const int b_n = (int)std::floor(src_coord_h(s.pc_y + rn, s.ry, offy, (float)s.src_y)) + 1;
+                            maxnew = std::max(maxnew, b_n - std::max(b_k + 1, a_n) + 1);
+                        }
+                    }
+                }
+            }
+            s.strip_rows = ring;
+            s.flags = (s.flags & 0xffffu) | ((uint32_t)std::min(maxnew, 0xffff) << 16);
+            lds = std::max(lds, ring * pitch_max * 4);
         }
         if (lds <= budget || tile_w <= 64) break;
         tile_w = std::max(64, (tile_w / 2 + 7) / 8 * 8);
@@ -424,9 +469,25 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     op->waves_per_block = std::max(1, std::min(4, op->ctx->max_lds_per_block / std::max(1, op->lds_per_wave)));
     op->tile_w = tile_w;
     op->aux1 = tile_w;
-    op->strip_rows = 8;
-    op->aux0 = op->strip_rows;
-    op->strips = std::max(1, (max_dh + op->strip_rows - 1) / op->strip_rows);
+    // strips: short ones. A wave's steps are serialised by memory latency, so many short-lived
+    // waves (several residency rounds) overlap better than one long-lived wave per slot; the
+    // price is one extra window of source rows per strip. 8 rows measured best on MI355X.
+    {
+        int rows = 8;
+        if (const char *e = getenv("RMX_EXP_STRIP_ROWS")) rows = atoi(e);
+        if (const char *e = getenv("RMX_EXP_WPB")) op->waves_per_block = atoi(e);
+        if (const char *e = getenv("RMX_EXP_LDS")) op->lds_per_wave = atoi(e);
+        op->strip_rows = rows;
+        op->aux0 = rows;
+        op->strips = std::max(1, (max_dh + rows - 1) / rows);
+    }
+    // fast path: every written width a multiple of 8 and aligned destination rows
+    op->fn_fast = nullptr;
+    if (op->interp == RMX_INTERP_LINEAR && op->dst.w % 8 == 0) {
+        bool ok = true;
+        for (int i = 0; i < op->n && ok; i++) ok = (t[i].dst_w % 8 == 0);
+        if (ok) op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->fast_name);
+    }
     return RMX_OK;
 }
 

@@ -37,6 +37,7 @@ struct RmxKArgs {
     int32_t strips;          // wave strips per sample (grid = n*strips waves)
     int32_t lds_bytes;       // dynamic LDS per wave
     int32_t aux0, aux1;
+    uint64_t *dbg;           // experiment builds only: per-wave timestamps (NULL otherwise)
 };
 
 #define RMX_WAVE 64

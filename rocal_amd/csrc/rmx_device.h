@@ -51,9 +51,8 @@ RMX_DEV uint32_t xcd_swizzle(uint32_t b, uint32_t nblocks) {
 // past the dword that holds the last byte of the batch buffer.
 template <int ND>
 RMX_DEV void load_realigned(const uint8_t *p, const uint8_t *buf_end, uint32_t (&out)[ND - 1]) {
-    uintptr_t a = (uintptr_t)p;
-    uint32_t phase = (uint32_t)(a & 3u);
-    const uint32_t *q = (const uint32_t *)(a & ~(uintptr_t)3);
+    const uint32_t phase = (uint32_t)((uintptr_t)p & 3u);
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(p - phase);  // keeps the global address space
     uint32_t d[ND];
     if ((const uint8_t *)(q + ND) <= buf_end) {
         if constexpr (ND == 4) {
@@ -73,6 +72,34 @@ RMX_DEV void load_realigned(const uint8_t *p, const uint8_t *buf_end, uint32_t (
     }
 #pragma unroll
     for (int i = 0; i < ND - 1; i++) out[i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], phase);
+}
+
+// Split form of load_realigned<4> for software pipelining: issue the 128-bit load now, realign
+// later (so that several loads can be in flight before the first use).
+RMX_DEV uint32_t load_raw4(const uint8_t *p, const uint8_t *buf_end, uint32_t (&d)[4]) {
+    const uint32_t phase = (uint32_t)((uintptr_t)p & 3u);
+    const uint32_t *q = reinterpret_cast<const uint32_t *>(p - phase);
+    if ((const uint8_t *)(q + 4) <= buf_end) {
+        u32x4_a4 t = *reinterpret_cast<const u32x4_a4 *>(q);
+        d[0] = t.x; d[1] = t.y; d[2] = t.z; d[3] = t.w;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; i++) d[i] = ((const uint8_t *)(q + i) < buf_end) ? q[i] : 0u;
+    }
+    return phase;
+}
+
+// raw dwords + byte phase -> 4 packed pixels expanded to one dword each (top byte is don't-care)
+RMX_DEV uint4 expand4(const uint32_t (&d)[4], uint32_t phase) {
+    uint32_t w0 = __builtin_amdgcn_alignbyte(d[1], d[0], phase);
+    uint32_t w1 = __builtin_amdgcn_alignbyte(d[2], d[1], phase);
+    uint32_t w2 = __builtin_amdgcn_alignbyte(d[3], d[2], phase);
+    uint4 px;
+    px.x = w0;
+    px.y = __builtin_amdgcn_alignbyte(w1, w0, 3);
+    px.z = __builtin_amdgcn_alignbyte(w2, w1, 2);
+    px.w = w2 >> 8;
+    return px;
 }
 
 // 8 packed RGB pixels (24 bytes = 6 dwords, byte 0 = R of pixel 0) -> v[c][k]
@@ -138,6 +165,108 @@ RMX_DEV void store_run(T *p, const T (&e)[N], int cnt) {
 #pragma unroll
     for (int i = 0; i < N; i++)
         if (i < cnt) p[i] = e[i];
+}
+
+// Full-group store for callers that have established alignment: N*sizeof(T) is a multiple of 8
+// and p is aligned to min(16, N*sizeof(T) & -N*sizeof(T)) bytes.
+template <typename T, int N>
+RMX_DEV void store_run_aligned(T *p, const T (&e)[N]) {
+    constexpr int BYTES = N * (int)sizeof(T);
+    if constexpr (BYTES % 16 == 0) {
+        uint4 t[BYTES / 16];
+        __builtin_memcpy(t, e, BYTES);
+#pragma unroll
+        for (int i = 0; i < BYTES / 16; i++) reinterpret_cast<uint4 *>(p)[i] = t[i];
+    } else {
+        static_assert(BYTES % 8 == 0, "group must be a multiple of 8 bytes");
+        uint2 t[BYTES / 8];
+        __builtin_memcpy(t, e, BYTES);
+#pragma unroll
+        for (int i = 0; i < BYTES / 8; i++) reinterpret_cast<uint2 *>(p)[i] = t[i];
+    }
+}
+
+// Full, aligned group of PX pixels (see store_group for the meaning of rev).
+template <typename T, int LAYOUT>
+RMX_DEV void store_group_aligned(T *sample, int H, int W, int y, int x0, const float (&v)[3][PX], bool rev) {
+    if constexpr (LAYOUT == RMX_NCHW) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            T e[PX];
+#pragma unroll
+            for (int k = 0; k < PX; k++) e[k] = OutCvt<T>::cvt(rev ? v[c][PX - 1 - k] : v[c][k]);
+            store_run_aligned<T, PX>(sample + ((size_t)c * H + y) * W + x0, e);
+        }
+    } else {
+        T e[PX * 3];
+#pragma unroll
+        for (int k = 0; k < PX; k++)
+#pragma unroll
+            for (int c = 0; c < 3; c++) e[k * 3 + c] = OutCvt<T>::cvt(rev ? v[c][PX - 1 - k] : v[c][k]);
+        store_run_aligned<T, PX * 3>(sample + ((size_t)y * W + x0) * 3, e);
+    }
+}
+
+// Split form of store_group_aligned: pack now (values become PX*3*sizeof(T) bytes of registers in
+// memory order), store later. Lets a kernel keep finished pixels in few registers while other
+// memory operations complete.
+template <typename T>
+struct PackedGroup {
+    static constexpr int WORDS = PX * 3 * (int)sizeof(T) / 4;
+    uint32_t w[WORDS];
+};
+
+template <typename T, int LAYOUT, bool REV>
+RMX_DEV void pack_group_dir(const float (&v)[3][PX], PackedGroup<T> &out) {
+    T e[PX * 3];
+    if constexpr (LAYOUT == RMX_NCHW) {
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+#pragma unroll
+            for (int k = 0; k < PX; k++) e[c * PX + k] = OutCvt<T>::cvt(REV ? v[c][PX - 1 - k] : v[c][k]);
+    } else {
+#pragma unroll
+        for (int k = 0; k < PX; k++)
+#pragma unroll
+            for (int c = 0; c < 3; c++) e[k * 3 + c] = OutCvt<T>::cvt(REV ? v[c][PX - 1 - k] : v[c][k]);
+    }
+    __builtin_memcpy(out.w, e, sizeof(e));
+}
+
+// rev is wave-uniform (one sample per wave): branch once instead of selecting per element
+template <typename T, int LAYOUT>
+RMX_DEV void pack_group(const float (&v)[3][PX], bool rev, PackedGroup<T> &out) {
+    if (rev) pack_group_dir<T, LAYOUT, true>(v, out);
+    else pack_group_dir<T, LAYOUT, false>(v, out);
+}
+
+template <typename T, int LAYOUT>
+RMX_DEV void store_packed(T *sample, int H, int W, int y, int x0, const PackedGroup<T> &g) {
+    constexpr int PW = PX * (int)sizeof(T) / 4;  // dwords per channel run
+    if constexpr (LAYOUT == RMX_NCHW) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            T *p = sample + ((size_t)c * H + y) * W + x0;
+            if constexpr (PW % 4 == 0) {
+#pragma unroll
+                for (int i = 0; i < PW / 4; i++)
+                    reinterpret_cast<uint4 *>(p)[i] = make_uint4(g.w[c * PW + 4 * i], g.w[c * PW + 4 * i + 1], g.w[c * PW + 4 * i + 2], g.w[c * PW + 4 * i + 3]);
+            } else {
+#pragma unroll
+                for (int i = 0; i < PW / 2; i++) reinterpret_cast<uint2 *>(p)[i] = make_uint2(g.w[c * PW + 2 * i], g.w[c * PW + 2 * i + 1]);
+            }
+        }
+    } else {
+        T *p = sample + ((size_t)y * W + x0) * 3;
+        constexpr int TW = PackedGroup<T>::WORDS;
+        if constexpr (TW % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < TW / 4; i++) reinterpret_cast<uint4 *>(p)[i] = make_uint4(g.w[4 * i], g.w[4 * i + 1], g.w[4 * i + 2], g.w[4 * i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < TW / 2; i++) reinterpret_cast<uint2 *>(p)[i] = make_uint2(g.w[2 * i], g.w[2 * i + 1]);
+        }
+    }
 }
 
 // Write one lane's group of N horizontally adjacent pixels (v[c][k], k-th pixel of the group)

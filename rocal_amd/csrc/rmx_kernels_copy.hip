@@ -14,7 +14,7 @@ __global__ void __launch_bounds__(256) rmx_copy_kernel(const uint4 *__restrict__
 void launch_copy(hipStream_t stream, const void *src, void *dst, size_t nbytes, int num_cus) {
     const size_t n16 = nbytes / 16;
     size_t blocks = (n16 + 255) / 256;
-    const size_t cap = (size_t)num_cus * 16;
+    const size_t cap = (size_t)num_cus * 4;  // 4 resident workgroups per CU measured best for large copies
     if (blocks > cap) blocks = cap;
     if (blocks == 0) return;
     hipLaunchKernelGGL(rmx_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint4 *)src, (uint4 *)dst, n16);

@@ -3,14 +3,17 @@
 //     ResizeCropMirror / ResizeMirrorNormalize and the fused RandomResizedCrop + CMN chain.
 //
 // Scheduling is wavefront-granular: every wavefront owns a strip of output rows of one sample
-// and a private slice of LDS; there is no workgroup barrier anywhere. Per step the wave
-//   1. stages the source rows its G output rows touch into LDS with dword-aligned 128-bit
-//      global loads (12 useful bytes = 4 packed pixels per lane), expanding each pixel to one
-//      dword so that the gather below is bank-friendly and needs no byte addressing,
-//   2. gathers the 2x2 neighbourhoods from LDS (two adjacent-dword reads per pixel), blends
-//      in fp32 in the reference's FMA order, applies the epilogue and
-//   3. writes 8 pixels per lane with 128-bit stores (fp16 planar).
-// HBM-bound: each source byte of the window is fetched once per strip (halo rows hit L1/L2).
+// and a private slice of LDS; there is no workgroup barrier anywhere. The wave walks down its
+// strip in steps of G output rows (G = 64 / lanes-per-row) and keeps a ring of staged source
+// rows in LDS, so every source row is fetched once per strip:
+//   stage    rows entering the window are read with dword-aligned 128-bit global loads
+//            (12 useful bytes = 4 packed pixels per lane; the row base is wave-uniform, so the
+//            per-lane address is one precomputed offset) and expanded to one dword per pixel,
+//            which makes the gather bank-friendly and free of byte addressing;
+//   gather   two adjacent-dword LDS reads per neighbour row and pixel, fp32 blend in the
+//            reference's FMA order, epilogue, eight pixels per lane written with 128-bit stores.
+// The loads of step k+1 are issued before the arithmetic of step k and committed to LDS after
+// it, so HBM latency overlaps the blend. HBM-bound by design: window bytes in, tensor bytes out.
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
@@ -18,12 +21,82 @@ namespace rmx {
 
 extern __shared__ uint32_t rmx_lds[];
 
+constexpr int NL = 8;   // 128-bit loads a lane may hold in flight across the blend of a step
+
 // source coordinate of resized index u (rocal bilinear law: u*ratio + (ratio-1)/2 + roi.lo)
 RMX_DEV float src_coord(int u, float ratio, float off, float lo) {
     float s = (float)u * ratio;
     s = s + off;
     s = s + lo;
     return s;
+}
+
+// Everything the staging of one x-tile needs; all members are wave-uniform.
+struct StageCtx {
+    const uint8_t *base4;  // sample base rounded down to 4 bytes (global memory)
+    uint32_t skew;         // sample base - base4
+    uint32_t lim;          // bytes from base4 to the end of the batch buffer (saturated to 32 bits)
+    uint32_t row_stride;   // bytes
+    int cs;                // first staged source column
+    int items;             // 4-pixel items per row
+    int ipl;               // items per lane per row = ceil(items/64)
+    int pitch;             // LDS row pitch in dwords
+    int ylo, yhi;          // ROI rows
+    int R;                 // ring rows
+};
+
+// byte offset (from base4) of the first staged pixel of virtual source row v
+RMX_DEV uint32_t stage_row_offset(const StageCtx &S, int v) {
+    const int ysrc = max(min(v, S.yhi), S.ylo);
+    return (uint32_t)ysrc * S.row_stride + (uint32_t)S.cs * 3u + S.skew;
+}
+
+// Issue the loads of staging items [first, first+NL) of the row set starting at virtual row
+// new_lo; item t is (row t / ipl, chunk t % ipl); a lane handles 4-pixel item j = lane + 64*chunk
+// of its row with one dword-aligned 128-bit load (uniform base + 32-bit lane offset).
+RMX_DEV void stage_issue(const StageCtx &S, int lane, int new_lo, int nit, int first, uint32_t (&raw)[NL][4]) {
+    int q = first / S.ipl, c = first - q * S.ipl;
+#pragma unroll
+    for (int t = 0; t < NL; t++) {
+        if (first + t < nit) {
+            const uint32_t ro4 = stage_row_offset(S, new_lo + q) & ~3u;
+            const int j = lane + RMX_WAVE * c;
+            if (j < S.items) {
+                const uint32_t vo = ro4 + 12u * (uint32_t)j;
+                if (ro4 + 12u * (uint32_t)S.items + 8u <= S.lim) {  // row segment + realign slack inside the batch
+                    u32x4_a4 v = *reinterpret_cast<const u32x4_a4 *>(S.base4 + vo);
+                    raw[t][0] = v.x; raw[t][1] = v.y; raw[t][2] = v.z; raw[t][3] = v.w;
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) raw[t][i] = (vo + 4u * i < S.lim) ? *reinterpret_cast<const uint32_t *>(S.base4 + vo + 4u * i) : 0u;
+                }
+            }
+            if (++c == S.ipl) {
+                c = 0;
+                q++;
+            }
+        }
+    }
+}
+
+// Expand the loaded items and write them to their ring slots.
+RMX_DEV void stage_commit(const StageCtx &S, uint32_t *lds, int lane, int new_lo, int slot_new, int nit, int first,
+                          const uint32_t (&raw)[NL][4]) {
+    int q = first / S.ipl, c = first - q * S.ipl;
+#pragma unroll
+    for (int t = 0; t < NL; t++) {
+        if (first + t < nit) {
+            const uint32_t phase = stage_row_offset(S, new_lo + q) & 3u;
+            int sl = slot_new + q;
+            if (sl >= S.R) sl -= S.R;
+            const int j = lane + RMX_WAVE * c;
+            if (j < S.items) *reinterpret_cast<uint4 *>(lds + sl * S.pitch + 4 + 4 * j) = expand4(raw[t], phase);
+            if (++c == S.ipl) {
+                c = 0;
+                q++;
+            }
+        }
+    }
 }
 
 template <typename T, int LAYOUT, bool NORM, bool QUANT, bool NEAREST>
@@ -52,9 +125,6 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
     const float fxlo = (float)xlo, fylo = (float)ylo;
     const int pcx = P.pc_x, pcy = P.pc_y;
 
-    const size_t row_stride = (size_t)a.src_w * 3;
-    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
-    const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
     uint32_t *lds = rmx_lds + (size_t)wib * (a.lds_bytes >> 2);
 
@@ -65,6 +135,20 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
         bi[c] = P.bias[c];
     }
 
+    StageCtx S;
+    S.row_stride = (uint32_t)a.src_w * 3u;
+    {
+        const uint8_t *simg = a.src + (size_t)s * a.src_h * S.row_stride;
+        S.skew = (uint32_t)((uintptr_t)simg & 3u);
+        S.base4 = simg - S.skew;
+        const uint64_t left = (uint64_t)((a.src + a.src_bytes) - S.base4);
+        S.lim = left > 0xffffffffull ? 0xffffffffu : (uint32_t)left;
+    }
+    S.ylo = ylo;
+    S.yhi = yhi;
+    S.R = P.strip_rows;
+    const int R = S.R;
+
     const int tile_w = a.aux1;  // output columns per x-tile (multiple of PX, <= 64*PX)
     for (int xt = 0; xt < dw; xt += tile_w) {
         const int tw = min(dw - xt, tile_w);
@@ -72,9 +156,9 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
         const int G = RMX_WAVE / L;
         const int lr = lane / L;
         const int g = lane - lr * L;
-        const int t0 = xt + g * PX;                 // first window-relative column of the group
+        const int t0 = xt + g * PX;  // first window-relative column of the group
         const int cnt = min(PX, dw - t0);
-        const bool lane_on = lr < G;
+        const bool lane_on = lr < G && cnt > 0;
 
         // tile-wide source column range (wave-uniform)
         const int u_first = pcx + xt, u_last = pcx + xt + tw - 1;
@@ -83,11 +167,14 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
         const int cs = max(min(ixmin, xhi), xlo);
         const int ce = max(min(ixmax + 1, xhi), xlo);
         const int nc = ce - cs + 1;
-        const int items = (nc + 3) >> 2;
-        const int pitch = 4 + items * 4 + 4;
         const bool rep_l = ixmin < xlo, rep_r = ixmax + 1 > xhi;
+        S.cs = cs;
+        S.items = (nc + 3) >> 2;
+        S.ipl = (S.items + RMX_WAVE - 1) / RMX_WAVE;
+        S.pitch = 4 + S.items * 4 + 4;
+        const int pitch = S.pitch;
 
-        // per-lane column taps, fixed for the whole strip
+        // per-lane column taps, fixed for the whole strip (LDS dword index of the left neighbour)
         int off[PX];
         float wx[PX];
 #pragma unroll
@@ -99,50 +186,56 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
             off[k] = 4 + ((int)fx - cs);
         }
 
-        for (int rs = r0; rs < r1; rs += G) {
-            // rows of this step: rs .. min(rs+G, r1)-1 ; virtual source rows they touch
-            const int re = min(rs + G, r1) - 1;
-            const int iy_first = (int)floorf(src_coord(pcy + rs, ry, offy, fylo));
-            const int iy_last = (int)floorf(src_coord(pcy + re, ry, offy, fylo));
-            const int nrows = iy_last - iy_first + 2;
-
-            // ---- stage: (row slot q, item j) pairs dealt over the lanes
-            {
-                int q = 0, j = lane;
-                while (j >= items) { j -= items; q++; }
-                while (q < nrows) {
-                    const int ysrc = max(min(iy_first + q, yhi), ylo);
-                    const uint8_t *p = simg + (size_t)ysrc * row_stride + (size_t)(cs + 4 * j) * 3;
-                    uint32_t w[3];
-                    load_realigned<4>(p, buf_end, w);
-                    uint4 px;
-                    px.x = w[0];
-                    px.y = __builtin_amdgcn_alignbyte(w[1], w[0], 3);
-                    px.z = __builtin_amdgcn_alignbyte(w[2], w[1], 2);
-                    px.w = w[2] >> 8;
-                    *reinterpret_cast<uint4 *>(lds + q * pitch + 4 + 4 * j) = px;
-                    j += RMX_WAVE;
-                    while (j >= items) { j -= items; q++; }
-                }
+        // ---- first step: stage its whole window
+        int a_k = (int)floorf(src_coord(pcy + r0, ry, offy, fylo));
+        int b_k = (int)floorf(src_coord(pcy + min(r0 + G, r1) - 1, ry, offy, fylo)) + 1;
+        int base_slot = 0;
+        uint32_t raw[NL][4];
+        {
+            const int nnew = b_k - a_k + 1, nit = nnew * S.ipl;
+            for (int first = 0; first < nit; first += NL) {
+                stage_issue(S, lane, a_k, nit, first, raw);
+                stage_commit(S, lds, lane, a_k, 0, nit, first, raw);
             }
             wave_sync();
-            if (rep_l || rep_r) {
-                if (lane < nrows) {
-                    uint32_t *row = lds + lane * pitch;
-                    if (rep_l) row[3] = row[4];
-                    if (rep_r) row[4 + nc] = row[4 + nc - 1];
-                }
-                wave_sync();
+            if ((rep_l || rep_r) && lane < nnew) {
+                uint32_t *row = lds + lane * pitch;
+                if (rep_l) row[3] = row[4];
+                if (rep_r) row[4 + nc] = row[4 + nc - 1];
+            }
+            wave_sync();
+        }
+
+        for (int rs = r0; rs < r1; rs += G) {
+            const int re = min(rs + G, r1) - 1;
+            // ---- next step's window; issue its loads before this step's arithmetic
+            const bool has_next = rs + G < r1;
+            int a_n = a_k, b_n = b_k, new_lo = 0, nnew = 0, nit = 0, base_slot_n = base_slot, slot_new = 0;
+            if (has_next) {
+                a_n = (int)floorf(src_coord(pcy + rs + G, ry, offy, fylo));
+                b_n = (int)floorf(src_coord(pcy + min(rs + 2 * G, r1) - 1, ry, offy, fylo)) + 1;
+                base_slot_n = base_slot + (a_n - a_k);
+                while (base_slot_n >= R) base_slot_n -= R;
+                new_lo = max(b_k + 1, a_n);
+                nnew = b_n - new_lo + 1;
+                nit = nnew * S.ipl;
+                slot_new = base_slot_n + (new_lo - a_n);
+                if (slot_new >= R) slot_new -= R;
+                stage_issue(S, lane, new_lo, nit, 0, raw);
             }
 
-            // ---- gather + blend + epilogue
+            // ---- gather + blend + epilogue for rows rs..re
             const int r = rs + lr;
-            if (lane_on && r <= re && cnt > 0) {
+            if (lane_on && r <= re) {
                 float sy = src_coord(pcy + r, ry, offy, fylo);
                 float fy = floorf(sy);
                 float wy = sy - fy;
-                const uint32_t *row0 = lds + ((int)fy - iy_first) * pitch;
-                const uint32_t *row1 = row0 + pitch;
+                int s0 = base_slot + ((int)fy - a_k);
+                if (s0 >= R) s0 -= R;
+                int s1 = s0 + 1;
+                if (s1 >= R) s1 -= R;
+                const uint32_t *row0 = lds + s0 * pitch;
+                const uint32_t *row1 = lds + s1 * pitch;
                 float v[3][PX];
                 if constexpr (NEAREST) {
                     const uint32_t *rsel = wy < 0.5f ? row0 : row1;
@@ -171,14 +264,36 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
 #pragma unroll
                     for (int k = 0; k < PX; k++) {
                         float t = v[c][k];
-                        if constexpr (QUANT) t = round_u8(t);
+                        // a convex blend of u8 values stays inside [0,255]: rounding alone saturates it
+                        if constexpr (QUANT) t = NEAREST ? t : __builtin_rintf(t);
                         if constexpr (NORM) t = __builtin_fmaf(t, sc[c], bi[c]);
                         v[c][k] = t;
                     }
                 const int x0 = hf ? (dw - t0 - cnt) : t0;
                 store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, x0, cnt, v, hf);
             }
-            wave_sync();  // next step overwrites the LDS rows just read
+            wave_sync();  // ring rows of this step may be overwritten from here on
+
+            // ---- commit the next step's rows
+            if (has_next) {
+                stage_commit(S, lds, lane, new_lo, slot_new, nit, 0, raw);
+                for (int first = NL; first < nit; first += NL) {
+                    stage_issue(S, lane, new_lo, nit, first, raw);
+                    stage_commit(S, lds, lane, new_lo, slot_new, nit, first, raw);
+                }
+                wave_sync();
+                if ((rep_l || rep_r) && lane < nnew) {
+                    int sl = slot_new + lane;
+                    if (sl >= R) sl -= R;
+                    uint32_t *row = lds + sl * pitch;
+                    if (rep_l) row[3] = row[4];
+                    if (rep_r) row[4 + nc] = row[4 + nc - 1];
+                }
+                wave_sync();
+                base_slot = base_slot_n;
+                a_k = a_n;
+                b_k = b_n;
+            }
         }
     }
 }

@@ -8,6 +8,7 @@ typedef void (*KernelFn)(RmxKArgs);
 
 KernelFn select_cmn_kernel(int dtype, int layout, bool norm, const char **name);
 KernelFn select_resize_linear_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
+KernelFn select_resize_fast_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_color_kernel(int kind, int dtype, int layout, const char **name);

@@ -123,6 +123,10 @@ class Op:
     def kernel_name(self):
         return _lib.lib().rmx_op_kernel_name(self._h).decode()
 
+    @property
+    def plan(self):
+        return _lib.lib().rmx_op_plan(self._h).decode()
+
     def close(self):
         if self._h:
             _lib.lib().rmx_op_destroy(self._h)
