@@ -1,0 +1,343 @@
+"""CPU tests that pin the oracle (oracle/rocal_oracle.c) against evidence that does not come
+from the oracle itself: closed forms, special cases that reduce to a library routine (numpy,
+torch.nn.functional.interpolate, colorsys), standard known answers, and invariants. A plausible
+mistake in the restatement (dropped term, wrong sign/index, transposed operand) fails one of them.
+Reference citations are relative to the rocAL tree."""
+import colorsys
+import math
+
+import numpy as np
+import pytest
+
+from oracle import orc
+
+RNG = np.random.default_rng(20240101)
+
+
+def _img(n, h, w, rng=RNG):
+    return rng.integers(0, 256, (n, h, w, 3), dtype=np.uint8)
+
+
+def _full(n, h, w):
+    return np.tile(np.array([0, 0, w, h], np.uint32), (n, 1))
+
+
+# ------------------------------------------------------------------ fp16 / stores
+
+def test_fp16_round_to_nearest_even_matches_numpy():
+    rng = np.random.default_rng(1)
+    mags = np.array([1e-8, 6e-8, 1e-6, 6.1e-5, 1e-3, 1.0, 100.0, 2047.0, 65000.0, 7e4], np.float32)
+    v = (rng.standard_normal(200000).astype(np.float32) * rng.choice(mags, 200000)).astype(np.float32)
+    edge = np.array([0.0, -0.0, 65504.0, 65519.99, 65520.0, 1e9, -1e9, 2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0001,
+                     2.0 ** -14, 2.0 ** -14 * 0.9999, 1.0009765625, 1.00048828125, 1.00146484375], np.float32)
+    v = np.concatenate([v, edge])
+    got = np.array([orc.f32_to_f16(x) for x in v], np.uint16)
+    with np.errstate(over="ignore"):
+        exp = v.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, exp)
+
+
+def test_fp16_truncation_mode_never_rounds_up_in_magnitude():
+    rng = np.random.default_rng(2)
+    v = (rng.standard_normal(20000) * 50).astype(np.float32)
+    for x in v:
+        h = np.array([orc.f32_to_f16(x, trunc=True)], np.uint16).view(np.float16)[0]
+        assert abs(float(h)) <= abs(float(x))
+        nxt = np.nextafter(np.float16(h), np.float16(np.inf if x > 0 else -np.inf))  # next half away from zero
+        assert abs(float(nxt)) > abs(float(x)) or float(h) == float(x)
+
+
+# ------------------------------------------------------------------ CropMirrorNormalize
+
+def test_cmn_scale_bias_follows_node_derivation():
+    # node_crop_mirror_normalize.cpp:56-61 : offset = 1/std (fp32), multiplier = -(mean*offset) (fp32)
+    mean = np.array([123.675, 116.28, 103.53], np.float32)
+    std = np.array([58.395, 57.12, 57.375], np.float32)
+    scale, bias = orc.cmn_scale_bias(mean, std, 2)
+    inv = (np.float32(1) / std).astype(np.float32)
+    assert np.array_equal(scale, np.tile(inv, 2))
+    assert np.array_equal(bias, np.tile(-(mean * inv), 2))
+
+
+def test_cmn_identity_normalisation_is_exact_gather():
+    img = _img(3, 20, 30)
+    crop = np.array([[2, 3, 17, 11], [0, 0, 30, 20], [29, 19, 1, 1]], np.uint32)
+    mirror = np.array([1, 0, 1], np.uint32)
+    one, zero = np.ones(9, np.float32), np.zeros(9, np.float32)
+    out = orc.crop_mirror_normalize(img, crop, one, zero, mirror, 20, 30, orc.NCHW, orc.FP32)
+    for i in range(3):
+        x, y, w, h = crop[i]
+        ref = img[i, y:y + h, x:x + w].astype(np.float32)
+        if mirror[i]:
+            ref = ref[:, ::-1]
+        assert np.array_equal(out[i, :, :h, :w], ref.transpose(2, 0, 1))
+        assert not out[i, :, h:, :].any() and not out[i, :, :, w:].any()  # padding untouched
+
+
+def test_cmn_value_is_one_fp32_fma():
+    img = _img(1, 8, 8)
+    crop = _full(1, 8, 8)
+    scale, bias = orc.cmn_scale_bias([123.675, 116.28, 103.53], [58.395, 57.12, 57.375], 1)
+    out = orc.crop_mirror_normalize(img, crop, scale, bias, None, 8, 8, orc.NHWC, orc.FP32)
+    # an fma rounds once: compare with the exactly computed product-sum rounded to fp32
+    exact = img[0].astype(np.float64) * scale.astype(np.float64)[None, None, :] + bias.astype(np.float64)[None, None, :]
+    assert np.array_equal(out[0], exact.astype(np.float32))
+
+
+def test_cmn_mirror_is_involution_and_layouts_are_permutations():
+    img = _img(2, 16, 24)
+    crop = _full(2, 16, 24)
+    m1 = np.array([1, 1], np.uint32)
+    a = orc.crop_mirror_normalize(img, crop, None, None, m1, 16, 24, orc.NHWC, orc.UINT8)
+    b = orc.crop_mirror_normalize(a, crop, None, None, m1, 16, 24, orc.NHWC, orc.UINT8)
+    assert np.array_equal(b, img)
+    c = orc.crop_mirror_normalize(img, crop, None, None, None, 16, 24, orc.NCHW, orc.UINT8)
+    assert np.array_equal(c, img.transpose(0, 3, 1, 2))
+
+
+def test_fixed_crop_window_law():
+    # parameter_rocal_crop.cpp:49-85
+    assert list(orc.fixed_crop(256, 256, 224, 224, anchor=(0.5, 0.5))) == [16, 16, 224, 224]
+    assert list(orc.fixed_crop(299, 299, 224, 224, anchor=(0.5, 0.5))) == [38, 38, 224, 224]  # nearbyint(37.5) = 38 (ties to even)
+    assert list(orc.fixed_crop(300, 300, 224, 224, anchor=(0.5, 0.5))) == [38, 38, 224, 224]
+    assert list(orc.fixed_crop(100, 80, 224, 224, anchor=(0.5, 0.5))) == [0, 0, 100, 80]  # crop larger than ROI -> ROI
+    assert list(orc.fixed_crop(100, 80, 50, 40, x1=120, y1=10)) == [0, 10, 50, 40]  # x1 outside ROI -> 0
+
+
+# ------------------------------------------------------------------ bilinear resize
+
+def _torch_bilinear(img_hw3, dh, dw, antialias=False):
+    import torch
+    import torch.nn.functional as F
+    t = torch.from_numpy(img_hw3.astype(np.float32)).permute(2, 0, 1)[None]
+    r = F.interpolate(t, size=(dh, dw), mode="bilinear", align_corners=False, antialias=antialias)
+    return r[0].permute(1, 2, 0).numpy()
+
+
+def test_bilinear_equals_half_pixel_centre_textbook_form():
+    img = _img(3, 37, 53)
+    roi = np.array([[0, 0, 53, 37], [5, 4, 40, 30], [10, 0, 20, 37]], np.uint32)
+    dw = np.array([80, 23, 20], np.uint32)
+    dh = np.array([19, 44, 37], np.uint32)
+    out = orc.resize(img, roi, dw, dh, 44, 80, interp=orc.LINEAR, dtype=orc.FP32)
+    for i in range(3):
+        x, y, w, h = roi[i]
+        ref = _torch_bilinear(img[i, y:y + h, x:x + w], int(dh[i]), int(dw[i]))
+        assert np.abs(out[i, :dh[i], :dw[i]] - ref).max() < 2e-3
+
+
+def test_bilinear_exact_cases():
+    img = _img(1, 24, 32)
+    roi = _full(1, 24, 32)
+    same = orc.resize(img, roi, [32], [24], 24, 32, interp=orc.LINEAR)
+    assert np.array_equal(same, img)  # scale 1 is the identity
+    half = orc.resize(img, roi, [16], [12], 12, 16, interp=orc.LINEAR, dtype=orc.FP32)
+    box = img[0].astype(np.float32).reshape(12, 2, 16, 2, 3).mean(axis=(1, 3))
+    assert np.array_equal(half[0], box)  # 2x down samples exactly between 4 pixels
+    const = np.full((1, 9, 7, 3), 201, np.uint8)
+    up = orc.resize(const, _full(1, 9, 7), [40], [33], 33, 40, interp=orc.LINEAR)
+    assert (up == 201).all()  # weights sum to one
+    ramp = np.zeros((1, 4, 40, 3), np.uint8)
+    ramp[0, :, :, :] = (np.arange(40) * 5)[None, :, None]
+    r = orc.resize(ramp, _full(1, 4, 40), [100], [4], 4, 100, interp=orc.LINEAR, dtype=orc.FP32)
+    xs = (np.arange(100) + 0.5) * 0.4 - 0.5
+    inner = (xs >= 0) & (xs <= 39)
+    assert np.abs(r[0, 0, inner, 0] - xs[inner] * 5).max() < 1e-3  # linear functions are reproduced
+
+
+def test_bilinear_edge_switch_only_touches_last_row_and_column():
+    img = _img(1, 12, 14)
+    roi = _full(1, 12, 14)
+    a = orc.resize(img, roi, [28], [24], 24, 28, interp=orc.LINEAR)
+    b = orc.resize(img, roi, [28], [24], 24, 28, interp=orc.LINEAR, flags=orc.F_BILINEAR_EDGE_QUIRK)
+    assert np.array_equal(a[0, :20, :24], b[0, :20, :24])
+    assert not np.array_equal(a, b)
+
+
+def test_mirror_reverses_destination_columns():
+    img = _img(2, 20, 30)
+    roi = _full(2, 20, 30)
+    a = orc.resize(img, roi, [17, 17], [11, 11], 11, 17, interp=orc.LINEAR)
+    b = orc.resize(img, roi, [17, 17], [11, 11], 11, 17, interp=orc.LINEAR, mirror=[1, 0])
+    assert np.array_equal(b[0], a[0][:, ::-1]) and np.array_equal(b[1], a[1])
+
+
+def test_quantised_chain_equals_two_nodes():
+    img = _img(2, 50, 60)
+    roi = np.array([[3, 2, 50, 40], [0, 0, 60, 50]], np.uint32)
+    dw = dh = np.array([32, 32], np.uint32)
+    scale, bias = orc.cmn_scale_bias([123.675, 116.28, 103.53], [58.395, 57.12, 57.375], 2)
+    fused = orc.resize(img, roi, dw, dh, 32, 32, interp=orc.LINEAR, mirror=[1, 0], scale=scale, bias=bias, layout=orc.NCHW,
+                       dtype=orc.FP32, flags=orc.F_QUANTIZE_U8)
+    mid = orc.resize(img, roi, dw, dh, 32, 32, interp=orc.LINEAR)
+    two = orc.crop_mirror_normalize(mid, _full(2, 32, 32), scale, bias, [1, 0], 32, 32, orc.NCHW, orc.FP32)
+    assert np.array_equal(fused, two)
+    unq = orc.resize(img, roi, dw, dh, 32, 32, interp=orc.LINEAR, mirror=[1, 0], scale=scale, bias=bias, layout=orc.NCHW, dtype=orc.FP32)
+    assert np.abs(unq - fused).max() <= 0.5 / 57.0 + 1e-6  # at most half a grey level before normalisation
+
+
+def test_resize_destination_size_policy():
+    # node_resize.cpp:98-138 (0 default, 1 stretch, 2 not_smaller, 3 not_larger)
+    assert orc.resize_out_size(640, 480, 0, 240, mode=0) == (320, 240)
+    assert orc.resize_out_size(640, 480, 320, 0, mode=0) == (320, 240)
+    assert orc.resize_out_size(640, 480, 300, 0, mode=1) == (300, 480)
+    assert orc.resize_out_size(640, 480, 256, 256, mode=2) == (341, 256)
+    assert orc.resize_out_size(640, 480, 256, 256, mode=3) == (256, 192)
+    assert orc.resize_out_size(640, 480, 256, 256, mode=2, max_w=300, max_h=0) == (300, 225)
+    assert orc.resize_out_size(333, 500, 256, 0, mode=3) == (256, 384)
+
+
+# ------------------------------------------------------------------ triangular resize
+
+def test_triangular_partition_of_unity_and_separability():
+    const = np.full((1, 40, 52, 3), 77, np.uint8)
+    out = orc.resize(const, _full(1, 40, 52), [17], [13], 13, 17, interp=orc.TRIANGULAR)
+    assert (out == 77).all()
+    img = _img(1, 40, 52)
+    a = orc.resize(img, _full(1, 40, 52), [17], [13], 13, 17, interp=orc.TRIANGULAR, dtype=orc.FP32)
+    b = orc.resize(img, _full(1, 40, 52), [17], [13], 13, 17, interp=orc.TRIANGULAR, dtype=orc.FP32, flags=orc.F_TRI_2D)
+    assert np.abs(a - b).max() < 1e-3  # separable evaluation == the reference's 2-D loop up to rounding
+
+
+def test_triangular_interior_matches_antialiased_bilinear():
+    img = _img(1, 90, 120)
+    out = orc.resize(img, _full(1, 90, 120), [40], [30], 30, 40, interp=orc.TRIANGULAR, dtype=orc.FP32)
+    ref = _torch_bilinear(img[0], 30, 40, antialias=True)
+    assert np.abs(out[0, 3:-3, 3:-3] - ref[3:-3, 3:-3]).max() < 5e-3
+    # integer factor 2: the taps are the (1,3,3,1)/8 triangle in each axis
+    out2 = orc.resize(img, _full(1, 90, 120), [60], [45], 45, 60, interp=orc.TRIANGULAR, dtype=orc.FP32)
+    k = np.array([1, 3, 3, 1], np.float64) / 8
+    f = img[0].astype(np.float64)
+    y, x = 10, 12
+    win = f[2 * y - 1:2 * y + 3, 2 * x - 1:2 * x + 3]
+    exp = np.einsum("i,j,ijc->c", k, k, win)
+    assert np.abs(out2[0, y, x] - exp).max() < 1e-3
+
+
+def test_triangular_upscale_degenerates_to_bilinear():
+    img = _img(1, 20, 24)
+    a = orc.resize(img, _full(1, 20, 24), [48], [40], 40, 48, interp=orc.TRIANGULAR, dtype=orc.FP32)
+    b = orc.resize(img, _full(1, 20, 24), [48], [40], 40, 48, interp=orc.LINEAR, dtype=orc.FP32)
+    assert np.abs(a - b).max() < 1e-3
+
+
+# ------------------------------------------------------------------ colour
+
+def test_brightness_contrast_closed_forms():
+    img = _img(2, 9, 11)
+    roi = _full(2, 9, 11)
+    a, b = np.array([1.9, 0.5], np.float32), np.array([20.0, -7.5], np.float32)
+    out = orc.brightness(img, roi, a, b)
+    # one fp32 FMA = the exact product-sum rounded once to fp32, then the u8 store rule
+    exact = img.astype(np.float64) * a.astype(np.float64)[:, None, None, None] + b.astype(np.float64)[:, None, None, None]
+    exp = np.clip(np.rint(exact.astype(np.float32)), 0, 255)
+    assert np.abs(out.astype(np.int32) - exp.astype(np.int32)).max() == 0
+    f, c = np.array([30.0, 0.7], np.float32), np.array([80.0, 128.0], np.float32)
+    out = orc.contrast(img, roi, f, c)
+    exact = (img.astype(np.float64) - c.astype(np.float64)[:, None, None, None]) * f.astype(np.float64)[:, None, None, None] + c.astype(np.float64)[:, None, None, None]
+    exp = np.clip(np.rint(exact.astype(np.float32)), 0, 255)
+    assert np.abs(out.astype(np.int32) - exp.astype(np.int32)).max() == 0
+
+
+def test_color_twist_invariants():
+    img = _img(1, 32, 32)
+    roi = _full(1, 32, 32)
+    ident = orc.color_twist(img, roi, [1.0], [0.0], [0.0], [1.0])
+    assert np.abs(ident.astype(np.int32) - img.astype(np.int32)).max() <= 1
+    a = orc.color_twist(img, roi, [1.1], [3.0], [37.0], [0.8])
+    b = orc.color_twist(img, roi, [1.1], [3.0], [397.0], [0.8])
+    c = orc.color_twist(img, roi, [1.1], [3.0], [-323.0], [0.8])
+    assert np.array_equal(a, b) and np.array_equal(a, c)  # hue is 360-periodic
+    grey = np.repeat(RNG.integers(0, 256, (1, 8, 8, 1), dtype=np.uint8), 3, axis=3)
+    g = orc.color_twist(grey, _full(1, 8, 8), [1.0], [0.0], [123.0], [1.7])
+    assert np.array_equal(g, grey)  # greys are fixed points of hue and saturation
+    s0 = orc.color_twist(img, roi, [1.0], [0.0], [0.0], [0.0])
+    assert np.array_equal(s0[..., 0], img.max(axis=3)) and np.array_equal(s0[..., 1], s0[..., 2])  # sat 0 -> V
+
+
+def test_color_twist_matches_colorsys():
+    img = _img(1, 24, 24)
+    roi = _full(1, 24, 24)
+    out = orc.color_twist(img, roi, [0.9], [5.0], [-18.0], [1.3])
+    worst = 0
+    for y in range(24):
+        for x in range(24):
+            r, g, b = img[0, y, x] / 255.0
+            h, s, v = colorsys.rgb_to_hsv(r, g, b)
+            h = (h - 18.0 / 360.0) % 1.0
+            s = min(max(s * 1.3, 0.0), 1.0)
+            e = np.array(colorsys.hsv_to_rgb(h, s, v)) * 255.0 * 0.9 + 5.0
+            e = np.clip(np.rint(e), 0, 255)
+            worst = max(worst, np.abs(e - out[0, y, x]).max())
+    assert worst <= 1
+
+
+# ------------------------------------------------------------------ warp / rotate
+
+def test_warp_identity_translation_and_out_of_bounds():
+    img = _img(1, 21, 31)
+    roi = _full(1, 21, 31)
+    ident = np.array([[1, 0, 0, 0, 1, 0]], np.float32)
+    out = orc.warp_affine(img, roi, ident, [31], [21], 21, 31)
+    assert np.array_equal(out, img)
+    shift = np.array([[1, 0, 3, 0, 1, -2]], np.float32)  # source = destination + (3,-2)
+    out = orc.warp_affine(img, roi, shift, [31], [21], 21, 31)
+    assert np.array_equal(out[0, 2:, :28], img[0, :19, 3:])
+    assert not out[0, :2].any() and not out[0, :, 28:].any()  # outside the ROI -> 0
+
+
+def test_rocal_affine_order_and_rotation_direction():
+    # rocAL fills x0,y0,x1,y1,o0,o1 (node_warp_affine.cpp:43-48)
+    assert list(orc.affine_from_rocal([1, 2, 3, 4, 5, 6])) == [1, 3, 5, 2, 4, 6]
+    # meta_node_rotate.cpp:53-77: forward map about the centres is [[c, s], [-s, c]]
+    n = 41
+    img = np.zeros((1, n, n, 3), np.uint8)
+    cx = cy = n // 2
+    img[0, cy, cx + 10] = 255
+    m = orc.rotate_matrix(90.0)[None]
+    out = orc.warp_affine(img, _full(1, n, n), m, [n], [n], n, n)
+    yy, xx = np.unravel_index(out[0, :, :, 0].argmax(), (n, n))
+    assert (xx, yy) == (cx, cy - 10)
+    assert np.array_equal(out[0], np.rot90(img[0], 1))  # odd size: exact quarter turn
+    r30 = orc.rotate_matrix(30.0)
+    assert np.allclose(r30, [math.cos(math.pi / 6), -0.5, 0, 0.5, math.cos(math.pi / 6), 0], atol=1e-6)
+
+
+# ------------------------------------------------------------------ to_tensor
+
+def test_to_tensor_closed_form():
+    img = _img(2, 6, 8)
+    mul, add = np.array([0.5, 0.25, 2.0], np.float32), np.array([1.0, -3.0, 0.5], np.float32)
+    out = orc.to_tensor(img, mul, add, reverse_channels=True, layout=orc.NCHW, dtype=orc.FP32)
+    exp = img[..., ::-1].astype(np.float32) * mul + add  # exact in fp32 for these constants
+    assert np.array_equal(out, exp.transpose(0, 3, 1, 2))
+
+
+# ------------------------------------------------------------------ parameter laws
+
+def test_mt19937_and_seed_seq_known_answers():
+    g = orc.MT19937(5489)
+    for _ in range(9999):
+        g.next()
+    assert g.next() == 4123659995  # C++ [rand.predef]: 10000th value of a default-constructed mt19937
+    # numpy's MT19937 seeds with the same init_genrand recurrence
+    rs = np.random.RandomState(1234)
+    g = orc.MT19937(1234)
+    assert [g.next() for _ in range(50)] == [int(x) for x in rs.randint(0, 2 ** 32, 50, dtype=np.uint64)]
+
+
+def test_uniform_rand_law():
+    # parameter_random.h:59-71: draws even when start == end; int result truncates
+    g, h = orc.MT19937(7), orc.MT19937(7)
+    raw = [h.next() for _ in range(6)]
+    assert g.uniform_f32(2.0, 2.0) == 2.0
+    v = g.uniform_f32(-1.0, 3.0)
+    assert v == np.float32(raw[1] / 4294967295.0 * 4.0 - 1.0)
+    assert g.uniform_i32(0, 1) == int(raw[2] / 4294967295.0)  # ~always 0: why rocAL coin flips use CustomRand
+    assert g.uniform_i32(5, 5) == 5 and g.next() == raw[4]
+    # CustomRand (parameter_random.h:176-193): upper_bound on the cumulative distribution
+    g = orc.MT19937(9)
+    h = orc.MT19937(9)
+    for _ in range(200):
+        r = h.next() / 4294967295.0
+        assert g.custom_index([0.5, 0.5]) == (0 if r < 0.5 else 1 if r < 1.0 else 2)
