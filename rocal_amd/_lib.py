@@ -74,6 +74,12 @@ def lib():
     if _lib is None:
         if not os.path.exists(LIB_PATH):
             raise RmxError(-1, "HIP library not built: %s is missing (run `python -m rocal_amd.build`)" % LIB_PATH)
+        # PyTorch bundles its own HIP runtime; load it first so that this library binds to the same
+        # runtime instance (two instances in one process do not see each other's devices/streams).
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         l = C.CDLL(LIB_PATH)
         for name, args in _SIGS.items():
             fn = getattr(l, name)
