@@ -18,7 +18,13 @@
  *   orc_crop_mirror_normalize  pinned: closed form (integer gather + one fp32 FMA), brute force.
  *   orc_resize (bilinear)      pinned: in-tree kernel rocAL/rocAL_hip/rocal_hip_kernels.cpp:311-485
  *                              (compiled as oracle/_ref and compared on the GPU with
- *                              ORC_F_BILINEAR_EDGE_QUIRK), torch F.interpolate closed forms.
+ *                              ORC_F_BILINEAR_EDGE_QUIRK; that source builds `(float4)scalar` as
+ *                              (scalar,0,0,0) under this toolchain's HIP headers, so the comparison
+ *                              holds on lane 0 of each 8-pixel group at vertical ratio 1: x law,
+ *                              weights, fmaf chain, edge clamp and the rounding store, bit-exact),
+ *                              torch F.interpolate closed forms, box-mean and ramp special cases
+ *                              for both axes. Which edge clamp RPP's HOST path uses (hi or hi-1)
+ *                              is parity unpinned; the default is the textbook clamp to hi.
  *   orc_resize (triangular)    pinned: in-tree kernel rocal_hip_kernels.cpp:487-589 (oracle/_ref,
  *                              ORC_F_ROUND_TRUNC), partition of unity, box-mean special cases.
  *   orc_to_tensor              pinned: rocal_hip_kernels.cpp:131-217 (oracle/_ref), closed form.
