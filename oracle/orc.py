@@ -219,6 +219,50 @@ def fixed_crop(roi_w, roi_h, crop_w, crop_h, anchor=None, x1=0, y1=0):
     return out
 
 
+class _FParam(C.Structure):
+    _fields_ = [("g", _MT), ("lo", C.c_float), ("hi", C.c_float), ("simple", C.c_int), ("value", C.c_float)]
+
+
+class FParam:
+    """A float parameter as the crop laws see it: FParam.uniform(lo, hi, seed) is a UniformRand<float>
+    (its constructor draws once), FParam.simple(v) a SimpleParameter<float>."""
+
+    def __init__(self):
+        self.p = _FParam()
+
+    @classmethod
+    def uniform(cls, lo, hi, seed):
+        o = cls()
+        lib().orc_fparam_uniform(C.byref(o.p), C.c_float(lo), C.c_float(hi), C.c_uint32(seed & 0xFFFFFFFF))
+        return o
+
+    @classmethod
+    def simple(cls, v):
+        o = cls()
+        lib().orc_fparam_simple(C.byref(o.p), C.c_float(v))
+        return o
+
+    def renew(self):
+        lib().orc_fparam_renew.restype = C.c_float
+        return float(lib().orc_fparam_renew(C.byref(self.p)))
+
+    @property
+    def value(self):
+        return float(self.p.value)
+
+
+def random_crop(area, aspect, x_drift, y_drift, roi_w, roi_h):
+    out = np.empty(4, np.uint32)
+    lib().orc_random_crop(C.byref(area.p), C.byref(aspect.p), C.byref(x_drift.p), C.byref(y_drift.p), C.c_uint32(roi_w), C.c_uint32(roi_h), _p(out))
+    return out
+
+
+def factor_crop(h_factor, w_factor, x_drift, y_drift, roi_w, roi_h):
+    out = np.empty(4, np.uint32)
+    lib().orc_factor_crop(C.byref(h_factor.p), C.byref(w_factor.p), C.byref(x_drift.p), C.byref(y_drift.p), C.c_uint32(roi_w), C.c_uint32(roi_h), _p(out))
+    return out
+
+
 def resize_out_size(sw, sh, dw, dh, mode=0, max_w=0, max_h=0):
     ow, oh = C.c_uint(0), C.c_uint(0)
     lib().orc_resize_out_size(sw, sh, dw, dh, mode, max_w, max_h, C.byref(ow), C.byref(oh))

@@ -663,6 +663,78 @@ void orc_fixed_crop(uint32_t roi_w, uint32_t roi_h, uint32_t crop_w, uint32_t cr
     (void)x2; (void)y2; /* the reference clamps x2/y2 but publishes x1,y1,cw,ch */
 }
 
+void orc_fparam_uniform(orc_fparam *p, float lo, float hi, uint32_t seed) {
+    orc_mt19937_seed(&p->g, seed);
+    p->lo = lo;
+    p->hi = hi < lo ? lo : hi;
+    p->simple = 0;
+    p->value = orc_uniform_rand_f32(&p->g, p->lo, p->hi);
+}
+
+void orc_fparam_simple(orc_fparam *p, float value) {
+    p->simple = 1;
+    p->value = value;
+}
+
+float orc_fparam_renew(orc_fparam *p) {
+    if (!p->simple) p->value = orc_uniform_rand_f32(&p->g, p->lo, p->hi);
+    return p->value;
+}
+
+void orc_random_crop(orc_fparam *area, orc_fparam *aspect, orc_fparam *x_drift, orc_fparam *y_drift, uint32_t W,
+                     uint32_t H, uint32_t out[4]) {
+    const float ar_lo = 0.75f, ar_hi = 1.333f; /* parameter_random_crop.h:43 */
+    uint32_t cw = 0, ch = 0, x = 0, y = 0;
+    int ok = 0;
+    for (int attempt = 0; attempt < 5 && !ok; attempt++) { /* :50 */
+        float a = orc_fparam_renew(area);
+        float r = orc_fparam_renew(aspect);
+        float t32 = a * (float)H; /* float arithmetic, left to right, widened to double on assignment (:64) */
+        t32 = t32 * (float)W;
+        double target = (double)t32;
+        cw = (uint32_t)(size_t)sqrt(target * (double)r);
+        ch = (uint32_t)(size_t)sqrt(target * (double)(1 / r));
+        if (ch < H && cw < W) { /* strictly smaller (:55-57) */
+            float xd = orc_fparam_renew(x_drift);
+            orc_fparam_renew(y_drift);
+            float yd = orc_fparam_renew(y_drift); /* renewed twice (:70-72) */
+            x = (uint32_t)(size_t)(xd * (float)(W - cw));
+            y = (uint32_t)(size_t)(yd * (float)(H - ch));
+            ok = 1;
+        }
+    }
+    if (!ok) { /* central crop, aspect ratio pulled into range (:81-94) */
+        float in_ratio = (float)W / (float)H;
+        if (in_ratio < ar_lo) {
+            cw = W;
+            ch = (uint32_t)((float)cw / ar_lo);
+        } else if (in_ratio > ar_hi) {
+            ch = H;
+            cw = (uint32_t)((float)ch * ar_hi);
+        } else {
+            ch = H;
+            cw = W;
+        }
+        x = (W - cw) / 2;
+        y = (H - ch) / 2;
+    }
+    out[0] = x; out[1] = y; out[2] = cw; out[3] = ch;
+}
+
+void orc_factor_crop(orc_fparam *h_factor, orc_fparam *w_factor, orc_fparam *x_drift, orc_fparam *y_drift, uint32_t W,
+                     uint32_t H, uint32_t out[4]) {
+    float fh = orc_fparam_renew(h_factor);
+    float fw = orc_fparam_renew(w_factor);
+    uint32_t cw = (uint32_t)(size_t)(fw * (float)W);
+    uint32_t ch = (uint32_t)(size_t)(fh * (float)H);
+    float xd = orc_fparam_renew(x_drift);
+    float yd = orc_fparam_renew(y_drift);
+    out[0] = (uint32_t)(size_t)(xd * (float)(W - cw));
+    out[1] = (uint32_t)(size_t)(yd * (float)(H - ch));
+    out[2] = cw;
+    out[3] = ch;
+}
+
 void orc_resize_out_size(unsigned sw, unsigned sh, unsigned dw, unsigned dh, int mode, unsigned max_w,
                          unsigned max_h, unsigned *out_w, unsigned *out_h) {
     int has_max = (max_w | max_h) > 0;

@@ -37,7 +37,7 @@
  *   orc_rotate                 direction/centre pinned by rocAL/source/meta_data/meta_node_rotate.cpp:53-77;
  *                              fp path from angle to matrix PARITY UNPINNED.
  *   parameter laws (orc_mt19937*, orc_seed_seq, orc_uniform_rand*, orc_custom_rand,
- *   orc_fixed_crop, orc_random_crop, orc_random_crop_dec)
+ *   orc_fixed_crop, orc_random_crop, orc_factor_crop)
  *                              pinned: C++ standard known answers (10000th mt19937 output),
  *                              libstdc++ cross-check in tests.
  */
@@ -140,6 +140,19 @@ int orc_custom_rand_index(orc_mt19937 *g, const double *freq, int size);
 void orc_fixed_crop(uint32_t roi_w, uint32_t roi_h, uint32_t crop_w, uint32_t crop_h,
                     int is_fixed_anchor, float anchor_x, float anchor_y, uint32_t x1, uint32_t y1,
                     uint32_t out_xywh[4]);
+/* A float parameter as the crop laws see it: either a UniformRand<float> (own generator, one draw per
+ * renew) or a SimpleParameter<float> (renew draws nothing). */
+typedef struct { orc_mt19937 g; float lo, hi; int simple; float value; } orc_fparam;
+void orc_fparam_uniform(orc_fparam *p, float lo, float hi, uint32_t seed); /* constructor draws once (parameter_random.h:40-43) */
+void orc_fparam_simple(orc_fparam *p, float value);
+float orc_fparam_renew(orc_fparam *p);
+/* RocalRandomCropParam::fill_crop_dims for one sample (parameter_random_crop.cpp:44-100); out = x1,y1,w,h.
+ * prev_wh = this sample's w,h from the previous batch (what the arrays still hold). */
+void orc_random_crop(orc_fparam *area, orc_fparam *aspect, orc_fparam *x_drift, orc_fparam *y_drift,
+                     uint32_t roi_w, uint32_t roi_h, uint32_t out_xywh[4]);
+/* RocalCropParam::fill_crop_dims, random-factor branch (parameter_rocal_crop.cpp:66-78) */
+void orc_factor_crop(orc_fparam *h_factor, orc_fparam *w_factor, orc_fparam *x_drift, orc_fparam *y_drift,
+                     uint32_t roi_w, uint32_t roi_h, uint32_t out_xywh[4]);
 /* ResizeNode::adjust_out_roi_size (node_resize.cpp:98-138). mode: 0 default,1 stretch,2 not_smaller,3 not_larger */
 void orc_resize_out_size(unsigned src_w, unsigned src_h, unsigned dst_w, unsigned dst_h, int mode,
                          unsigned max_w, unsigned max_h, unsigned *out_w, unsigned *out_h);

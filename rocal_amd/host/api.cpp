@@ -1,0 +1,438 @@
+// rocAL C API entry points of the hot-path operators (rocAL/source/api/rocal_api.cpp:82-107,
+// rocal_api_parameter.cpp, rocal_api_augmentation.cpp). Each one derives the output TensorInfo from the
+// input's exactly as the reference does, adds the node and calls its init(); exceptions are caught here,
+// stored in the context, printed, and turned into a null tensor / ROCAL_RUNTIME_ERROR.
+#include "rocal_host.h"
+
+#include <iostream>
+
+namespace {
+
+void report(Context *context, const std::exception &e) {
+    context->capture_error(e.what());
+    std::cerr << e.what() << std::endl;
+}
+
+enum class Dims { KEEP, SET };
+
+// Common frame of every augmentation entry point.
+template <typename NodeT, typename InitFn>
+Tensor *add_op(RocalContext p_context, RocalTensor p_input, bool is_output, RocalTensorLayout output_layout, RocalTensorOutputType output_datatype,
+               Dims dims, unsigned width, unsigned height, const char *precondition_error, InitFn init) {
+    Tensor *output = nullptr;
+    if (!p_context) {
+        std::cerr << "Invalid rocal context passed" << std::endl;
+        return output;
+    }
+    auto *context = static_cast<Context *>(p_context);
+    if (!p_input) {
+        context->capture_error("Invalid rocal tensor passed");
+        std::cerr << "Invalid rocal tensor passed" << std::endl;
+        return output;
+    }
+    auto *input = static_cast<Tensor *>(p_input);
+    try {
+        if (precondition_error) THROW(precondition_error)
+        if (context->master_graph->built()) THROW("the graph is already verified; nodes cannot be added")
+        TensorInfo output_info = input->info();
+        const auto layout = static_cast<RocalTensorlayout>(output_layout);
+        output_info.set_data_type(static_cast<RocalTensorDataType>(output_datatype));
+        if (dims == Dims::SET)
+            output_info.modify_dims_width_and_height(layout, width, height);
+        else
+            output_info.set_tensor_layout(layout);
+        output = context->master_graph->create_tensor(output_info, is_output);
+        auto node = context->master_graph->add_node<NodeT>({input}, {output});
+        init(*node);
+    } catch (const std::exception &e) {
+        report(context, e);
+        output = nullptr;
+    }
+    return output;
+}
+
+FloatParam *F(RocalFloatParam p) { return static_cast<FloatParam *>(p); }
+IntParam *I(RocalIntParam p) { return static_cast<IntParam *>(p); }
+
+}  // namespace
+
+/* ------------------------------------------------------------------ context */
+
+RocalContext rocalCreate(size_t batch_size, RocalProcessMode affinity, int gpu_id, size_t, size_t, RocalTensorOutputType) {
+    try {
+        if (batch_size == 0) THROW("batch size must be positive")
+        if (affinity != ROCAL_PROCESS_GPU) THROW("only ROCAL_PROCESS_GPU is available: this build has no CPU path")
+        return new Context(batch_size, gpu_id, nullptr);
+    } catch (const std::exception &e) {
+        std::cerr << e.what() << std::endl;
+        return nullptr;
+    }
+}
+
+RocalStatus rocalVerify(RocalContext p_context) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->build();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+RocalStatus rocalRun(RocalContext p_context) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->run();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+RocalStatus rocalRelease(RocalContext p_context) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    delete static_cast<Context *>(p_context);
+    return ROCAL_OK;
+}
+
+const char *rocalGetErrorMessage(RocalContext p_context) { return p_context ? static_cast<Context *>(p_context)->error.c_str() : "Invalid rocal context passed"; }
+
+/* ------------------------------------------------------------------ decoded batches in device memory */
+
+RocalTensor rocalDeviceSource(RocalContext p_context, unsigned max_width, unsigned max_height, bool is_output) {
+    if (!p_context) return nullptr;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        if (max_width == 0 || max_height == 0) THROW("source needs non-zero maximum dimensions")
+        TensorInfo info({context->master_graph->batch_size(), max_height, max_width, 3}, RocalTensorlayout::NHWC, RocalTensorDataType::UINT8);
+        return context->master_graph->create_tensor(info, is_output);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return nullptr;
+    }
+}
+
+RocalStatus rocalDeviceSourceFeed(RocalContext p_context, RocalTensor p_source, const void *device_ptr, const unsigned *roi_width, const unsigned *roi_height) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        if (!p_source || !device_ptr || !roi_width || !roi_height) THROW("null argument")
+        auto *t = static_cast<Tensor *>(p_source);
+        const size_t n = t->info().batch_size();
+        t->swap_handle(const_cast<void *>(device_ptr));
+        t->update_tensor_roi(std::vector<uint32_t>(roi_width, roi_width + n), std::vector<uint32_t>(roi_height, roi_height + n));
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+void *rocalTensorBuffer(RocalTensor t) { return t ? static_cast<Tensor *>(t)->buffer() : nullptr; }
+const unsigned *rocalTensorRoi(RocalTensor t) { return t ? reinterpret_cast<const unsigned *>(static_cast<Tensor *>(t)->info().roi()) : nullptr; }
+size_t rocalTensorDataSize(RocalTensor t) { return t ? static_cast<Tensor *>(t)->info().data_size() : 0; }
+
+/* ------------------------------------------------------------------ parameters */
+
+void rocalSetSeed(unsigned seed) { ParameterFactory::instance()->set_seed(seed); }
+unsigned rocalGetSeed() { return ParameterFactory::instance()->get_seed(); }
+int rocalGetIntValue(RocalIntParam p) { return I(p)->core->get(); }
+float rocalGetFloatValue(RocalFloatParam p) { return F(p)->core->get(); }
+RocalIntParam rocalCreateIntUniformRand(int start, int end) { return ParameterFactory::instance()->create_uniform_int_rand_param(start, end); }
+RocalFloatParam rocalCreateFloatUniformRand(float start, float end) { return ParameterFactory::instance()->create_uniform_float_rand_param(start, end); }
+RocalFloatParam rocalCreateFloatParameter(float val) { return ParameterFactory::instance()->create_single_value_float_param(val); }
+RocalIntParam rocalCreateIntParameter(int val) { return ParameterFactory::instance()->create_single_value_int_param(val); }
+RocalIntParam rocalCreateIntRand(const int *values, const double *frequencies, unsigned size) {
+    return ParameterFactory::instance()->create_custom_int_rand_param(values, frequencies, size);
+}
+RocalFloatParam rocalCreateFloatRand(const float *values, const double *frequencies, unsigned size) {
+    return ParameterFactory::instance()->create_custom_float_rand_param(values, frequencies, size);
+}
+
+namespace {
+template <typename Derived, typename Wrapper, typename Fn>
+RocalStatus update_param(Wrapper *w, RocalParameterType expected, Fn fn) {
+    if (!w || w->type != expected) return ROCAL_INVALID_PARAMETER_TYPE;
+    auto *obj = dynamic_cast<Derived *>(w->core);
+    if (!obj) return ROCAL_INVALID_PARAMETER_TYPE;
+    return fn(obj) == 0 ? ROCAL_OK : ROCAL_UPDATE_PARAMETER_FAILED;
+}
+}  // namespace
+
+RocalStatus rocalUpdateIntUniformRand(int start, int end, RocalIntParam p) {
+    return update_param<UniformRand<int>>(I(p), RocalParameterType::RANDOM_UNIFORM, [&](auto *o) { return o->update(start, end); });
+}
+RocalStatus rocalUpdateFloatUniformRand(float start, float end, RocalFloatParam p) {
+    return update_param<UniformRand<float>>(F(p), RocalParameterType::RANDOM_UNIFORM, [&](auto *o) { return o->update(start, end); });
+}
+RocalStatus rocalUpdateFloatParameter(float v, RocalFloatParam p) {
+    return update_param<SimpleParameter<float>>(F(p), RocalParameterType::DETERMINISTIC, [&](auto *o) { return o->update(v); });
+}
+RocalStatus rocalUpdateIntParameter(int v, RocalIntParam p) {
+    return update_param<SimpleParameter<int>>(I(p), RocalParameterType::DETERMINISTIC, [&](auto *o) { return o->update(v); });
+}
+RocalStatus rocalUpdateIntRand(const int *values, const double *frequencies, unsigned size, RocalIntParam p) {
+    return update_param<CustomRand<int>>(I(p), RocalParameterType::RANDOM_CUSTOM, [&](auto *o) { return o->update(values, frequencies, size); });
+}
+RocalStatus rocalUpdateFloatRand(const float *values, const double *frequencies, unsigned size, RocalFloatParam p) {
+    return update_param<CustomRand<float>>(F(p), RocalParameterType::RANDOM_CUSTOM, [&](auto *o) { return o->update(values, frequencies, size); });
+}
+
+/* ------------------------------------------------------------------ resize family */
+
+namespace {
+
+// rocal_api_augmentation.cpp:449-505: which size the node is given and how large the padded output is.
+constexpr float MAX_ASPECT_RATIO = 6.0f;  // rocAL/include/pipeline/commons.h:39
+
+struct ResizePlan {
+    unsigned out_w, out_h, max_w, max_h;
+    RocalResizeScalingMode mode;
+    std::vector<unsigned> maximum_size;
+    const char *error = nullptr;
+};
+
+ResizePlan plan_resize(Tensor *input, unsigned dest_width, unsigned dest_height, RocalResizeScalingMode scaling_mode, const std::vector<unsigned> &max_size,
+                       unsigned resize_shorter, unsigned resize_longer) {
+    ResizePlan p{};
+    if ((dest_width | dest_height | resize_longer | resize_shorter) == 0) {
+        p.error = "Atleast one size 'dest_width' or 'dest_height' or 'resize_shorter' or 'resize_longer' must be specified";
+        return p;
+    }
+    if ((dest_width | dest_height) && (resize_longer | resize_shorter)) {
+        p.error = "Only one method of specifying size can be used \ndest_width and/or dest_height\nresize_shorter\nresize_longer";
+        return p;
+    }
+    if (resize_longer && resize_shorter) {
+        p.error = "'resize_longer' and 'resize_shorter' cannot be passed together. They are mutually exclusive.";
+        return p;
+    }
+    if (resize_shorter) {
+        p.mode = ROCAL_SCALING_MODE_NOT_SMALLER;
+        p.out_w = p.out_h = resize_shorter;
+    } else if (resize_longer) {
+        p.mode = ROCAL_SCALING_MODE_NOT_LARGER;
+        p.out_w = p.out_h = resize_longer;
+    } else {
+        p.mode = scaling_mode;
+        p.out_w = dest_width;
+        p.out_h = dest_height;
+    }
+    if (max_size.size() == 1)
+        p.maximum_size = {max_size[0], max_size[0]};
+    else if (max_size.size() == 2)
+        p.maximum_size = {max_size[0], max_size[1]};
+    else if (max_size.size() > 2) {
+        p.error = "The length of max_size vector exceeds the image dimension.";
+        return p;
+    }
+    if (p.maximum_size.size() && p.maximum_size[0] != 0 && p.maximum_size[1] != 0) {
+        p.max_w = p.maximum_size[0];
+        p.max_h = p.maximum_size[1];
+    } else {
+        if (p.mode == ROCAL_SCALING_MODE_STRETCH) {
+            p.max_w = p.out_w ? p.out_w : (unsigned)input->info().max_shape()[0];
+            p.max_h = p.out_h ? p.out_h : (unsigned)input->info().max_shape()[1];
+        } else if (p.mode == ROCAL_SCALING_MODE_NOT_SMALLER) {
+            p.max_w = (p.out_w ? p.out_w : p.out_h) * MAX_ASPECT_RATIO;
+            p.max_h = (p.out_h ? p.out_h : p.out_w) * MAX_ASPECT_RATIO;
+        } else {
+            p.max_w = p.out_w ? p.out_w : p.out_h * MAX_ASPECT_RATIO;
+            p.max_h = p.out_h ? p.out_h : p.out_w * MAX_ASPECT_RATIO;
+        }
+        if (p.maximum_size.size() == 2) {
+            p.max_w = p.maximum_size[0] ? p.maximum_size[0] : p.max_w;
+            p.max_h = p.maximum_size[1] ? p.maximum_size[1] : p.max_h;
+        }
+    }
+    return p;
+}
+
+}  // namespace
+
+RocalTensor rocalResize(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, RocalResizeScalingMode scaling_mode,
+                        std::vector<unsigned> max_size, unsigned resize_shorter, unsigned resize_longer, RocalResizeInterpolationType interpolation_type,
+                        RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    if (!c || !in) return add_op<ResizeNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [](ResizeNode &) {});
+    ResizePlan p = plan_resize(static_cast<Tensor *>(in), dest_width, dest_height, scaling_mode, max_size, resize_shorter, resize_longer);
+    return add_op<ResizeNode>(c, in, is_output, layout, dtype, Dims::SET, p.max_w, p.max_h, p.error,
+                              [&](ResizeNode &n) { n.init(p.out_w, p.out_h, p.mode, p.maximum_size, interpolation_type); });
+}
+
+RocalTensor rocalResizeMirrorNormalize(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, std::vector<float> &mean,
+                                       std::vector<float> &std_dev, bool is_output, RocalResizeScalingMode scaling_mode, std::vector<unsigned> max_size,
+                                       unsigned resize_shorter, unsigned resize_longer, RocalResizeInterpolationType interpolation_type, RocalIntParam mirror,
+                                       RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    if (!c || !in) return add_op<ResizeMirrorNormalizeNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [](ResizeMirrorNormalizeNode &) {});
+    ResizePlan p = plan_resize(static_cast<Tensor *>(in), dest_width, dest_height, scaling_mode, max_size, resize_shorter, resize_longer);
+    return add_op<ResizeMirrorNormalizeNode>(c, in, is_output, layout, dtype, Dims::SET, p.max_w, p.max_h, p.error, [&](ResizeMirrorNormalizeNode &n) {
+        n.init(p.out_w, p.out_h, p.mode, p.maximum_size, interpolation_type, mean, std_dev, I(mirror));
+    });
+}
+
+RocalTensor rocalCropResize(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, RocalFloatParam area,
+                            RocalFloatParam aspect_ratio, RocalFloatParam x_center_drift, RocalFloatParam y_center_drift, RocalTensorLayout layout,
+                            RocalTensorOutputType dtype) {
+    const char *err = (dest_width == 0 || dest_height == 0) ? "CropResize node needs tp receive non-zero destination dimensions" : nullptr;
+    return add_op<CropResizeNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, err,
+                                  [&](CropResizeNode &n) { n.init(F(area), F(aspect_ratio), F(x_center_drift), F(y_center_drift)); });
+}
+
+RocalTensor rocalCropResizeFixed(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, float area, float aspect_ratio,
+                                 float x_center_drift, float y_center_drift, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    const char *err = (dest_width == 0 || dest_height == 0) ? "CropResize node needs tp receive non-zero destination dimensions" : nullptr;
+    return add_op<CropResizeNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, err,
+                                  [&](CropResizeNode &n) { n.init(area, aspect_ratio, x_center_drift, y_center_drift); });
+}
+
+RocalTensor rocalROIResize(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, unsigned roi_h, unsigned roi_w,
+                           float roi_pos_x, float roi_pos_y, RocalResizeInterpolationType interpolation_type, RocalTensorLayout layout,
+                           RocalTensorOutputType dtype) {
+    const char *err = (dest_width == 0 || dest_height == 0) ? "ROI Resize needs to receive non-zero destination dimensions" : nullptr;
+    return add_op<CropResizeNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, err,
+                                  [&](CropResizeNode &n) { n.init(roi_h, roi_w, roi_pos_x, roi_pos_y, interpolation_type); });
+}
+
+RocalTensor rocalResizeCropMirrorFixed(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, unsigned crop_h,
+                                       unsigned crop_w, RocalIntParam mirror, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    const char *err = (dest_width == 0 || dest_height == 0) ? "Crop Mirror node needs tp receive non-zero destination dimensions" : nullptr;
+    return add_op<ResizeCropMirrorNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, err,
+                                        [&](ResizeCropMirrorNode &n) { n.init(crop_h, crop_w, I(mirror), ROCAL_LINEAR_INTERPOLATION); });
+}
+
+RocalTensor rocalResizeCropMirror(RocalContext c, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, RocalFloatParam crop_height,
+                                  RocalFloatParam crop_width, RocalIntParam mirror, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    const char *err = (dest_width == 0 || dest_height == 0) ? "Crop Mirror node needs tp receive non-zero destination dimensions" : nullptr;
+    return add_op<ResizeCropMirrorNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, err, [&](ResizeCropMirrorNode &n) {
+        n.init(F(crop_height), F(crop_width), I(mirror), ROCAL_LINEAR_INTERPOLATION);
+    });
+}
+
+/* ------------------------------------------------------------------ crop / flip / CMN */
+
+RocalTensor rocalCropMirrorNormalize(RocalContext c, RocalTensor in, unsigned crop_height, unsigned crop_width, float start_x, float start_y,
+                                     std::vector<float> &mean, std::vector<float> &std_dev, bool is_output, RocalIntParam mirror, RocalTensorLayout layout,
+                                     RocalTensorOutputType dtype) {
+    const char *err = (crop_width == 0 || crop_height == 0) ? "Null values passed as input" : nullptr;
+    return add_op<CropMirrorNormalizeNode>(c, in, is_output, layout, dtype, Dims::SET, crop_width, crop_height, err, [&](CropMirrorNormalizeNode &n) {
+        n.init(crop_height, crop_width, start_x, start_y, mean, std_dev, I(mirror));
+    });
+}
+
+RocalTensor rocalCrop(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam crop_width, RocalFloatParam crop_height, RocalFloatParam,
+                      RocalFloatParam crop_pos_x, RocalFloatParam crop_pos_y, RocalFloatParam, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<CropNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr,
+                            [&](CropNode &n) { n.init(F(crop_height), F(crop_width), F(crop_pos_x), F(crop_pos_y)); });
+}
+
+RocalTensor rocalCropFixed(RocalContext c, RocalTensor in, unsigned crop_width, unsigned crop_height, unsigned, bool is_output, float crop_pos_x,
+                           float crop_pos_y, float, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    const char *err = (crop_width == 0 || crop_height == 0) ? "Crop node needs to receive non-zero destination dimensions" : nullptr;
+    return add_op<CropNode>(c, in, is_output, layout, dtype, Dims::SET, crop_width, crop_height, err,
+                            [&](CropNode &n) { n.init(crop_height, crop_width, crop_pos_x, crop_pos_y); });
+}
+
+RocalTensor rocalCropCenterFixed(RocalContext c, RocalTensor in, unsigned crop_width, unsigned crop_height, unsigned, bool is_output,
+                                 RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    const char *err = (crop_width == 0 || crop_height == 0) ? "Crop node needs to receive non-zero destination dimensions" : nullptr;
+    return add_op<CropNode>(c, in, is_output, layout, dtype, Dims::SET, crop_width, crop_height, err, [&](CropNode &n) { n.init(crop_height, crop_width); });
+}
+
+RocalTensor rocalRandomCrop(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam crop_area_factor, RocalFloatParam crop_aspect_ratio,
+                            RocalFloatParam crop_pos_x, RocalFloatParam crop_pos_y, int num_of_attempts, RocalTensorLayout layout,
+                            RocalTensorOutputType dtype) {
+    return add_op<RandomCropNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](RandomCropNode &n) {
+        n.init(F(crop_area_factor), F(crop_aspect_ratio), F(crop_pos_x), F(crop_pos_y), num_of_attempts);
+    });
+}
+
+RocalTensor rocalFlip(RocalContext c, RocalTensor in, bool is_output, RocalIntParam h, RocalIntParam v, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<FlipNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](FlipNode &n) { n.init(I(h), I(v)); });
+}
+
+RocalTensor rocalFlipFixed(RocalContext c, RocalTensor in, int h, int v, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<FlipNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](FlipNode &n) { n.init(h, v); });
+}
+
+/* ------------------------------------------------------------------ colour family */
+
+RocalTensor rocalBrightness(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam alpha, RocalFloatParam beta, RocalTensorLayout layout,
+                            RocalTensorOutputType dtype) {
+    return add_op<BrightnessNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](BrightnessNode &n) { n.init(F(alpha), F(beta)); });
+}
+RocalTensor rocalBrightnessFixed(RocalContext c, RocalTensor in, float alpha, float beta, bool is_output, RocalTensorLayout layout,
+                                 RocalTensorOutputType dtype) {
+    return add_op<BrightnessNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](BrightnessNode &n) { n.init(alpha, beta); });
+}
+RocalTensor rocalContrast(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam factor, RocalFloatParam center, RocalTensorLayout layout,
+                          RocalTensorOutputType dtype) {
+    return add_op<ContrastNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](ContrastNode &n) { n.init(F(factor), F(center)); });
+}
+RocalTensor rocalContrastFixed(RocalContext c, RocalTensor in, float factor, float center, bool is_output, RocalTensorLayout layout,
+                               RocalTensorOutputType dtype) {
+    return add_op<ContrastNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](ContrastNode &n) { n.init(factor, center); });
+}
+RocalTensor rocalHue(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam hue, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<HueNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](HueNode &n) { n.init(F(hue)); });
+}
+RocalTensor rocalHueFixed(RocalContext c, RocalTensor in, float hue, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<HueNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](HueNode &n) { n.init(hue); });
+}
+RocalTensor rocalSaturation(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam sat, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<SaturationNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](SaturationNode &n) { n.init(F(sat)); });
+}
+RocalTensor rocalSaturationFixed(RocalContext c, RocalTensor in, float sat, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<SaturationNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](SaturationNode &n) { n.init(sat); });
+}
+RocalTensor rocalColorTwist(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam alpha, RocalFloatParam beta, RocalFloatParam hue,
+                            RocalFloatParam sat, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<ColorTwistNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr,
+                                  [&](ColorTwistNode &n) { n.init(F(alpha), F(beta), F(hue), F(sat)); });
+}
+RocalTensor rocalColorTwistFixed(RocalContext c, RocalTensor in, float alpha, float beta, float hue, float sat, bool is_output, RocalTensorLayout layout,
+                                 RocalTensorOutputType dtype) {
+    return add_op<ColorTwistNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](ColorTwistNode &n) { n.init(alpha, beta, hue, sat); });
+}
+
+/* ------------------------------------------------------------------ warp affine / rotate */
+
+namespace {
+void default_dims(RocalTensor in, unsigned &w, unsigned &h) {
+    if (in && (w == 0 || h == 0)) {
+        w = (unsigned)static_cast<Tensor *>(in)->info().max_shape()[0];
+        h = (unsigned)static_cast<Tensor *>(in)->info().max_shape()[1];
+    }
+}
+}  // namespace
+
+RocalTensor rocalRotate(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam angle, unsigned dest_width, unsigned dest_height,
+                        RocalResizeInterpolationType interpolation_type, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    default_dims(in, dest_width, dest_height);
+    return add_op<RotateNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, nullptr,
+                              [&](RotateNode &n) { n.init(F(angle), interpolation_type); });
+}
+RocalTensor rocalRotateFixed(RocalContext c, RocalTensor in, float angle, bool is_output, unsigned dest_width, unsigned dest_height,
+                             RocalResizeInterpolationType interpolation_type, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    default_dims(in, dest_width, dest_height);
+    return add_op<RotateNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, nullptr,
+                              [&](RotateNode &n) { n.init(angle, interpolation_type); });
+}
+RocalTensor rocalWarpAffine(RocalContext c, RocalTensor in, bool is_output, unsigned dest_height, unsigned dest_width, RocalFloatParam x0,
+                            RocalFloatParam x1, RocalFloatParam y0, RocalFloatParam y1, RocalFloatParam o0, RocalFloatParam o1,
+                            RocalResizeInterpolationType interpolation_type, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    default_dims(in, dest_width, dest_height);
+    return add_op<WarpAffineNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, nullptr, [&](WarpAffineNode &n) {
+        n.init(F(x0), F(x1), F(y0), F(y1), F(o0), F(o1), interpolation_type);
+    });
+}
+RocalTensor rocalWarpAffineFixed(RocalContext c, RocalTensor in, float x0, float x1, float y0, float y1, float o0, float o1, bool is_output,
+                                 unsigned dest_height, unsigned dest_width, RocalResizeInterpolationType interpolation_type, RocalTensorLayout layout,
+                                 RocalTensorOutputType dtype) {
+    default_dims(in, dest_width, dest_height);
+    return add_op<WarpAffineNode>(c, in, is_output, layout, dtype, Dims::SET, dest_width, dest_height, nullptr,
+                                  [&](WarpAffineNode &n) { n.init(x0, x1, y0, y1, o0, o1, interpolation_type); });
+}

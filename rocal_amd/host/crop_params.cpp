@@ -1,0 +1,139 @@
+#include "crop_params.h"
+
+#include <algorithm>
+
+static Parameter<float> *uniform_default(const float range[2]) {
+    return ParameterFactory::instance()->create_uniform_float_rand_param(range[0], range[1])->core;
+}
+
+static void replace_param(Parameter<float> *&slot, Parameter<float> *p) {
+    if (!p) return;
+    ParameterFactory::instance()->destroy_param(slot);
+    slot = p;
+}
+
+CropParam::CropParam(unsigned n) : batch_size(n) {
+    x_drift_factor = uniform_default(CROP_X_DRIFT_RANGE);
+    y_drift_factor = uniform_default(CROP_Y_DRIFT_RANGE);
+    array_init();
+}
+
+void CropParam::array_init() {
+    for (auto *v : {&x1_arr_val, &y1_arr_val, &croph_arr_val, &cropw_arr_val, &x2_arr_val, &y2_arr_val}) v->resize(batch_size);
+}
+
+void CropParam::set_x_drift_factor(Parameter<float> *p) { replace_param(x_drift_factor, p); }
+void CropParam::set_y_drift_factor(Parameter<float> *p) { replace_param(y_drift_factor, p); }
+
+std::vector<uint32_t> CropParam::xywh() const {
+    std::vector<uint32_t> out(4 * batch_size);
+    for (unsigned i = 0; i < batch_size; i++) {
+        out[4 * i + 0] = x1_arr_val[i];
+        out[4 * i + 1] = y1_arr_val[i];
+        out[4 * i + 2] = cropw_arr_val[i];
+        out[4 * i + 3] = croph_arr_val[i];
+    }
+    return out;
+}
+
+RocalCropParam::RocalCropParam(unsigned n) : CropParam(n) {
+    crop_height_factor = uniform_default(CROP_HEIGHT_FACTOR_RANGE);
+    crop_width_factor = uniform_default(CROP_WIDTH_FACTOR_RANGE);
+}
+
+void RocalCropParam::set_crop_height_factor(Parameter<float> *p) { replace_param(crop_height_factor, p); }
+void RocalCropParam::set_crop_width_factor(Parameter<float> *p) { replace_param(crop_width_factor, p); }
+
+// parameter_rocal_crop.cpp:49-85. Three modes: user size at a user position, user size at an anchor
+// (nearbyintf of anchor * slack, round-half-even), or random factors of the ROI (truncating casts;
+// draw order per sample: height factor, width factor, x drift, y drift).
+void RocalCropParam::update_array() {
+    for (unsigned i = 0; i < batch_size; i++) {
+        const uint32_t W = in_roi[i].xywh.w, H = in_roi[i].xywh.h;
+        uint32_t cw, ch, px, py;
+        if (!_random) {
+            cw = (crop_w > 0 && crop_w <= W) ? crop_w : W;
+            ch = (crop_h > 0 && crop_h <= H) ? crop_h : H;
+            if (_is_fixed_crop) {
+                px = static_cast<size_t>(std::nearbyintf(_crop_anchor[0] * (W - cw)));
+                py = static_cast<size_t>(std::nearbyintf(_crop_anchor[1] * (H - ch)));
+            } else {
+                px = x1 >= W ? 0 : x1;
+                py = y1 >= H ? 0 : y1;
+            }
+        } else {
+            crop_height_factor->renew();
+            const float fh = crop_height_factor->get();
+            crop_width_factor->renew();
+            const float fw = crop_width_factor->get();
+            cw = static_cast<size_t>(fw * W);
+            ch = static_cast<size_t>(fh * H);
+            x_drift_factor->renew();
+            y_drift_factor->renew();
+            px = static_cast<size_t>(x_drift_factor->get() * (W - cw));
+            py = static_cast<size_t>(y_drift_factor->get() * (H - ch));
+        }
+        x1_arr_val[i] = px;
+        y1_arr_val[i] = py;
+        cropw_arr_val[i] = cw;
+        croph_arr_val[i] = ch;
+        x2_arr_val[i] = std::min(px + cw, W);
+        y2_arr_val[i] = std::min(py + ch, H);
+    }
+}
+
+RocalRandomCropParam::RocalRandomCropParam(unsigned n) : CropParam(n) {
+    area_factor = uniform_default(AREA_FACTOR_RANGE);
+    aspect_ratio = uniform_default(ASPECT_RATIO_RANGE);
+}
+
+void RocalRandomCropParam::set_area_factor(Parameter<float> *p) { replace_param(area_factor, p); }
+void RocalRandomCropParam::set_aspect_ratio(Parameter<float> *p) { replace_param(aspect_ratio, p); }
+
+// parameter_random_crop.cpp:44-100. Up to 5 attempts of (area, aspect ratio); a candidate is kept when it
+// is strictly smaller than the ROI in both directions. Sizes are truncated square roots computed in
+// double from a float area factor; the y drift parameter is renewed twice per accepted attempt.
+void RocalRandomCropParam::update_array() {
+    constexpr int attempts = 5;
+    for (unsigned i = 0; i < batch_size; i++) {
+        const uint32_t W = in_roi[i].xywh.w, H = in_roi[i].xywh.h;
+        auto fits = [&](uint32_t h, uint32_t w) { return h < H && w < W; };
+        uint32_t cw = cropw_arr_val[i], ch = croph_arr_val[i];  // the last batch's values when no attempt is made
+        for (int a = 0; a < attempts; a++) {
+            area_factor->renew();
+            aspect_ratio->renew();
+            const float area = area_factor->get();
+            const float ratio = aspect_ratio->get();
+            const double target = area * H * W;  // float products, widened on assignment
+            cw = static_cast<size_t>(std::sqrt(target * ratio));
+            ch = static_cast<size_t>(std::sqrt(target * (1 / ratio)));
+            if (fits(ch, cw)) {
+                x_drift_factor->renew();
+                y_drift_factor->renew();
+                y_drift_factor->renew();
+                x1_arr_val[i] = static_cast<size_t>(x_drift_factor->get() * (W - cw));
+                y1_arr_val[i] = static_cast<size_t>(y_drift_factor->get() * (H - ch));
+                break;
+            }
+        }
+        if (!fits(ch, cw)) {  // centre crop with the aspect ratio clamped into the allowed range
+            const float in_ratio = static_cast<float>(W) / H;
+            if (in_ratio < ASPECT_RATIO_RANGE[0]) {
+                cw = W;
+                ch = cw / ASPECT_RATIO_RANGE[0];
+            } else if (in_ratio > ASPECT_RATIO_RANGE[1]) {
+                ch = H;
+                cw = ch * ASPECT_RATIO_RANGE[1];
+            } else {
+                ch = H;
+                cw = W;
+            }
+            x1_arr_val[i] = (W - cw) / 2;
+            y1_arr_val[i] = (H - ch) / 2;
+        }
+        cropw_arr_val[i] = cw;
+        croph_arr_val[i] = ch;
+        x2_arr_val[i] = x1_arr_val[i] + cw;
+        y2_arr_val[i] = y1_arr_val[i] + ch;
+    }
+}

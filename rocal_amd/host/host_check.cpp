@@ -1,0 +1,258 @@
+// Test driver of the host layer, run by the test-suite as a child process.
+//   host_check params <seed>            prints, as JSON, what the parameter system produces (no GPU needed)
+//   host_check pipeline <scenario> <dir> builds a pipeline through the rocal* API, feeds <dir>/input.bin
+//                                        twice and writes every output batch + ROI to <dir> (needs the GPU)
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+#include <string>
+#include <vector>
+
+#include "rocal_host.h"
+
+namespace {
+
+template <typename T>
+std::string arr(const std::vector<T> &v) {
+    std::ostringstream s;
+    s.precision(9);
+    s << "[";
+    for (size_t i = 0; i < v.size(); i++) s << (i ? "," : "") << v[i];
+    s << "]";
+    return s.str();
+}
+
+int run_params(unsigned seed) {
+    auto *pf = ParameterFactory::instance();
+    pf->set_seed(seed);
+    std::ostringstream js;
+    js << "{";
+    // 1. seed sequence: the first four values are consumed here
+    std::vector<long long> seeds;
+    for (int i = 0; i < 4; i++) seeds.push_back(pf->get_seed_from_seedsequence());
+    js << "\"seeds\":" << arr(seeds);
+    // 2. user-created uniform / custom parameters (seeds 4,5,6)
+    auto *uf = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.08f, 1.0f));
+    auto *ui = static_cast<IntParam *>(rocalCreateIntUniformRand(0, 1));
+    const int cv[4] = {10, 20, 30, 40};
+    const double cf[4] = {0.1, 0.4, 0.3, 0.2};
+    auto *ci = static_cast<IntParam *>(rocalCreateIntRand(cv, cf, 4));
+    std::vector<float> vf{rocalGetFloatValue(uf)};
+    std::vector<int> vi{rocalGetIntValue(ui)}, vc{rocalGetIntValue(ci)};
+    for (int k = 0; k < 12; k++) {
+        pf->renew_parameters();
+        vf.push_back(rocalGetFloatValue(uf));
+        vi.push_back(rocalGetIntValue(ui));
+        vc.push_back(rocalGetIntValue(ci));
+    }
+    js << ",\"uniform_f\":" << arr(vf) << ",\"uniform_i\":" << arr(vi) << ",\"custom_i\":" << arr(vc);
+    // 3. a batch-sized mirror array on a node default (seeded with the factory seed itself)
+    ParameterVX<int> mirror(0, 1);
+    mirror.create_array(8);
+    std::vector<int> mv;
+    for (int b = 0; b < 3; b++) {
+        pf->renew_parameters();
+        mirror.update_array();
+        mv.insert(mv.end(), mirror.values().begin(), mirror.values().end());
+    }
+    js << ",\"mirror_default\":" << arr(mv);
+    // 4. random-resized-crop windows: user parameters first (seeds 7..10), then the crop object, whose own
+    //    defaults take seeds 11..14 before being replaced
+    const unsigned n = 6;
+    std::vector<Roi2DCords> roi(n);
+    const unsigned ws[n] = {640, 240, 333, 500, 64, 1000}, hs[n] = {480, 240, 500, 333, 48, 200};
+    for (unsigned i = 0; i < n; i++) roi[i].xywh = {0, 0, ws[i], hs[i]};
+    auto *area = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.08f, 1.0f));
+    auto *aspect = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.75f, 1.333f));
+    auto *xd = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.0f, 1.0f));
+    auto *yd = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.0f, 1.0f));
+    RocalRandomCropParam rrc(n);
+    rrc.set_area_factor(core(area));
+    rrc.set_aspect_ratio(core(aspect));
+    rrc.set_x_drift_factor(core(xd));
+    rrc.set_y_drift_factor(core(yd));
+    rrc.create_array();
+    std::vector<uint32_t> win;
+    for (int b = 0; b < 3; b++) {
+        pf->renew_parameters();
+        rrc.set_image_dimensions(roi.data());
+        rrc.update_array();
+        auto w = rrc.xywh();
+        win.insert(win.end(), w.begin(), w.end());
+    }
+    js << ",\"rrc_windows\":" << arr(win);
+    // 5. factor crops (seeds 15..18 for the user parameters)
+    auto *hf = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.55f, 0.95f));
+    auto *wf = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.55f, 0.95f));
+    auto *fx = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.01f, 0.99f));
+    auto *fy = static_cast<FloatParam *>(rocalCreateFloatUniformRand(0.01f, 0.99f));
+    RocalCropParam fc(n);
+    fc.set_crop_height_factor(core(hf));
+    fc.set_crop_width_factor(core(wf));
+    fc.set_x_drift_factor(core(fx));
+    fc.set_y_drift_factor(core(fy));
+    fc.set_random();
+    fc.create_array();
+    win.clear();
+    for (int b = 0; b < 2; b++) {
+        pf->renew_parameters();
+        fc.set_image_dimensions(roi.data());
+        fc.update_array();
+        auto w = fc.xywh();
+        win.insert(win.end(), w.begin(), w.end());
+    }
+    js << ",\"factor_windows\":" << arr(win);
+    // 6. anchored fixed crops and the resize size policy
+    RocalCropParam fixed(n);
+    fixed.crop_w = 224;
+    fixed.crop_h = 200;
+    fixed.set_fixed_crop(0.5f, 0.5f);
+    fixed.set_image_dimensions(roi.data());
+    fixed.update_array();
+    js << ",\"fixed_windows\":" << arr(fixed.xywh());
+    struct Probe : ResizeFamilyNode {
+        using ResizeFamilyNode::adjust_out_roi_size;
+    };
+    std::vector<unsigned> sizes;
+    const unsigned cases[][5] = {{640, 480, 256, 0, 0}, {640, 480, 0, 256, 0}, {640, 480, 300, 200, 1}, {640, 480, 256, 256, 2}, {480, 640, 256, 256, 2},
+                                 {640, 480, 256, 256, 3}, {333, 500, 0, 300, 3}, {333, 500, 300, 0, 2}, {1000, 200, 256, 256, 2}};
+    for (auto &c : cases)
+        for (unsigned mw : {0u, 400u}) {
+            unsigned w = c[2], h = c[3];
+            Probe::adjust_out_roi_size(c[0], c[1], w, h, (RocalResizeScalingMode)c[4], mw, mw ? 300 : 0);
+            sizes.push_back(w);
+            sizes.push_back(h);
+        }
+    js << ",\"resize_sizes\":" << arr(sizes) << "}";
+    std::cout << js.str() << std::endl;
+    return 0;
+}
+
+#define HIPCHK(x)                                                            \
+    if ((x) != hipSuccess) {                                                 \
+        std::cerr << "HIP call failed: " #x << std::endl;                   \
+        return 3;                                                            \
+    }
+
+int run_pipeline(const std::string &scenario, const std::string &dir) {
+    unsigned n, H, W;
+    std::vector<unsigned> rw, rh;
+    {
+        std::ifstream meta(dir + "/meta.txt");
+        if (!(meta >> n >> H >> W)) return 2;
+        rw.resize(n);
+        rh.resize(n);
+        for (unsigned i = 0; i < n; i++) meta >> rw[i] >> rh[i];
+    }
+    std::vector<unsigned char> host((size_t)n * H * W * 3);
+    {
+        std::ifstream in(dir + "/input.bin", std::ios::binary);
+        in.read(reinterpret_cast<char *>(host.data()), host.size());
+        if ((size_t)in.gcount() != host.size()) return 2;
+    }
+    rocalSetSeed(77);
+    RocalContext ctx = rocalCreate(n, ROCAL_PROCESS_GPU, 0);
+    if (!ctx) return 4;
+    void *dev = nullptr;
+    HIPCHK(hipMalloc(&dev, host.size() + 64));
+    HIPCHK(hipMemcpy(dev, host.data(), host.size(), hipMemcpyHostToDevice));
+    RocalTensor src = rocalDeviceSource(ctx, W, H, false);
+    std::vector<float> mean{123.675f, 116.28f, 103.53f}, stdv{58.395f, 57.12f, 57.375f};
+    std::vector<RocalTensor> outs;
+    RocalTensor mid = nullptr;
+    // A fair coin for the mirror flags, created first so that it takes the first seed of the sequence.
+    // (rocalCreateIntUniformRand(0, 1) truncates to 0 for every draw but one in 2^32, as in the reference.)
+    const int coin_v[2] = {0, 1};
+    const double coin_f[2] = {0.5, 0.5};
+    RocalIntParam coin = rocalCreateIntRand(coin_v, coin_f, 2);
+    if (scenario == "cmn") {
+        RocalIntParam mirror = coin;
+        outs.push_back(rocalCropMirrorNormalize(ctx, src, 40, 48, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP32));
+    } else if (scenario == "rrc_cmn") {
+        mid = rocalCropResizeFixed(ctx, src, 64, 64, false, 0.5f, 1.2f, 0.3f, 0.7f);
+        RocalIntParam mirror = coin;
+        outs.push_back(rocalCropMirrorNormalize(ctx, mid, 56, 56, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP16));
+    } else if (scenario == "chain") {
+        RocalTensor a = rocalResize(ctx, src, 40, 32, false);
+        RocalTensor b = rocalColorTwistFixed(ctx, a, 1.1f, 5.0f, 30.0f, 1.2f, true);
+        outs.push_back(b);
+        outs.push_back(rocalFlipFixed(ctx, b, 1, 0, true));
+    } else if (scenario == "rotate") {
+        outs.push_back(rocalRotateFixed(ctx, src, 30.0f, true));
+    } else if (scenario == "warp") {
+        outs.push_back(rocalWarpAffineFixed(ctx, src, 1.05f, 0.1f, -0.08f, 0.95f, 3.0f, -2.0f, true, 48, 56));
+    } else if (scenario == "rmn") {
+        RocalIntParam mirror = rocalCreateIntParameter(1);
+        outs.push_back(rocalResizeMirrorNormalize(ctx, src, 0, 0, mean, stdv, true, ROCAL_SCALING_MODE_STRETCH, {96, 96}, 48, 0, ROCAL_LINEAR_INTERPOLATION, mirror,
+                                                  ROCAL_NCHW, ROCAL_FP16));
+    } else if (scenario == "crops") {
+        outs.push_back(rocalCropCenterFixed(ctx, src, 32, 24, 1, true));
+        outs.push_back(rocalCropFixed(ctx, src, 30, 20, 1, true, 5, 7, 0));
+        outs.push_back(rocalResizeCropMirrorFixed(ctx, src, 36, 28, true, 40, 50, rocalCreateIntParameter(1)));
+        outs.push_back(rocalBrightnessFixed(ctx, src, 1.2f, 10.0f, true));
+        outs.push_back(rocalContrastFixed(ctx, src, 1.3f, 70.0f, true));
+    } else if (scenario == "errors") {
+        // every line must fail the way the reference's API does: null tensor / runtime error + a message
+        std::vector<float> zero_std{58.0f, 0.0f, 57.0f};
+        int bad = 0;
+        if (rocalCreate(n, ROCAL_PROCESS_CPU, 0) != nullptr) bad |= 1;
+        if (rocalCropMirrorNormalize(ctx, src, 0, 10, 0.5f, 0.5f, mean, stdv, true) != nullptr) bad |= 2;
+        if (rocalResize(ctx, src, 0, 0, true) != nullptr) bad |= 4;
+        if (rocalResize(ctx, src, 10, 10, true, ROCAL_SCALING_MODE_STRETCH, {}, 5, 0) != nullptr) bad |= 8;
+        if (rocalCropMirrorNormalize(ctx, nullptr, 10, 10, 0.5f, 0.5f, mean, stdv, true) != nullptr) bad |= 16;
+        RocalTensor t = rocalCropMirrorNormalize(ctx, src, 10, 10, 0.5f, 0.5f, mean, zero_std, true);
+        if (t == nullptr) bad |= 32;  // creation succeeds; the zero std is found in create_node()
+        if (rocalVerify(ctx) != ROCAL_RUNTIME_ERROR) bad |= 64;
+        if (std::string(rocalGetErrorMessage(ctx)).find("Standard deviation value cannot be 0") == std::string::npos) bad |= 128;
+        if (rocalRun(nullptr) != ROCAL_CONTEXT_INVALID) bad |= 256;
+        if (rocalUpdateFloatParameter(1.0f, rocalCreateFloatUniformRand(0, 1)) != ROCAL_INVALID_PARAMETER_TYPE) bad |= 512;
+        std::cout << "errors_bad_mask " << bad << std::endl;
+        return bad ? 5 : 0;
+    } else {
+        return 2;
+    }
+    for (auto t : outs)
+        if (!t) {
+            std::cerr << "node creation failed: " << rocalGetErrorMessage(ctx) << std::endl;
+            return 6;
+        }
+    if (rocalVerify(ctx) != ROCAL_OK) {
+        std::cerr << "verify failed: " << rocalGetErrorMessage(ctx) << std::endl;
+        return 7;
+    }
+    if (mid) std::cout << "intermediate_elided " << (rocalTensorBuffer(mid) == nullptr ? 1 : 0) << std::endl;
+    for (int b = 0; b < 2; b++) {
+        if (rocalDeviceSourceFeed(ctx, src, dev, rw.data(), rh.data()) != ROCAL_OK || rocalRun(ctx) != ROCAL_OK) {
+            std::cerr << "run failed: " << rocalGetErrorMessage(ctx) << std::endl;
+            return 8;
+        }
+        for (size_t k = 0; k < outs.size(); k++) {
+            const size_t bytes = rocalTensorDataSize(outs[k]);
+            std::vector<char> out(bytes);
+            HIPCHK(hipMemcpy(out.data(), rocalTensorBuffer(outs[k]), bytes, hipMemcpyDeviceToHost));
+            std::ofstream f(dir + "/out" + std::to_string(k) + "_b" + std::to_string(b) + ".bin", std::ios::binary);
+            f.write(out.data(), bytes);
+            const unsigned *roi = rocalTensorRoi(outs[k]);
+            std::ofstream r(dir + "/roi" + std::to_string(k) + "_b" + std::to_string(b) + ".txt");
+            for (unsigned i = 0; i < n; i++) r << roi[4 * i] << " " << roi[4 * i + 1] << " " << roi[4 * i + 2] << " " << roi[4 * i + 3] << "\n";
+        }
+    }
+    rocalRelease(ctx);
+    (void)hipFree(dev);
+    std::cout << "ok " << outs.size() << std::endl;
+    return 0;
+}
+
+}  // namespace
+
+int main(int argc, char **argv) {
+    if (argc >= 3 && !strcmp(argv[1], "params")) return run_params((unsigned)strtoul(argv[2], nullptr, 10));
+    if (argc >= 4 && !strcmp(argv[1], "pipeline")) return run_pipeline(argv[2], argv[3]);
+    std::cerr << "usage: host_check params <seed> | pipeline <scenario> <dir>" << std::endl;
+    return 1;
+}

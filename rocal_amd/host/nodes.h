@@ -1,0 +1,310 @@
+// The augmentation nodes of the hot path with rocAL's class names, init() overloads and default ranges.
+// create_node() builds one rmx_op where the reference calls vxExtRpp<Op>(); update_node() refreshes
+// the per-sample arrays every batch where the reference refreshes its vx_arrays and crop tensor.
+#pragma once
+#include <memory>
+#include <vector>
+
+#include "crop_params.h"
+#include "parameters.h"
+#include "pipeline.h"
+
+// rocAL/include/api/rocal_api_types.h:326-366
+enum RocalResizeScalingMode {
+    ROCAL_SCALING_MODE_DEFAULT = 0,
+    ROCAL_SCALING_MODE_STRETCH = 1,
+    ROCAL_SCALING_MODE_NOT_SMALLER = 2,
+    ROCAL_SCALING_MODE_NOT_LARGER = 3,
+    ROCAL_SCALING_MODE_MIN_MAX = 4
+};
+enum RocalResizeInterpolationType {
+    ROCAL_NEAREST_NEIGHBOR_INTERPOLATION = 0,
+    ROCAL_LINEAR_INTERPOLATION = 1,
+    ROCAL_CUBIC_INTERPOLATION = 2,
+    ROCAL_LANCZOS_INTERPOLATION = 3,
+    ROCAL_GAUSSIAN_INTERPOLATION = 4,
+    ROCAL_TRIANGULAR_INTERPOLATION = 5
+};
+
+// node_crop_mirror_normalize.cpp:34-123
+class CropMirrorNormalizeNode : public Node {
+   public:
+    CropMirrorNormalizeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(int crop_h, int crop_w, float anchor_x, float anchor_y, std::vector<float> &mean, std::vector<float> &std_dev, IntParam *mirror);
+    std::shared_ptr<RocalCropParam> get_crop_param() { return _crop_param; }
+    // for the resize node that absorbs this one
+    void scale_bias(std::vector<float> &scale, std::vector<float> &bias) const;
+    void refresh_for_fusion();  // the update_node() work when this node is fused away
+    const std::vector<int> &mirror_values() const { return _mirror.values(); }
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    std::shared_ptr<RocalCropParam> _crop_param;
+    std::vector<float> _mean, _std_dev, _scale, _bias;
+    ParameterVX<int> _mirror;
+    static constexpr int MIRROR_RANGE[2] = {0, 1};
+    friend class ResizeFamilyNode;
+};
+
+// node_crop.cpp:34-132
+class CropNode : public Node {
+   public:
+    CropNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(unsigned crop_h, unsigned crop_w, float x_drift, float y_drift);
+    void init(unsigned crop_h, unsigned crop_w);  // centre crop
+    void init(FloatParam *crop_h_factor, FloatParam *crop_w_factor, FloatParam *x_drift, FloatParam *y_drift);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    std::shared_ptr<RocalCropParam> _crop_param;
+};
+
+// node_random_crop.cpp:34-79
+class RandomCropNode : public Node {
+   public:
+    RandomCropNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(FloatParam *crop_area_factor, FloatParam *crop_aspect_ratio, FloatParam *x_drift, FloatParam *y_drift, int num_of_attempts);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    std::shared_ptr<RocalRandomCropParam> _crop_param;
+    int _num_of_attempts = 20;
+};
+
+// node_flip.cpp:31-64
+class FlipNode : public Node {
+   public:
+    FlipNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(int h_flag, int v_flag);
+    void init(IntParam *h_flag, IntParam *v_flag);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<int> _horizontal, _vertical;
+    static constexpr int HORIZONTAL_RANGE[2] = {0, 1};
+    static constexpr int VERTICAL_RANGE[2] = {0, 1};
+};
+
+// Shared part of the four resize nodes: one rmx resize op, per-sample destination sizes, optional
+// absorbed CropMirrorNormalize.
+class ResizeFamilyNode : public Node {
+   public:
+    using Node::Node;
+    bool try_absorb(Node *next) override;
+
+   protected:
+    void create_resize_op(int interpolation);
+    // window = source window per sample (x,y,w,h); mirror/mean/std optional
+    void update_resize_op(const std::vector<uint32_t> &window, const std::vector<uint32_t> &dst_w, const std::vector<uint32_t> &dst_h,
+                          const std::vector<int> *mirror, const std::vector<float> *mean, const std::vector<float> *std_dev);
+    void launch() override;
+    // ResizeNode::adjust_out_roi_size (node_resize.cpp:98-138), with the MIN_MAX mode of
+    // ResizeMirrorNormalizeNode (node_resize_mirror_normalize.cpp:138-160)
+    static void adjust_out_roi_size(unsigned src_w, unsigned src_h, unsigned &dst_w, unsigned &dst_h, RocalResizeScalingMode mode,
+                                    unsigned max_w, unsigned max_h);
+    int _interpolation_type = ROCAL_LINEAR_INTERPOLATION;
+    CropMirrorNormalizeNode *_absorbed = nullptr;
+};
+
+// node_resize.cpp:31-138
+class ResizeNode : public ResizeFamilyNode {
+   public:
+    using ResizeFamilyNode::ResizeFamilyNode;
+    void init(unsigned dest_width, unsigned dest_height, RocalResizeScalingMode scaling_mode, const std::vector<unsigned> &max_size,
+              RocalResizeInterpolationType interpolation_type);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    unsigned _out_width = 0, _out_height = 0, _max_width = 0, _max_height = 0;
+    RocalResizeScalingMode _scaling_mode = ROCAL_SCALING_MODE_STRETCH;
+};
+
+// node_crop_resize.cpp:32-123 (RandomResizedCrop when the window is random)
+class CropResizeNode : public ResizeFamilyNode {
+   public:
+    using ResizeFamilyNode::ResizeFamilyNode;
+    void init(float area, float aspect_ratio, float x_center_drift, float y_center_drift);
+    void init(FloatParam *area, FloatParam *aspect_ratio, FloatParam *x_center_drift, FloatParam *y_center_drift);
+    void init(unsigned crop_h, unsigned crop_w, float x_drift, float y_drift, RocalResizeInterpolationType interpolation_type);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    std::shared_ptr<RocalRandomCropParam> _crop_param;
+    std::shared_ptr<RocalCropParam> _crop_fixed_param;
+    bool _is_random_crop = true;
+};
+
+// node_resize_crop_mirror.cpp:33-101
+class ResizeCropMirrorNode : public ResizeFamilyNode {
+   public:
+    ResizeCropMirrorNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(unsigned crop_h, unsigned crop_w, IntParam *mirror, RocalResizeInterpolationType interpolation_type);
+    void init(FloatParam *crop_h_factor, FloatParam *crop_w_factor, IntParam *mirror, RocalResizeInterpolationType interpolation_type);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    std::shared_ptr<RocalCropParam> _crop_param;
+    ParameterVX<int> _mirror;
+    static constexpr int MIRROR_RANGE[2] = {0, 1};
+};
+
+// node_resize_mirror_normalize.cpp:34-198
+class ResizeMirrorNormalizeNode : public ResizeFamilyNode {
+   public:
+    ResizeMirrorNormalizeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(unsigned dest_width, unsigned dest_height, RocalResizeScalingMode scaling_mode, std::vector<unsigned> max_size,
+              RocalResizeInterpolationType interpolation_type, std::vector<float> &mean, std::vector<float> &std_dev, IntParam *mirror);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    unsigned _out_width = 0, _out_height = 0, _max_width = 0, _max_height = 0;
+    RocalResizeScalingMode _scaling_mode = ROCAL_SCALING_MODE_STRETCH;
+    std::vector<float> _mean, _std_dev, _mean_vec, _std_vec;
+    ParameterVX<int> _mirror;
+    static constexpr int MIRROR_RANGE[2] = {0, 1};
+};
+
+// color_augmentations/node_color_twist.cpp:33-74, node_brightness.cpp, node_contrast.cpp, node_hue.cpp, node_saturation.cpp
+class ColorTwistNode : public Node {
+   public:
+    ColorTwistNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float alpha, float beta, float hue, float sat);
+    void init(FloatParam *alpha, FloatParam *beta, FloatParam *hue, FloatParam *sat);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _alpha, _beta, _hue, _sat;
+    static constexpr float ALPHA_RANGE[2] = {0.1f, 1.95f};
+    static constexpr float BETA_RANGE[2] = {0.1f, 25.0f};
+    static constexpr float HUE_RANGE[2] = {5.0f, 170.0f};
+    static constexpr float SAT_RANGE[2] = {0.1f, 0.4f};
+};
+
+class BrightnessNode : public Node {
+   public:
+    BrightnessNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float alpha, float beta);
+    void init(FloatParam *alpha, FloatParam *beta);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _alpha, _beta;
+    static constexpr float ALPHA_RANGE[2] = {0.1f, 1.95f};
+    static constexpr float BETA_RANGE[2] = {0.0f, 25.0f};
+};
+
+class ContrastNode : public Node {
+   public:
+    ContrastNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float contrast_factor, float contrast_center);
+    void init(FloatParam *contrast_factor, FloatParam *contrast_center);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _factor, _center;
+    static constexpr float CONTRAST_FACTOR_RANGE[2] = {0.1f, 1.95f};
+    static constexpr float CONTRAST_CENTER_RANGE[2] = {60.0f, 90.0f};
+};
+
+class HueNode : public Node {
+   public:
+    HueNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float hue);
+    void init(FloatParam *hue);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _hue;
+    static constexpr float HUE_RANGE[2] = {-359.0f, 359.0f};
+};
+
+class SaturationNode : public Node {
+   public:
+    SaturationNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float sat);
+    void init(FloatParam *sat);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _sat;
+    static constexpr float SAT_RANGE[2] = {-0.5f, 0.5f};
+};
+
+// node_warp_affine.cpp:37-105
+class WarpAffineNode : public Node {
+   public:
+    WarpAffineNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float x0, float x1, float y0, float y1, float o0, float o1, RocalResizeInterpolationType interpolation_type);
+    void init(FloatParam *x0, FloatParam *x1, FloatParam *y0, FloatParam *y1, FloatParam *o0, FloatParam *o1,
+              RocalResizeInterpolationType interpolation_type);
+    const std::vector<float> &affine() const { return _affine; }
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    void draw_affine();
+    ParameterVX<float> _x0, _x1, _y0, _y1, _o0, _o1;
+    std::vector<float> _affine;
+    int _interpolation_type = ROCAL_LINEAR_INTERPOLATION;
+    static constexpr float COEFFICIENT_RANGE_0[2] = {-0.35f, 0.35f};
+    static constexpr float COEFFICIENT_RANGE_1[2] = {0.65f, 1.35f};
+    static constexpr float COEFFICIENT_RANGE_OFFSET[2] = {-10.0f, 10.0f};
+};
+
+// node_rotate.cpp:30-61
+class RotateNode : public Node {
+   public:
+    RotateNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float angle, RocalResizeInterpolationType interpolation_type);
+    void init(FloatParam *angle, RocalResizeInterpolationType interpolation_type);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _angle;
+    int _interpolation_type = ROCAL_LINEAR_INTERPOLATION;
+    static constexpr float ROTATE_ANGLE_RANGE[2] = {0.0f, 180.0f};
+};

@@ -1,0 +1,210 @@
+#include "pipeline.h"
+
+#include <hip/hip_runtime_api.h>
+
+#include <algorithm>
+#include <iostream>
+
+#include "parameters.h"
+
+/* ---------------------------------------------------------------- TensorInfo / Tensor */
+
+TensorInfo::TensorInfo(std::vector<size_t> dims, RocalTensorlayout layout, RocalTensorDataType dtype)
+    : _dims(std::move(dims)), _layout(layout), _dtype(dtype) {
+    if (_dims.size() != 4) THROW("image tensors have 4 dimensions")
+    recompute();
+    reallocate_roi();
+}
+
+void TensorInfo::recompute() {
+    if (_dims.size() != 4) return;
+    if (_layout == RocalTensorlayout::NHWC) {
+        _max_shape = {_dims[2], _dims[1]};
+        _channels = (unsigned)_dims[3];
+    } else {
+        _max_shape = {_dims[3], _dims[2]};
+        _channels = (unsigned)_dims[1];
+    }
+    _data_size = _dims[0] * _dims[1] * _dims[2] * _dims[3] * data_type_size();
+}
+
+void TensorInfo::modify_dims_width_and_height(RocalTensorlayout layout, size_t width, size_t height) {
+    const size_t n = _dims[0], c = _channels;
+    if (layout != RocalTensorlayout::NONE) _layout = layout;
+    if (_layout == RocalTensorlayout::NHWC)
+        _dims = {n, height, width, c};
+    else
+        _dims = {n, c, height, width};
+    recompute();
+    reallocate_roi();
+}
+
+void TensorInfo::set_tensor_layout(RocalTensorlayout layout) {
+    if (layout == RocalTensorlayout::NONE || layout == _layout) return;
+    const size_t n = _dims[0], c = _channels, w = _max_shape[0], h = _max_shape[1];
+    _layout = layout;
+    if (_layout == RocalTensorlayout::NHWC)
+        _dims = {n, h, w, c};
+    else
+        _dims = {n, c, h, w};
+    recompute();
+}
+
+void TensorInfo::reset_roi() {
+    for (size_t i = 0; i < batch_size(); i++) {
+        _roi.get()[i].xywh.x = 0;
+        _roi.get()[i].xywh.y = 0;
+        _roi.get()[i].xywh.w = (unsigned)_max_shape[0];
+        _roi.get()[i].xywh.h = (unsigned)_max_shape[1];
+    }
+}
+
+rmx_tensor_desc TensorInfo::desc() const {
+    rmx_tensor_desc d;
+    d.n = (uint32_t)_dims[0];
+    d.w = (uint32_t)_max_shape[0];
+    d.h = (uint32_t)_max_shape[1];
+    d.c = _channels;
+    d.layout = (int32_t)_layout;
+    d.dtype = (int32_t)_dtype;
+    return d;
+}
+
+void Tensor::update_tensor_roi(const std::vector<uint32_t> &width, const std::vector<uint32_t> &height) {
+    const unsigned max_w = (unsigned)_info.max_shape()[0], max_h = (unsigned)_info.max_shape()[1];
+    if (width.size() != height.size()) THROW("Batch size of Tensor height and width info does not match")
+    if (width.size() != _info.batch_size())
+        THROW("The batch size of actual Tensor height and width different from Tensor batch size " + TOSTR(width.size()) + " != " + TOSTR(_info.batch_size()))
+    Roi2DCords *roi = _info.roi();
+    for (size_t i = 0; i < width.size(); i++) {
+        roi[i].xywh.w = std::min(width[i], max_w);
+        roi[i].xywh.h = std::min(height[i], max_h);
+    }
+}
+
+/* ---------------------------------------------------------------- Graph */
+
+Graph::Graph(int gpu_id, void *stream) {
+    if (rmx_ctx_create(gpu_id, stream, stream ? 0 : 1, &_ctx) != RMX_OK) THROW(std::string("rmx_ctx_create failed: ") + rmx_last_error())
+}
+
+Graph::~Graph() { release(); }
+
+// Chain planning: a node may take over the work of the node that follows it (resize -> CropMirrorNormalize
+// through a virtual tensor nobody else reads). Everything else about verification happens in rmx_create_*.
+Graph::Status Graph::verify() {
+    for (size_t i = 0; i + 1 < _order.size(); i++) {
+        Node *a = _order[i], *b = _order[i + 1];
+        if (a->fused_away || b->fused_away) continue;
+        Tensor *mid = a->output()[0];
+        if (b->input()[0] != mid || mid->is_output) continue;
+        bool other_reader = false;
+        for (size_t k = 0; k < _order.size(); k++)
+            if (k != i + 1 && _order[k]->input()[0] == mid) other_reader = true;
+        if (other_reader) continue;
+        if (a->try_absorb(b)) {
+            b->fused_away = true;
+            mid->elided = true;
+        }
+    }
+    return Status::OK;
+}
+
+Graph::Status Graph::process() {
+    for (Node *n : _order)
+        if (!n->fused_away) n->launch();
+    if (rmx_ctx_sync(_ctx) != RMX_OK) THROW(std::string("rmx_ctx_sync failed: ") + rmx_last_error())
+    return Status::OK;
+}
+
+Graph::Status Graph::release() {
+    if (_ctx) {
+        rmx_ctx_destroy(_ctx);
+        _ctx = nullptr;
+    }
+    return Status::OK;
+}
+
+/* ---------------------------------------------------------------- Node */
+
+Node::~Node() { release(); }
+
+void Node::create(std::shared_ptr<Graph> graph) {
+    if (_outputs.empty() || _inputs.empty()) THROW("Uninitialized input/output arguments")
+    _graph = graph;
+    create_node();  // a node that is fused away still sets up its parameters here, on the user thread
+}
+
+void Node::update_parameters() { update_node(); }
+
+void Node::release() {
+    if (_node) {
+        rmx_op_destroy(_node);
+        _node = nullptr;
+    }
+}
+
+void Node::launch() {
+    Tensor *in = _inputs[0], *out = _outputs[0];
+    if (!in->buffer() || !out->buffer()) THROW("tensor without a device buffer at launch")
+    check(rmx_op_launch(_node, in->buffer(), out->buffer()), "rmx_op_launch");
+}
+
+void Node::check(int status, const char *what) {
+    if (status != RMX_OK) THROW(std::string(what) + " failed: " + rmx_last_error())
+}
+
+std::vector<uint32_t> Node::roi_as_array(const Roi2DCords *roi) const {
+    std::vector<uint32_t> out(4 * _batch_size);
+    for (size_t i = 0; i < _batch_size; i++) {
+        out[4 * i + 0] = roi[i].xywh.x;
+        out[4 * i + 1] = roi[i].xywh.y;
+        out[4 * i + 2] = roi[i].xywh.w;
+        out[4 * i + 3] = roi[i].xywh.h;
+    }
+    return out;
+}
+
+/* ---------------------------------------------------------------- MasterGraph */
+
+MasterGraph::MasterGraph(size_t batch_size, int gpu_id, void *stream) : _batch_size(batch_size), _graph(std::make_shared<Graph>(gpu_id, stream)) {}
+
+MasterGraph::~MasterGraph() {
+    _nodes.clear();
+    for (void *p : _owned_buffers) (void)hipFree(p);
+}
+
+Tensor *MasterGraph::create_tensor(const TensorInfo &info, bool is_output) {
+    _tensors.emplace_back(new Tensor(info));
+    Tensor *t = _tensors.back().get();
+    t->is_output = is_output;
+    if (is_output) _outputs.push_back(t);
+    return t;
+}
+
+// rocalVerify: plan chains, create every node's op on the user thread, then give every tensor that is
+// written by a launch a device buffer (the reference's ring buffer / virtual tensors).
+void MasterGraph::build() {
+    if (_built) THROW("graph already built")
+    for (auto &n : _nodes) _graph->add(n.get());
+    _graph->verify();
+    for (auto &n : _nodes) n->create(_graph);
+    for (auto &n : _nodes) {
+        Tensor *out = n->output()[0];
+        if (out->elided || out->buffer()) continue;
+        void *p = nullptr;
+        if (hipMalloc(&p, out->info().data_size() + 64) != hipSuccess) THROW("hipMalloc of " + TOSTR(out->info().data_size()) + " bytes failed")
+        if (hipMemset(p, 0, out->info().data_size() + 64) != hipSuccess) THROW("hipMemset failed")
+        _owned_buffers.push_back(p);
+        out->swap_handle(p);
+    }
+    _built = true;
+}
+
+// One batch: master_graph.cpp:408 (renew), :1010-1013 (update_parameters per node), :1015-1017 (process).
+void MasterGraph::run() {
+    if (!_built) THROW("rocalVerify must be called before rocalRun")
+    ParameterFactory::instance()->renew_parameters();
+    for (auto &n : _nodes) n->update_parameters();
+    _graph->process();
+}

@@ -1,0 +1,167 @@
+// Tensor / Graph / Node / pipeline context of the hot path, with rocAL's interface
+// (rocAL/include/pipeline/tensor.h:65-309, graph.h:29-44, node.h:30-63, master_graph.h:245-263) on top of
+// the C ABI in include/rocal_mi355x.h. A Node owns one rmx_op; Graph::process() launches the nodes in
+// creation order on one stream and waits, which is what vxProcessGraph does for the reference
+// (rocAL/source/pipeline/graph.cpp:96-103).
+#pragma once
+#include <cstdint>
+#include <list>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "exception.h"
+#include "rocal_mi355x.h"
+
+// rocAL/include/pipeline/commons.h:45-70,110-113 (same numeric values as the C ABI's enums)
+enum class RocalTensorlayout { NHWC = 0, NCHW = 1, NONE = 9 };
+enum class RocalTensorDataType { FP32 = 0, FP16 = 1, UINT8 = 2 };
+enum class RocalROIType { LTRB = 0, XYWH = 1 };
+
+// rocAL/include/pipeline/commons.h:115-140
+union Roi2DCords {
+    struct { unsigned l, t, r, b; } ltrb;
+    struct { unsigned x, y, w, h; } xywh;
+};
+
+class TensorInfo {
+   public:
+    TensorInfo() = default;
+    // dims in the order of the layout: NHWC -> {N,H,W,C}, NCHW -> {N,C,H,W}
+    TensorInfo(std::vector<size_t> dims, RocalTensorlayout layout, RocalTensorDataType dtype);
+    size_t batch_size() const { return _dims.at(0); }
+    const std::vector<size_t> &dims() const { return _dims; }
+    RocalTensorlayout layout() const { return _layout; }
+    RocalTensorDataType data_type() const { return _dtype; }
+    RocalROIType roi_type() const { return _roi_type; }
+    unsigned get_channels() const { return _channels; }
+    // {max_width, max_height}, as TensorInfo::max_shape() for images (tensor.h:262)
+    const std::vector<size_t> &max_shape() const { return _max_shape; }
+    size_t data_size() const { return _data_size; }
+    size_t data_type_size() const { return _dtype == RocalTensorDataType::FP32 ? 4 : _dtype == RocalTensorDataType::FP16 ? 2 : 1; }
+    void set_data_type(RocalTensorDataType t) { _dtype = t; recompute(); }
+    void set_roi_type(RocalROIType t) { _roi_type = t; }
+    // Permutes the dims when the layout changes; the ROI buffer stays shared (tensor.h:205-214).
+    void set_tensor_layout(RocalTensorlayout layout);
+    // Changes the layout when `layout` is not NONE and sets the padded width/height (tensor.h:223-245).
+    void modify_dims_width_and_height(RocalTensorlayout layout, size_t width, size_t height);
+    Roi2DCords *roi() const { return _roi.get(); }
+    void reallocate_roi() { _roi.reset(new Roi2DCords[batch_size()](), std::default_delete<Roi2DCords[]>()); reset_roi(); }
+    void reset_roi();
+    rmx_tensor_desc desc() const;
+
+   private:
+    void recompute();
+    std::vector<size_t> _dims;
+    RocalTensorlayout _layout = RocalTensorlayout::NHWC;
+    RocalTensorDataType _dtype = RocalTensorDataType::UINT8;
+    RocalROIType _roi_type = RocalROIType::XYWH;
+    unsigned _channels = 3;
+    std::vector<size_t> _max_shape{0, 0};
+    size_t _data_size = 0;
+    // Shared between copies of an info and re-allocated only when the padded width/height change
+    // (tensor.h:203,248): the output of a node that keeps the size (colour ops, flip) aliases its input's ROI.
+    std::shared_ptr<Roi2DCords> _roi;
+};
+
+class Tensor {
+   public:
+    explicit Tensor(const TensorInfo &info) : _info(info) {}
+    const TensorInfo &info() const { return _info; }
+    void *buffer() const { return _buffer; }
+    // The loader / ring buffer hands a new device buffer every batch (tensor.cpp:478-489).
+    void swap_handle(void *device_ptr) { _buffer = device_ptr; }
+    // Clamps to the padded maxima like Tensor::update_tensor_roi (tensor.cpp:193-220).
+    void update_tensor_roi(const std::vector<uint32_t> &width, const std::vector<uint32_t> &height);
+    bool is_output = false;
+    bool elided = false;  // virtual tensor inside a fused chain: never materialised
+
+   private:
+    TensorInfo _info;
+    void *_buffer = nullptr;
+};
+
+class Node;
+
+class Graph {
+   public:
+    enum class Status { OK = 0 };
+    explicit Graph(int gpu_id, void *stream = nullptr);
+    ~Graph();
+    Status verify();
+    Status process();
+    Status release();
+    rmx_ctx *get() { return _ctx; }
+    void add(Node *n) { _order.push_back(n); }
+
+   private:
+    rmx_ctx *_ctx = nullptr;
+    std::vector<Node *> _order;
+};
+
+class Node {
+   public:
+    Node(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)
+        : _inputs(inputs), _outputs(outputs), _batch_size(outputs[0]->info().batch_size()) {}
+    virtual ~Node();
+    void create(std::shared_ptr<Graph> graph);
+    void update_parameters();
+    std::vector<Tensor *> input() { return _inputs; }
+    std::vector<Tensor *> output() { return _outputs; }
+    void release();
+    const Roi2DCords *get_src_roi() { return _inputs[0]->info().roi(); }
+    const Roi2DCords *get_dst_roi() { return _outputs[0]->info().roi(); }
+    // --- used by Graph ---
+    virtual void launch();
+    bool fused_away = false;  // this node's work is done by the launch of the node that precedes it
+    // A CropMirrorNormalize node directly behind a resize node: the pair runs as one kernel.
+    virtual bool try_absorb(Node *) { return false; }
+
+   protected:
+    virtual void create_node() = 0;
+    virtual void update_node() = 0;
+    const std::vector<Tensor *> _inputs;
+    const std::vector<Tensor *> _outputs;
+    std::shared_ptr<Graph> _graph = nullptr;
+    rmx_op *_node = nullptr;
+    size_t _batch_size;
+    void check(int status, const char *what);
+    std::vector<uint32_t> roi_as_array(const Roi2DCords *roi) const;
+};
+
+// The part of Context + MasterGraph the hot path needs (rocAL/include/pipeline/master_graph.h:245-263,
+// source/pipeline/master_graph.cpp:247-260,323-335,408,1010-1017): owns tensors and nodes, builds them
+// on verify, and per batch renews parameters, updates every node and processes the graph.
+class MasterGraph {
+   public:
+    MasterGraph(size_t batch_size, int gpu_id, void *stream);
+    ~MasterGraph();
+    Tensor *create_tensor(const TensorInfo &info, bool is_output);
+    template <typename T>
+    std::shared_ptr<T> add_node(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs) {
+        auto node = std::make_shared<T>(inputs, outputs);
+        _nodes.push_back(node);
+        return node;
+    }
+    void build();
+    void run();
+    size_t batch_size() const { return _batch_size; }
+    const std::vector<Tensor *> &outputs() const { return _outputs; }
+    bool built() const { return _built; }
+
+   private:
+    size_t _batch_size;
+    std::shared_ptr<Graph> _graph;
+    std::list<std::shared_ptr<Node>> _nodes;
+    std::list<std::unique_ptr<Tensor>> _tensors;
+    std::vector<Tensor *> _outputs;
+    std::vector<void *> _owned_buffers;
+    bool _built = false;
+};
+
+struct Context {
+    Context(size_t batch_size, int gpu_id, void *stream) : master_graph(new MasterGraph(batch_size, gpu_id, stream)) {}
+    std::unique_ptr<MasterGraph> master_graph;
+    std::string error;
+    void capture_error(const std::string &e) { error = e; }
+};

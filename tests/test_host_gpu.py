@@ -1,0 +1,166 @@
+"""The C++ host layer (rocal_amd/host: rocAL's Node / Graph / Parameter interface and rocal* entry points)
+driving the HIP kernels through the C ABI, checked against the oracle. Each scenario is a small
+pipeline built with the reference's own API calls; the expected result is computed here from the
+oracle's restatement of the parameter laws and of the pixel arithmetic."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import orc
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HOST_CHECK = os.path.join(ROOT, "rocal_amd", "lib", "host_check")
+SEED = 77  # set by the driver with rocalSetSeed
+N, H, W = 6, 80, 96
+ROIS = [(96, 80), (70, 60), (96, 64), (81, 80), (50, 77), (33, 41)]  # (w, h)
+MEAN, STD = [123.675, 116.28, 103.53], [58.395, 57.12, 57.375]
+
+
+def _image():
+    rng = np.random.default_rng(5)
+    base = rng.integers(0, 256, (N, H // 4 + 1, W // 4 + 1, 3)).astype(np.float32)
+    img = np.repeat(np.repeat(base, 4, axis=1), 4, axis=2)[:, :H, :W]
+    img += rng.normal(0, 12, img.shape)
+    return np.clip(np.rint(img), 0, 255).astype(np.uint8)
+
+
+def _run(scenario, tmp_path, n_out, shapes):
+    img = _image()
+    img.tofile(tmp_path / "input.bin")
+    with open(tmp_path / "meta.txt", "w") as f:
+        f.write("%d %d %d\n" % (N, H, W))
+        for w, h in ROIS:
+            f.write("%d %d\n" % (w, h))
+    print("host_check pipeline", scenario, flush=True)
+    p = subprocess.run([HOST_CHECK, "pipeline", scenario, str(tmp_path)], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, (p.returncode, p.stdout, p.stderr)
+    outs = []
+    for b in range(2):
+        row = []
+        for k in range(n_out):
+            dt, shape = shapes[k]
+            row.append((np.fromfile(tmp_path / ("out%d_b%d.bin" % (k, b)), dtype=dt).reshape(shape),
+                        np.loadtxt(tmp_path / ("roi%d_b%d.txt" % (k, b)), dtype=np.int64).reshape(N, 4)))
+        outs.append(row)
+    return img, outs, p.stdout
+
+
+def _roi():
+    return np.array([[0, 0, w, h] for w, h in ROIS], np.uint32)
+
+
+def _coin_batches(batches):
+    """The driver's first parameter: CustomRand<int>({0,1},{.5,.5}) seeded with the first value of the
+    seed sequence; one draw in its constructor, then N draws per batch."""
+    g = orc.MT19937(int(orc.seed_seq_generate([SEED], 1024)[0]))
+    g.custom_index([0.5, 0.5])
+    return [np.array([g.custom_index([0.5, 0.5]) for _ in range(N)], np.uint32) for _ in range(batches)]
+
+
+def _same(got, exp, what):
+    assert got.shape == exp.shape, what
+    assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), "%s: %d values differ" % (what, (got != exp).sum())
+
+
+def test_crop_mirror_normalize_node(tmp_path):
+    img, outs, _ = _run("cmn", tmp_path, 1, [(np.float32, (N, 3, 40, 48))])
+    crop = np.stack([orc.fixed_crop(w, h, 48, 40, anchor=(0.5, 0.5)) for w, h in ROIS])
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    mirrors = _coin_batches(2)
+    assert mirrors[0].tolist() != mirrors[1].tolist() or mirrors[0].any()
+    for b in range(2):
+        got, roi = outs[b][0]
+        exp = orc.crop_mirror_normalize(img, crop, scale, bias, mirrors[b], 40, 48, orc.NCHW, orc.FP32)
+        _same(got, exp, "cmn batch %d" % b)
+        assert np.array_equal(roi[:, 2:], crop[:, 2:])  # the output ROI is the crop size
+
+
+def test_random_resized_crop_then_cmn_runs_as_one_kernel(tmp_path):
+    img, outs, log = _run("rrc_cmn", tmp_path, 1, [(np.float16, (N, 3, 56, 56))])
+    assert "intermediate_elided 1" in log  # the u8 tensor between the two nodes is never materialised
+    s = orc.FParam.simple
+    window = np.stack([orc.random_crop(s(0.5), s(1.2), s(0.3), s(0.7), w, h) for w, h in ROIS])
+    full = np.full(N, 64, np.uint32)
+    mid = orc.resize(img, window, full, full, 64, 64, interp=orc.LINEAR)  # the u8 image of the two-node graph
+    # CropResizeNode publishes the crop size (capped to 64) as the ROI of its output; the CMN crop follows it
+    mid_w, mid_h = np.minimum(window[:, 2], 64), np.minimum(window[:, 3], 64)
+    crop = np.stack([orc.fixed_crop(int(w), int(h), 56, 56, anchor=(0.5, 0.5)) for w, h in zip(mid_w, mid_h)])
+    assert (crop[:, 2] < 56).any() and (crop[:, 2] == 56).any()
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    mirrors = _coin_batches(2)
+    for b in range(2):
+        got, roi = outs[b][0]
+        exp = orc.crop_mirror_normalize(mid, crop, scale, bias, mirrors[b], 56, 56, orc.NCHW, orc.FP16)
+        _same(got, exp, "rrc+cmn batch %d" % b)
+        assert np.array_equal(roi[:, 2:], crop[:, 2:])
+
+
+def test_resize_colortwist_flip_chain_with_intermediate_tensors(tmp_path):
+    img, outs, _ = _run("chain", tmp_path, 2, [(np.uint8, (N, 32, 40, 3))] * 2)
+    dw, dh = np.full(N, 40, np.uint32), np.full(N, 32, np.uint32)
+    a = orc.resize(img, _roi(), dw, dh, 32, 40, interp=orc.LINEAR)
+    roi_a = np.array([[0, 0, 40, 32]] * N, np.uint32)
+    one = lambda v: np.full(N, v, np.float32)
+    b_exp = orc.color_twist(a, roi_a, one(1.1), one(5.0), one(30.0), one(1.2))
+    c_exp = orc.crop_mirror_normalize(b_exp, roi_a, None, None, np.ones(N, np.uint32), 32, 40, orc.NHWC, orc.UINT8, vflip=np.zeros(N, np.uint32))
+    for b in range(2):
+        _same(outs[b][0][0], b_exp, "colour twist of the resized image")
+        _same(outs[b][1][0], c_exp, "flip of the twisted image")
+        assert np.array_equal(outs[b][1][1], roi_a)  # same-size nodes share the ROI of their input
+
+
+def test_rotate_node(tmp_path):
+    img, outs, _ = _run("rotate", tmp_path, 1, [(np.uint8, (N, H, W, 3))])
+    m = np.stack([orc.rotate_matrix(30.0)] * N)
+    exp = orc.warp_affine(img, _roi(), m, np.full(N, W, np.uint32), np.full(N, H, np.uint32), H, W, interp=orc.LINEAR)
+    _same(outs[1][0][0], exp, "rotate")
+
+
+def test_warp_affine_node(tmp_path):
+    img, outs, _ = _run("warp", tmp_path, 1, [(np.uint8, (N, 48, 56, 3))])
+    # rocAL's fill order x0,y0,x1,y1,o0,o1 (node_warp_affine.cpp:43-48)
+    m = np.stack([orc.affine_from_rocal([1.05, -0.08, 0.1, 0.95, 3.0, -2.0])] * N)
+    exp = orc.warp_affine(img, _roi(), m, np.full(N, 56, np.uint32), np.full(N, 48, np.uint32), 48, 56, interp=orc.LINEAR)
+    _same(outs[0][0][0], exp, "warp affine")
+
+
+def test_resize_mirror_normalize_node_with_shorter_side_policy(tmp_path):
+    img, outs, _ = _run("rmn", tmp_path, 1, [(np.float16, (N, 3, 96, 96))])
+    sizes = np.array([orc.resize_out_size(w, h, 48, 48, 2, 96, 96) for w, h in ROIS], np.uint32)
+    sizes = np.minimum(sizes, 96)
+    assert len({tuple(s) for s in sizes.tolist()}) > 3  # ragged destination sizes
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    exp = orc.resize(img, _roi(), sizes[:, 0], sizes[:, 1], 96, 96, interp=orc.LINEAR, mirror=np.ones(N, np.uint32), scale=scale, bias=bias,
+                     layout=orc.NCHW, dtype=orc.FP16)
+    for b in range(2):
+        got, roi = outs[b][0]
+        _same(got, exp, "resize-mirror-normalize")
+        assert np.array_equal(roi[:, 2:], sizes)
+
+
+def test_crop_variants_and_point_ops(tmp_path):
+    img, outs, _ = _run("crops", tmp_path, 5, [(np.uint8, (N, 24, 32, 3)), (np.uint8, (N, 20, 30, 3)), (np.uint8, (N, 28, 36, 3)),
+                                                 (np.uint8, (N, H, W, 3)), (np.uint8, (N, H, W, 3))])
+    o = outs[1]
+    centre = np.stack([orc.fixed_crop(w, h, 32, 24, anchor=(0.5, 0.5)) for w, h in ROIS])
+    _same(o[0][0], orc.crop_mirror_normalize(img, centre, None, None, None, 24, 32, orc.NHWC, orc.UINT8), "centre crop")
+    placed = np.stack([orc.fixed_crop(w, h, 30, 20, x1=5, y1=7) for w, h in ROIS])
+    _same(o[1][0], orc.crop_mirror_normalize(img, placed, None, None, None, 20, 30, orc.NHWC, orc.UINT8), "placed crop")
+    window = np.stack([orc.fixed_crop(w, h, 50, 40) for w, h in ROIS])
+    exp = orc.resize(img, window, np.full(N, 36, np.uint32), np.full(N, 28, np.uint32), 28, 36, interp=orc.LINEAR, mirror=np.ones(N, np.uint32))
+    _same(o[2][0], exp, "resize-crop-mirror")
+    one = lambda v: np.full(N, v, np.float32)
+    _same(o[3][0], orc.brightness(img, _roi(), one(1.2), one(10.0)), "brightness")
+    _same(o[4][0], orc.contrast(img, _roi(), one(1.3), one(70.0)), "contrast")
+
+
+def test_api_errors_follow_the_reference(tmp_path):
+    _image().tofile(tmp_path / "input.bin")
+    with open(tmp_path / "meta.txt", "w") as f:
+        f.write("%d %d %d\n" % (N, H, W) + "".join("%d %d\n" % r for r in ROIS))
+    p = subprocess.run([HOST_CHECK, "pipeline", "errors", str(tmp_path)], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0 and "errors_bad_mask 0" in p.stdout, (p.returncode, p.stdout, p.stderr[-2000:])
