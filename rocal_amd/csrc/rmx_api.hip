@@ -74,6 +74,7 @@ struct rmx_op {
     const char *fast_name = "";
     int strips = 1, strip_rows = 1, tile_w = 512, lds_per_wave = 0, waves_per_block = 4;
     int aux0 = 0, aux1 = 0;
+    int fast_lds = 0, fast_strips = 1, fast_rows = 8;  // plan of fn_fast
     uint64_t algo_bytes = 0;
 };
 
@@ -241,8 +242,12 @@ uint64_t rmx_op_algorithmic_bytes(const rmx_op *op) { return op ? op->algo_bytes
 const char *rmx_op_plan(const rmx_op *op) {
     static thread_local char buf[256];
     if (!op) return "";
-    snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=%d",
-             (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block, op->fn_fast != nullptr);
+    if (op->fn_fast)
+        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d fast=1 (x-tiles per sample)",
+                 (long long)op->n * op->fast_strips, op->fast_strips, op->fast_rows, op->fast_lds);
+    else
+        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=0",
+                 (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block);
     return buf;
 }
 const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : op->kernel_name) : ""; }
@@ -265,16 +270,26 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.lds_bytes = op->lds_per_wave;
     a.aux0 = op->aux0;
     a.aux1 = op->aux1;
-    a.dbg = nullptr;
-    if (const char *e = getenv("RMX_EXP_DBGPTR")) a.dbg = (uint64_t *)strtoull(e, nullptr, 0);
-    const uint64_t waves = (uint64_t)op->n * (uint64_t)op->strips;
-    const int wpb = op->waves_per_block;
+    if (((uintptr_t)src) & 3u) return fail(RMX_ERR_INVALID, "the source batch must start at a 4-byte aligned address");
+    // the fast specialisation wants 16-byte aligned batch bases (rows of both sides are then aligned too)
+    const bool fast = op->fn_fast && ((((uintptr_t)dst) | ((uintptr_t)src)) & 15u) == 0;
+    int wpb = op->waves_per_block;
+    if (fast) {
+        a.strips = op->fast_strips;
+        a.lds_bytes = op->fast_lds;
+        a.aux0 = op->fast_rows;
+        wpb = std::max(1, std::min(4, op->ctx->max_lds_per_block / std::max(1, op->fast_lds)));
+        if (const char *e = getenv("RMX_EXP_WPB")) wpb = atoi(e);
+    }
+    const uint64_t waves = (uint64_t)op->n * (uint64_t)a.strips;
     const uint64_t blocks = (waves + wpb - 1) / wpb;
     if (blocks == 0 || blocks > 0x7fffffffull) return fail(RMX_ERR_INVALID, "grid of %llu workgroups is out of range", (unsigned long long)blocks);
-    const size_t lds = (size_t)op->lds_per_wave * wpb;
+    const size_t lds = (size_t)a.lds_bytes * wpb;
     if (lds > (size_t)op->ctx->max_lds_per_block) return fail(RMX_ERR_INVALID, "plan needs %zu bytes of LDS per workgroup (limit %d)", lds, op->ctx->max_lds_per_block);
     HIP_TRY(hipSetDevice(op->ctx->device));
-    rmx::KernelFn fn = (op->fn_fast && (((uintptr_t)dst) & 15u) == 0) ? op->fn_fast : op->fn;
+    rmx::KernelFn fn = fast ? op->fn_fast : op->fn;
+    a.wpb = wpb;
+    a.nblocks = (uint32_t)blocks;
     hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
     HIP_TRY(hipGetLastError());
     return RMX_OK;
@@ -481,12 +496,62 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         op->aux0 = rows;
         op->strips = std::max(1, (max_dh + rows - 1) / rows);
     }
-    // fast path: every written width a multiple of 8 and aligned destination rows
+    // fast path: every written width a multiple of 8 and aligned destination rows. Its wavefronts stage
+    // the whole source window of a strip of `rows` destination rows at once; the x-tile of a sample is
+    // narrowed until that window fits the LDS budget of one wavefront. The sizes are computed with the
+    // kernel's own float formulas.
     op->fn_fast = nullptr;
     if (op->interp == RMX_INTERP_LINEAR && op->dst.w % 8 == 0) {
-        bool ok = true;
+        // (the kernel multiplies row indices and the row stride with 24-bit multiplies)
+        bool ok = op->src.w * 3u < (1u << 23) && op->src.h < (1u << 23);
         for (int i = 0; i < op->n && ok; i++) ok = (t[i].dst_w % 8 == 0);
-        if (ok) op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->fast_name);
+        int rows = 8, cap = 12 * 1024;
+        if (const char *e = getenv("RMX_EXP_FAST_ROWS")) rows = std::max(1, atoi(e));
+        if (const char *e = getenv("RMX_EXP_FAST_LDS")) cap = atoi(e);
+        int need_max = 64;
+        for (int i = 0; i < op->n && ok; i++) {
+            RmxSample &s = t[i];
+            s.plan[0] = 8;
+            if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+            const float offx = (s.rx - 1.0f) * 0.5f, offy = (s.ry - 1.0f) * 0.5f;
+            const int xlo = s.src_x, xhi = s.src_x + s.src_w - 1;
+            int nrows = 2;
+            for (int r0 = 0; r0 < s.dst_h; r0 += rows) {
+                const int r1 = std::min(r0 + rows, (int)s.dst_h);
+                const int a_v = (int)std::floor(src_coord_h(s.pc_y + r0, s.ry, offy, (float)s.src_y));
+                const int b_v = (int)std::floor(src_coord_h(s.pc_y + r1 - 1, s.ry, offy, (float)s.src_y)) + 1;
+                nrows = std::max(nrows, b_v - a_v + 1);
+            }
+            int tw = std::min<int>(s.dst_w, 512);
+            for (;;) {
+                int pitch = 0;
+                for (int xt = 0; xt < s.dst_w; xt += tw) {
+                    const int w = std::min<int>(s.dst_w - xt, tw);
+                    const int ixmin = (int)std::floor(src_coord_h(s.pc_x + xt, s.rx, offx, (float)xlo));
+                    const int ixmax = (int)std::floor(src_coord_h(s.pc_x + xt + w - 1, s.rx, offx, (float)xlo));
+                    const int cs = std::max(std::min(ixmin, xhi), xlo), ce = std::max(std::min(ixmax + 1, xhi), xlo);
+                    const int nc = ce - cs + 1;
+                    pitch = std::max(pitch, (8 + ((nc + 3) >> 2) * 4) * 4);  // bytes: one dword per pixel + replicas
+                }
+                const long need = (long)nrows * pitch;
+                if (need <= cap) {
+                    s.plan[0] = tw;
+                    need_max = std::max<int>(need_max, (int)need);
+                    break;
+                }
+                if (tw <= 8) {
+                    ok = false;  // a window this tall does not fit: the general kernel takes the batch
+                    break;
+                }
+                tw = std::max(8, (tw / 2) / 8 * 8);
+            }
+        }
+        if (ok) {
+            op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->fast_name);
+            op->fast_lds = (need_max + 15) / 16 * 16;
+            op->fast_rows = rows;
+            op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
+        }
     }
     return RMX_OK;
 }

@@ -19,7 +19,10 @@ struct __attribute__((aligned(16))) RmxSample {
     float rx, ry;                        // src_len / rs_len (IEEE division done on the host)
     float fsx, fsy;                      // triangular: ratio > 1 ? 1/ratio : 1
     float scale[3], bias[3];             // normalisation: out = v*scale + bias
-    float color[4];                      // colour twist: alpha, beta, hue shift in sextants [0,6], saturation
+    union {
+        float color[4];                  // colour twist: alpha, beta, hue shift in sextants [0,6], saturation
+        int32_t plan[4];                 // resize fast path: [0] = x-tile width for this sample
+    };
     float m[6];                          // warp: destination -> source affine about the centres
 };
 static_assert(sizeof(RmxSample) == 128, "parameter table row must stay 128 bytes");
@@ -37,7 +40,8 @@ struct RmxKArgs {
     int32_t strips;          // wave strips per sample (grid = n*strips waves)
     int32_t lds_bytes;       // dynamic LDS per wave
     int32_t aux0, aux1;
-    uint64_t *dbg;           // experiment builds only: per-wave timestamps (NULL otherwise)
+    int32_t wpb;             // wavefronts per workgroup of this launch
+    uint32_t nblocks;        // workgroups of this launch
 };
 
 #define RMX_WAVE 64

@@ -216,8 +216,30 @@ struct PackedGroup {
     uint32_t w[WORDS];
 };
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
 template <typename T, int LAYOUT, bool REV>
 RMX_DEV void pack_group_dir(const float (&v)[3][PX], PackedGroup<T> &out) {
+    if constexpr (sizeof(T) == 2) {
+        // fp16: two values per conversion (round-to-nearest-even, as __float2half_rn)
+#pragma unroll
+        for (int i = 0; i < PX * 3 / 2; i++) {
+            float lo, hi;
+            if constexpr (LAYOUT == RMX_NCHW) {
+                const int c = (2 * i) / PX, k = (2 * i) % PX;
+                lo = REV ? v[c][PX - 1 - k] : v[c][k];
+                hi = REV ? v[c][PX - 2 - k] : v[c][k + 1];
+            } else {
+                const int k0 = (2 * i) / 3, c0 = (2 * i) % 3, k1 = (2 * i + 1) / 3, c1 = (2 * i + 1) % 3;
+                lo = REV ? v[c0][PX - 1 - k0] : v[c0][k0];
+                hi = REV ? v[c1][PX - 1 - k1] : v[c1][k1];
+            }
+            const f16x2 h = __builtin_convertvector((f32x2){lo, hi}, f16x2);
+            __builtin_memcpy(&out.w[i], &h, 4);
+        }
+        return;
+    }
     T e[PX * 3];
     if constexpr (LAYOUT == RMX_NCHW) {
 #pragma unroll
