@@ -74,7 +74,8 @@ struct rmx_op {
     const char *fast_name = "";
     int strips = 1, strip_rows = 1, tile_w = 512, lds_per_wave = 0, waves_per_block = 4;
     int aux0 = 0, aux1 = 0;
-    int fast_lds = 0, fast_strips = 1, fast_rows = 8;  // plan of fn_fast
+    int fast_lds = 0, fast_strips = 1, fast_rows = 8, fast_wpb = 1;  // plan of fn_fast
+    bool fast_needs_src16 = false;                                   // fn_fast also wants a 16-byte aligned source base
     uint64_t algo_bytes = 0;
 };
 
@@ -243,8 +244,8 @@ const char *rmx_op_plan(const rmx_op *op) {
     static thread_local char buf[256];
     if (!op) return "";
     if (op->fn_fast)
-        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d fast=1 (x-tiles per sample)",
-                 (long long)op->n * op->fast_strips, op->fast_strips, op->fast_rows, op->fast_lds);
+        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d waves_per_block=%d fast=1",
+                 (long long)op->n * op->fast_strips, op->fast_strips, op->fast_rows, op->fast_lds, op->fast_wpb);
     else
         snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=0",
                  (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block);
@@ -272,13 +273,13 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.aux1 = op->aux1;
     if (((uintptr_t)src) & 3u) return fail(RMX_ERR_INVALID, "the source batch must start at a 4-byte aligned address");
     // the fast specialisation wants 16-byte aligned batch bases (rows of both sides are then aligned too)
-    const bool fast = op->fn_fast && ((((uintptr_t)dst) | ((uintptr_t)src)) & 15u) == 0;
+    const bool fast = op->fn_fast && (((uintptr_t)dst) & 15u) == 0 && (!op->fast_needs_src16 || (((uintptr_t)src) & 15u) == 0);
     int wpb = op->waves_per_block;
     if (fast) {
         a.strips = op->fast_strips;
         a.lds_bytes = op->fast_lds;
         a.aux0 = op->fast_rows;
-        wpb = std::max(1, std::min(4, op->ctx->max_lds_per_block / std::max(1, op->fast_lds)));
+        wpb = op->fast_wpb;
         if (const char *e = getenv("RMX_EXP_WPB")) wpb = atoi(e);
     }
     const uint64_t waves = (uint64_t)op->n * (uint64_t)a.strips;
@@ -301,7 +302,7 @@ static int create_k1(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const r
     int rc = make_op(ctx, kind, src, dst, roi_type, out);
     if (rc) return rc;
     (*out)->norm = norm;
-    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, norm, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, norm, false, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -328,7 +329,21 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
         max_rows = std::max(max_rows, (int)s.dst_h);
     }
     op->algo_bytes = bytes;
-    plan_streaming(op, max_rows, 8);
+    int rows = 8;
+    if (const char *e = getenv("RMX_EXP_K1_ROWS")) rows = std::max(1, atoi(e));
+    plan_streaming(op, max_rows, rows);
+    // aligned specialisation: whole 8-pixel groups everywhere and 16-byte aligned destination rows
+    bool aligned = op->dst.w % 8 == 0;
+    for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
+    op->fn_fast = nullptr;
+    if (aligned) {
+        op->fn_fast = rmx::select_cmn_kernel(op->dst.dtype, op->dst.layout, op->norm, true, &op->fast_name);
+        op->fast_strips = op->strips;
+        op->fast_lds = 0;
+        op->fast_rows = op->aux0;
+        op->fast_wpb = op->waves_per_block;
+        op->fast_needs_src16 = false;
+    }
     return commit_slot(op, slot);
 }
 
@@ -505,7 +520,8 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         // (the kernel multiplies row indices and the row stride with 24-bit multiplies)
         bool ok = op->src.w * 3u < (1u << 23) && op->src.h < (1u << 23);
         for (int i = 0; i < op->n && ok; i++) ok = (t[i].dst_w % 8 == 0);
-        int rows = 8, cap = 12 * 1024;
+        // 4 rows and a 10 KB slice measured best on MI355X (more, shorter-lived wavefronts per CU)
+        int rows = 4, cap = 10 * 1024;
         if (const char *e = getenv("RMX_EXP_FAST_ROWS")) rows = std::max(1, atoi(e));
         if (const char *e = getenv("RMX_EXP_FAST_LDS")) cap = atoi(e);
         int need_max = 64;
@@ -551,6 +567,8 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             op->fast_lds = (need_max + 15) / 16 * 16;
             op->fast_rows = rows;
             op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
+            op->fast_wpb = 1;  // a workgroup's LDS is released only when its last wavefront ends: one-wave groups keep the CU full
+            op->fast_needs_src16 = false;  // its loads only need dword alignment
         }
     }
     return RMX_OK;
@@ -640,7 +658,7 @@ static int create_color(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, cons
     int rc = make_op(ctx, kind, src, dst, roi_type, out);
     if (rc) return rc;
     const bool twist = (kind == OP_COLOR_TWIST || kind == OP_HUE || kind == OP_SATURATION);
-    (*out)->fn = rmx::select_color_kernel(twist ? 1 : 0, dst->dtype, dst->layout, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_color_kernel(twist ? 1 : 0, dst->dtype, dst->layout, false, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -673,7 +691,22 @@ static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const 
         max_rows = std::max(max_rows, (int)s.dst_h);
     }
     op->algo_bytes = bytes;
-    plan_streaming(op, max_rows, 8);
+    int rows = 8;
+    if (const char *e = getenv("RMX_EXP_K3_ROWS")) rows = std::max(1, atoi(e));
+    plan_streaming(op, max_rows, rows);
+    // aligned specialisation: whole 8-pixel groups everywhere and 16-byte aligned destination rows
+    bool aligned = op->dst.w % 8 == 0;
+    for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
+    op->fn_fast = nullptr;
+    if (aligned) {
+        const bool twist = (op->kind == OP_COLOR_TWIST || op->kind == OP_HUE || op->kind == OP_SATURATION);
+        op->fn_fast = rmx::select_color_kernel(twist ? 1 : 0, op->dst.dtype, op->dst.layout, true, &op->fast_name);
+        op->fast_strips = op->strips;
+        op->fast_lds = 0;
+        op->fast_rows = op->aux0;
+        op->fast_wpb = op->waves_per_block;
+        op->fast_needs_src16 = false;
+    }
     return commit_slot(op, slot);
 }
 

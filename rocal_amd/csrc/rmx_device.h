@@ -240,6 +240,28 @@ RMX_DEV void pack_group_dir(const float (&v)[3][PX], PackedGroup<T> &out) {
         }
         return;
     }
+    if constexpr (sizeof(T) == 1) {
+        // u8: v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 and drops the byte into place
+#pragma unroll
+        for (int i = 0; i < PX * 3 / 4; i++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int e = 4 * i + b;
+                float val;
+                if constexpr (LAYOUT == RMX_NCHW) {
+                    const int c = e / PX, k = e % PX;
+                    val = REV ? v[c][PX - 1 - k] : v[c][k];
+                } else {
+                    const int k = e / 3, c = e % 3;
+                    val = REV ? v[c][PX - 1 - k] : v[c][k];
+                }
+                w = __builtin_amdgcn_cvt_pk_u8_f32(val, b, w);
+            }
+            out.w[i] = w;
+        }
+        return;
+    }
     T e[PX * 3];
     if constexpr (LAYOUT == RMX_NCHW) {
 #pragma unroll

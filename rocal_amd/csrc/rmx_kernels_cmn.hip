@@ -5,22 +5,28 @@
 // wave covers G = 64/L rows at once, L = lanes per row, each lane producing 8 adjacent
 // pixels: a 28-byte realigned read of packed RGB in, three 128-bit planar stores out (fp16).
 // HBM-bound: 3 bytes read and 3*sizeof(T) written per output pixel, no reuse.
+//
+// FAST variant (every written width a multiple of 8, 16-byte aligned destination rows): the loads of up
+// to four row steps are issued back to back before the first one is used, and the stores follow, so a
+// wavefront pays one memory round trip per strip instead of one per row step (loads and stores share one
+// in-order counter on this hardware: a load issued behind a store waits for that store as well).
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
 namespace rmx {
 
-template <typename T, int LAYOUT, bool NORM>
+template <typename T, int LAYOUT, bool NORM, bool FAST>
 __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
-    const uint32_t nblocks = gridDim.x;
-    uint32_t wave = xcd_swizzle(blockIdx.x, nblocks) * (blockDim.x / RMX_WAVE) + (threadIdx.x / RMX_WAVE);
+    uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + (threadIdx.x / RMX_WAVE);
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
     const int s = (int)(wave / (uint32_t)a.strips);
     const int strip = (int)(wave % (uint32_t)a.strips);
-    const RmxSample &P = a.table[s];
+    // whole table row in one round trip (the empty statement keeps the fetch above the early exit)
+    const RmxSample P = a.table[s];
+    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.flags), "s"(P.scale[0]), "s"(P.bias[2]));
 
     const int cw = P.dst_w, ch = P.dst_h;
     const int srows = a.aux0;
@@ -54,51 +60,99 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
         const bool active = lr < G;
         // source column of group pixel 0 (mirror reads the mirrored run and reverses it)
         const int sx0 = x1 + (hf ? (cw - gx - cnt) : gx);
-        for (int r = r0 + lr; r < r1 && active; r += G) {
-            const int sy = y1 + (vf ? (ch - 1 - r) : r);
-            const uint8_t *p = simg + (size_t)sy * row_stride + (size_t)sx0 * 3;
-            uint32_t w[6];
-            load_realigned<7>(p, buf_end, w);
-            float v[3][PX];
-            unpack8(w, v);
-            if constexpr (NORM) {
+        if constexpr (FAST) {
+            constexpr int NI = 4;  // row steps in flight
+            for (int rb = r0 + lr; rb < r1 && active; rb += NI * G) {
+                const uint32_t *q[NI];
+                uint32_t ph[NI];
+                bool safe = true;
 #pragma unroll
-                for (int c = 0; c < 3; c++)
+                for (int i = 0; i < NI; i++) {
+                    const int r = min(rb + i * G, r1 - 1);  // steps beyond the strip repeat its last row (never stored)
+                    const int sy = y1 + (vf ? (ch - 1 - r) : r);
+                    const uint8_t *p = simg + (size_t)sy * row_stride + (size_t)sx0 * 3;
+                    ph[i] = (uint32_t)((uintptr_t)p & 3u);
+                    q[i] = reinterpret_cast<const uint32_t *>(p - ph[i]);
+                    safe = safe && ((const uint8_t *)(q[i] + 7) <= buf_end);
+                }
+                uint32_t w[NI][6];
+                if (safe) {
+                    u32x4_a4 t[NI];
+                    u32x3_a4 u[NI];
 #pragma unroll
-                    for (int k = 0; k < PX; k++) v[c][k] = __builtin_fmaf(v[c][k], sc[c], bi[c]);
+                    for (int i = 0; i < NI; i++) {
+                        t[i] = *reinterpret_cast<const u32x4_a4 *>(q[i]);
+                        u[i] = *reinterpret_cast<const u32x3_a4 *>(q[i] + 4);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NI; i++) {
+                        const uint32_t d[7] = {t[i].x, t[i].y, t[i].z, t[i].w, u[i].x, u[i].y, u[i].z};
+#pragma unroll
+                        for (int j = 0; j < 6; j++) w[i][j] = __builtin_amdgcn_alignbyte(d[j + 1], d[j], ph[i]);
+                    }
+                } else {
+                    // last bytes of the batch buffer: the bounds-checked loader
+#pragma unroll
+                    for (int i = 0; i < NI; i++)
+                        load_realigned<7>(reinterpret_cast<const uint8_t *>(q[i]) + ph[i], buf_end, w[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < NI; i++) {
+                    const int r = rb + i * G;
+                    if (r < r1) {
+                        float v[3][PX];
+                        unpack8(w[i], v);
+                        if constexpr (NORM) {
+#pragma unroll
+                            for (int c = 0; c < 3; c++)
+#pragma unroll
+                                for (int k = 0; k < PX; k++) v[c][k] = __builtin_fmaf(v[c][k], sc[c], bi[c]);
+                        }
+                        PackedGroup<T> packed;
+                        pack_group<T, LAYOUT>(v, hf, packed);
+                        store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                    }
+                }
             }
-            store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, cnt, v, hf);
+        } else {
+            for (int r = r0 + lr; r < r1 && active; r += G) {
+                const int sy = y1 + (vf ? (ch - 1 - r) : r);
+                const uint8_t *p = simg + (size_t)sy * row_stride + (size_t)sx0 * 3;
+                uint32_t w[6];
+                load_realigned<7>(p, buf_end, w);
+                float v[3][PX];
+                unpack8(w, v);
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int c = 0; c < 3; c++)
+#pragma unroll
+                        for (int k = 0; k < PX; k++) v[c][k] = __builtin_fmaf(v[c][k], sc[c], bi[c]);
+                }
+                store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, cnt, v, hf);
+            }
         }
     }
 }
 
-#define RMX_CMN_INST(T, LAY, NORM) template __global__ void rmx_cmn_kernel<T, LAY, NORM>(RmxKArgs);
-RMX_CMN_INST(float, RMX_NCHW, true)
-RMX_CMN_INST(float, RMX_NHWC, true)
-RMX_CMN_INST(__half, RMX_NCHW, true)
-RMX_CMN_INST(__half, RMX_NHWC, true)
-RMX_CMN_INST(uint8_t, RMX_NCHW, true)
-RMX_CMN_INST(uint8_t, RMX_NHWC, true)
-RMX_CMN_INST(float, RMX_NCHW, false)
-RMX_CMN_INST(float, RMX_NHWC, false)
-RMX_CMN_INST(__half, RMX_NCHW, false)
-RMX_CMN_INST(__half, RMX_NHWC, false)
-RMX_CMN_INST(uint8_t, RMX_NCHW, false)
-RMX_CMN_INST(uint8_t, RMX_NHWC, false)
-
-template <typename T>
-static KernelFn pick_layout(int layout, bool norm) {
-    if (layout == RMX_NCHW) return norm ? (KernelFn)rmx_cmn_kernel<T, RMX_NCHW, true> : (KernelFn)rmx_cmn_kernel<T, RMX_NCHW, false>;
-    return norm ? (KernelFn)rmx_cmn_kernel<T, RMX_NHWC, true> : (KernelFn)rmx_cmn_kernel<T, RMX_NHWC, false>;
+template <typename T, int LAYOUT>
+static KernelFn pick_variant(bool norm, bool fast) {
+    if (fast) return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, true> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, true>;
+    return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, false> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, false>;
 }
 
-KernelFn select_cmn_kernel(int dtype, int layout, bool norm, const char **name) {
+template <typename T>
+static KernelFn pick_layout(int layout, bool norm, bool fast) {
+    if (layout == RMX_NCHW) return pick_variant<T, RMX_NCHW>(norm, fast);
+    return pick_variant<T, RMX_NHWC>(norm, fast);
+}
+
+KernelFn select_cmn_kernel(int dtype, int layout, bool norm, bool fast, const char **name) {
     static const char *names[3] = {"rmx_cmn_kernel<float", "rmx_cmn_kernel<__half", "rmx_cmn_kernel<unsigned char"};
     *name = names[dtype];
     switch (dtype) {
-        case RMX_FP32: return pick_layout<float>(layout, norm);
-        case RMX_FP16: return pick_layout<__half>(layout, norm);
-        default: return pick_layout<uint8_t>(layout, norm);
+        case RMX_FP32: return pick_layout<float>(layout, norm, fast);
+        case RMX_FP16: return pick_layout<__half>(layout, norm, fast);
+        default: return pick_layout<uint8_t>(layout, norm, fast);
     }
 }
 

@@ -12,54 +12,42 @@ namespace rmx {
 
 enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
 
+// Branch-free: every choice is a select. Lanes of a wavefront hold pixels of different hue sectors, so
+// branches would run every case one after the other under changing execution masks.
 RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, float alpha, float beta, float shift, float satf) {
-    float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
-    float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
-    float delta = cmax - cmin;
-    float rd = rcp[(int)delta];      // 0 when delta == 0
+    const float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
+    const float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
+    const float delta = cmax - cmin;
+    const float rd = rcp[(int)delta];      // 0 when delta == 0
     float s = delta * rcp[(int)cmax];
-    float num, add;
-    if (cmax == r) {
-        num = g - b;
-        add = 0.0f;
-    } else if (cmax == g) {
-        num = b - r;
-        add = 2.0f;
-    } else {
-        num = r - g;
-        add = 4.0f;
-    }
-    if (delta == 0.0f) {
-        num = 0.0f;
-        add = 0.0f;
-    }
+    const bool is_r = cmax == r, is_g = cmax == g, grey = delta == 0.0f;
+    float num = is_r ? (g - b) : (is_g ? (b - r) : (r - g));
+    float add = is_r ? 0.0f : (is_g ? 2.0f : 4.0f);
+    num = grey ? 0.0f : num;
+    add = grey ? 0.0f : add;
     float hh = __builtin_fmaf(num, rd, add + shift);
-    if (hh < 0.0f) hh += 6.0f;
-    if (hh >= 6.0f) hh -= 6.0f;
+    hh = hh < 0.0f ? hh + 6.0f : hh;
+    hh = hh >= 6.0f ? hh - 6.0f : hh;
     s = s * satf;
     s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
-    int hi = (int)hh;
-    float hf = hh - (float)hi;
-    float vsat = cmax * s;
-    float vsatf = vsat * hf;
-    float pp = cmax - vsat;
-    float qq = cmax - vsatf;
-    float tt = pp + vsatf;
-    float ro, go, bo;
-    switch (hi) {
-        case 0: ro = cmax; go = tt; bo = pp; break;
-        case 1: ro = qq; go = cmax; bo = pp; break;
-        case 2: ro = pp; go = cmax; bo = tt; break;
-        case 3: ro = pp; go = qq; bo = cmax; break;
-        case 4: ro = tt; go = pp; bo = cmax; break;
-        default: ro = cmax; go = pp; bo = qq; break;
-    }
+    const int hi = (int)hh;
+    const float hf = hh - (float)hi;
+    const float vsat = cmax * s;
+    const float vsatf = vsat * hf;
+    const float pp = cmax - vsat;
+    const float qq = cmax - vsatf;
+    const float tt = pp + vsatf;
+    // sector table (hi >= 5 is the last sector):  r: V q p p t V   g: t V V q p p   b: p p t V V q
+    const bool h0 = hi == 0, h1 = hi == 1, h2 = hi == 2, h3 = hi == 3, h4 = hi == 4;
+    const float ro = h1 ? qq : ((h2 || h3) ? pp : (h4 ? tt : cmax));
+    const float go = h0 ? tt : ((h1 || h2) ? cmax : (h3 ? qq : pp));
+    const float bo = (h0 || h1) ? pp : (h2 ? tt : ((h3 || h4) ? cmax : qq));
     r = __builtin_fmaf(ro, alpha, beta);
     g = __builtin_fmaf(go, alpha, beta);
     b = __builtin_fmaf(bo, alpha, beta);
 }
 
-template <typename T, int LAYOUT, int KIND>
+template <typename T, int LAYOUT, int KIND, bool FAST>
 __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     __shared__ float rcp[256];
     if constexpr (KIND == COLOR_TWIST) {
@@ -69,12 +57,14 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
-    uint32_t wave = blockIdx.x * (blockDim.x / RMX_WAVE) + (threadIdx.x / RMX_WAVE);
+    uint32_t wave = blockIdx.x * (uint32_t)a.wpb + (threadIdx.x / RMX_WAVE);
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
     const int s = (int)(wave / (uint32_t)a.strips);
     const int strip = (int)(wave % (uint32_t)a.strips);
-    const RmxSample &P = a.table[s];
+    // whole table row in one round trip (the empty statement keeps the fetch above the early exit)
+    const RmxSample P = a.table[s];
+    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.flags), "s"(P.color[0]), "s"(P.color[3]));
     const int w = P.dst_w, h = P.dst_h;
     const int srows = a.aux0;
     const int r0 = strip * srows;
@@ -88,6 +78,18 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
 
+    auto colour = [&](float (&v)[3][PX]) {
+#pragma unroll
+        for (int k = 0; k < PX; k++) {
+            if constexpr (KIND == COLOR_TWIST) {
+                twist_px(v[0][k], v[1][k], v[2][k], rcp, p0, p1, p2, p3);
+            } else {
+#pragma unroll
+                for (int c = 0; c < 3; c++) v[c][k] = __builtin_fmaf(v[c][k] - p2, p0, p1);
+            }
+        }
+    };
+
     for (int xt = 0; xt < w; xt += RMX_WAVE * PX) {
         const int tw = min(w - xt, RMX_WAVE * PX);
         const int L = (tw + PX - 1) / PX;
@@ -96,45 +98,89 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
         const int g = lane - lr * L;
         const int gx = xt + g * PX;
         const int cnt = min(PX, w - gx);
-        for (int r = r0 + lr; r < r1 && lr < G; r += G) {
-            const uint8_t *p = simg + (size_t)(y1 + r) * row_stride + (size_t)(x1 + gx) * 3;
-            uint32_t wd[6];
-            load_realigned<7>(p, buf_end, wd);
-            float v[3][PX];
-            unpack8(wd, v);
+        if constexpr (FAST) {
+            // whole groups and aligned destination rows: the loads of up to NI row steps go out together,
+            // the stores follow (one memory round trip per strip, see the CropMirrorNormalize kernel)
+            constexpr int NI = (KIND == COLOR_TWIST) ? 2 : 4;
+            for (int rb = r0 + lr; rb < r1 && lr < G; rb += NI * G) {
+                const uint32_t *q[NI];
+                uint32_t ph[NI];
+                bool safe = true;
 #pragma unroll
-            for (int k = 0; k < PX; k++) {
-                if constexpr (KIND == COLOR_TWIST) {
-                    twist_px(v[0][k], v[1][k], v[2][k], rcp, p0, p1, p2, p3);
+                for (int i = 0; i < NI; i++) {
+                    const int r = min(rb + i * G, r1 - 1);
+                    const uint8_t *p = simg + (size_t)(y1 + r) * row_stride + (size_t)(x1 + gx) * 3;
+                    ph[i] = (uint32_t)((uintptr_t)p & 3u);
+                    q[i] = reinterpret_cast<const uint32_t *>(p - ph[i]);
+                    safe = safe && ((const uint8_t *)(q[i] + 7) <= buf_end);
+                }
+                uint32_t wd[NI][6];
+                if (safe) {
+                    u32x4_a4 t[NI];
+                    u32x3_a4 u[NI];
+#pragma unroll
+                    for (int i = 0; i < NI; i++) {
+                        t[i] = *reinterpret_cast<const u32x4_a4 *>(q[i]);
+                        u[i] = *reinterpret_cast<const u32x3_a4 *>(q[i] + 4);
+                    }
+#pragma unroll
+                    for (int i = 0; i < NI; i++) {
+                        const uint32_t d[7] = {t[i].x, t[i].y, t[i].z, t[i].w, u[i].x, u[i].y, u[i].z};
+#pragma unroll
+                        for (int j = 0; j < 6; j++) wd[i][j] = __builtin_amdgcn_alignbyte(d[j + 1], d[j], ph[i]);
+                    }
                 } else {
 #pragma unroll
-                    for (int c = 0; c < 3; c++) v[c][k] = __builtin_fmaf(v[c][k] - p2, p0, p1);
+                    for (int i = 0; i < NI; i++)
+                        load_realigned<7>(reinterpret_cast<const uint8_t *>(q[i]) + ph[i], buf_end, wd[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < NI; i++) {
+                    const int r = rb + i * G;
+                    if (r < r1) {
+                        float v[3][PX];
+                        unpack8(wd[i], v);
+                        colour(v);
+                        PackedGroup<T> packed;
+                        pack_group_dir<T, LAYOUT, false>(v, packed);
+                        store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                    }
                 }
             }
-            store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, cnt, v, false);
+        } else {
+            for (int r = r0 + lr; r < r1 && lr < G; r += G) {
+                const uint8_t *p = simg + (size_t)(y1 + r) * row_stride + (size_t)(x1 + gx) * 3;
+                uint32_t wd[6];
+                load_realigned<7>(p, buf_end, wd);
+                float v[3][PX];
+                unpack8(wd, v);
+                colour(v);
+                store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, cnt, v, false);
+            }
         }
     }
 }
 
-template <int KIND>
+template <int KIND, bool FAST>
 static KernelFn pick(int dtype, int layout) {
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NCHW, KIND>;
-            case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NCHW, KIND>;
-            default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NCHW, KIND>;
+            case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NCHW, KIND, FAST>;
+            case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NCHW, KIND, FAST>;
+            default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NCHW, KIND, FAST>;
         }
     }
     switch (dtype) {
-        case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NHWC, KIND>;
-        case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NHWC, KIND>;
-        default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NHWC, KIND>;
+        case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NHWC, KIND, FAST>;
+        case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NHWC, KIND, FAST>;
+        default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NHWC, KIND, FAST>;
     }
 }
 
-KernelFn select_color_kernel(int kind, int dtype, int layout, const char **name) {
+KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name) {
     *name = "rmx_color_kernel";
-    return kind == COLOR_TWIST ? pick<COLOR_TWIST>(dtype, layout) : pick<COLOR_LINEAR>(dtype, layout);
+    if (fast) return kind == COLOR_TWIST ? pick<COLOR_TWIST, true>(dtype, layout) : pick<COLOR_LINEAR, true>(dtype, layout);
+    return kind == COLOR_TWIST ? pick<COLOR_TWIST, false>(dtype, layout) : pick<COLOR_LINEAR, false>(dtype, layout);
 }
 
 }  // namespace rmx
