@@ -272,6 +272,7 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.aux0 = op->aux0;
     a.aux1 = op->aux1;
     if (((uintptr_t)src) & 3u) return fail(RMX_ERR_INVALID, "the source batch must start at a 4-byte aligned address");
+    if ((op->kind == OP_WARP_AFFINE || op->kind == OP_ROTATE) && (((uintptr_t)dst) & 15u)) a.aux1 = 0;  // packed stores need an aligned base
     // the fast specialisation wants 16-byte aligned batch bases (rows of both sides are then aligned too)
     const bool fast = op->fn_fast && (((uintptr_t)dst) & 15u) == 0 && (!op->fast_needs_src16 || (((uintptr_t)src) & 15u) == 0);
     int wpb = op->waves_per_block;
@@ -425,10 +426,12 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         int ring_rows = 2;
         while (ring_rows < ky + 1) ring_rows *= 2;
         const int src_cols = std::min<int>((int)op->src.w, (int)std::ceil(tile_w * (double)max_rx) + kx_cap + 4);
-        const int src_pitch = ((src_cols + 3) / 4) * 4 + 8;
-        // LDS slice: coef[kx_cap][128] | ring[ring_rows][3][128] | srcrow[src_pitch]
-        size_t words = (size_t)kx_cap * tile_w + (size_t)ring_rows * 3 * tile_w + src_pitch;
+        const int src_pitch = ((src_cols + 3) / 4) * 4 + 8 + 2 * ((kx_cap + 3) / 4 * 4);  // + room for the repeated border columns
+        // LDS slice: coef[kx_cap][128] (only above 8 taps) | ring[ring_rows][3][128] | srcrow[3][src_pitch]
+        size_t words = (size_t)(kx_cap > 8 ? kx_cap : 0) * tile_w + (size_t)ring_rows * 3 * tile_w + 3 * (size_t)src_pitch;  // 3 = rows per staging batch
         op->lds_per_wave = (int)((words * 4 + 15) / 16 * 16);
+        if ((uint64_t)op->src.h * op->src.w * 3 >= (1ull << 32) || op->src.w * 3ull >= (1ull << 23) || op->src.h >= (1u << 23))
+            return fail(RMX_ERR_UNSUPPORTED, "triangular resize: a source sample of %u x %u pixels is beyond the kernel's 32-bit offsets", op->src.w, op->src.h);
         if (op->lds_per_wave > op->ctx->max_lds_per_block || kx_cap > 0xffff)
             return fail(RMX_ERR_UNSUPPORTED, "triangular resize with scale %.1f x %.1f needs %d bytes of LDS per wave", max_rx, max_ry, op->lds_per_wave);
         op->waves_per_block = std::max(1, std::min(4, op->ctx->max_lds_per_block / op->lds_per_wave));
@@ -436,6 +439,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         const int xtiles = (max_dw + tile_w - 1) / tile_w;
         op->aux1 = xtiles;
         op->strip_rows = 12;
+        if (const char *e = getenv("RMX_EXP_TRI_ROWS")) op->strip_rows = std::max(1, atoi(e));
         op->aux0 = op->strip_rows;
         const int ystrips = (max_dh + op->strip_rows - 1) / op->strip_rows;
         op->strips = xtiles * ystrips;
@@ -812,7 +816,10 @@ static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, con
     const int tiles_x = (max_dw + 31) / 32, tiles_y = (max_dh + 15) / 16;
     op->strips = tiles_x * tiles_y;
     op->aux0 = tiles_x;
-    op->aux1 = tiles_y;
+    // aux1: the shapes allow packed 16-byte stores (whole 8-pixel groups, rows a multiple of 8 pixels wide)
+    bool aligned = op->dst.w % 8 == 0;
+    for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
+    op->aux1 = aligned ? 1 : 0;
     return commit_slot(op, slot);
 }
 

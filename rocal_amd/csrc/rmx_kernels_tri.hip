@@ -13,12 +13,15 @@
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
+#include <type_traits>
+
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_tri[];
 
 constexpr int TTW = 128;  // output columns per wave tile
 constexpr int TPX = 2;    // columns per lane
+constexpr int TRB = 3;    // source rows staged per batch (one memory round trip per batch, not per row)
 
 struct TriAxis {
     float ratio, radius, fscale, offset;
@@ -83,10 +86,11 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
 
-    // LDS slice: coef[kx_cap][TTW] | ring[ring_rows][3][TTW] | srcrow[...]
+    // LDS slice: coef[kx_cap][TTW] | ring[ring_rows][3][TTW] | srcrow[TRB][...]
     uint32_t *base = rmx_lds_tri + (size_t)wib * (a.lds_bytes >> 2);
+    // (the coefficient table exists only for kernels of more than 8 taps; shorter ones keep them in registers)
     float *coef = reinterpret_cast<float *>(base);
-    float *ring = coef + kx_cap * TTW;
+    float *ring = coef + (kx_cap > 8 ? kx_cap * TTW : 0);
     uint32_t *srcrow = reinterpret_cast<uint32_t *>(ring + ring_rows * 3 * TTW);
 
     float sc[3], bi[3];
@@ -109,10 +113,22 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
         float sum = 0.0f;
         for (int k = 0; k < kx; k++) {
             float c = tri_coeff(w0, ax.radius, k, ax.fscale);
-            coef[k * TTW + lane * TPX + i] = c;
+            if (kx_cap > 8) coef[k * TTW + lane * TPX + i] = c;
             sum += c;
         }
         colsum[i] = (sum == 0.0f) ? 1.0f : sum;
+    }
+    // register copies of the coefficients for the short-kernel path of the horizontal pass
+    const bool short_taps = kx_cap <= 8;  // kx <= kx_cap
+    float creg[TPX][8];
+#pragma unroll
+    for (int i = 0; i < TPX; i++) {
+        int u = pcx + min(t0 + i, dw - 1);
+        float w0;
+        int loc;
+        tri_loc(ax, u, (float)xlo, loc, w0);
+#pragma unroll
+        for (int k = 0; k < 8; k++) creg[i][k] = (k < kx) ? tri_coeff(w0, ax.radius, k, ax.fscale) : 0.0f;
     }
     // tile-wide staged source column range (wave-uniform)
     int l_first, l_last;
@@ -124,6 +140,11 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
     const int cs = max(min(l_first, xhi), xlo);
     const int ce = max(min(l_last + kx - 1, xhi), xlo);
     const int items = (ce - cs + 4) >> 2;
+    // staged row: [lpad: copies of the first column][items*4 pixels from column cs][copies of the last column].
+    // With the border columns repeated in LDS no tap index needs clamping in the horizontal pass.
+    const int nrep_l = max(cs - l_first, 0), nrep_r = max(l_last + kx - 1 - ce, 0);
+    const int lpad = (nrep_l + 3) & ~3;
+    const int spitch = lpad + items * 4 + ((nrep_r + 3) & ~3);  // dwords per staged row
     wave_sync();
 
     int next_row;
@@ -140,58 +161,134 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
         tri_loc(ay, pcy + r, (float)ylo, locy, w0y);
         const int rb = max(min(locy + ky - 1, yhi), ylo);
         // ---- horizontal pass for the source rows that enter the window
-        for (; next_row <= rb; next_row++) {
-            for (int j = lane; j < items; j += RMX_WAVE) {
-                const uint8_t *p = simg + (size_t)next_row * row_stride + (size_t)(cs + 4 * j) * 3;
-                uint32_t w[3];
-                load_realigned<4>(p, buf_end, w);
-                uint4 px;
-                px.x = w[0];
-                px.y = __builtin_amdgcn_alignbyte(w[1], w[0], 3);
-                px.z = __builtin_amdgcn_alignbyte(w[2], w[1], 2);
-                px.w = w[2] >> 8;
-                *reinterpret_cast<uint4 *>(srcrow + 4 * j) = px;
-            }
-            wave_sync();
-            float *slot = ring + (next_row & ring_mask) * 3 * TTW;
+        while (next_row <= rb) {
+            // stage up to TRB rows with one round trip: (row, item) pairs form one flat index space, four
+            // loads per lane are issued back to back before the first is consumed
+            const int nb = min(TRB, rb - next_row + 1);
+            const int total = nb * items;
+            const float inv_items = 1.0f / (float)items;
+            for (int base = 0; base < total; base += 4 * RMX_WAVE) {
+                uint32_t w[4][3];
+                int dsto[4];
+                const uint8_t *pp[4];
+                bool safe = true;
 #pragma unroll
-            for (int i = 0; i < TPX; i++) {
-                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
-                for (int k = 0; k < kx; k++) {
-                    const int ci = max(min(locx[i] + k, xhi), xlo) - cs;
-                    const uint32_t p = srcrow[ci];
-                    const float c = coef[k * TTW + lane * TPX + i];
-                    a0 = __builtin_fmaf(ubyte0(p), c, a0);
-                    a1 = __builtin_fmaf(ubyte1(p), c, a1);
-                    a2 = __builtin_fmaf(ubyte2(p), c, a2);
+                for (int i = 0; i < 4; i++) {
+                    const int idx = min(base + i * RMX_WAVE + lane, total - 1);
+                    const int q = (int)(((float)idx + 0.5f) * inv_items);  // idx / items (exact: see the bilinear kernel)
+                    const int j = idx - q * items;
+                    pp[i] = simg + ((uint32_t)__mul24(next_row + q, (int)row_stride) + (uint32_t)(cs + 4 * j) * 3u);
+                    dsto[i] = q * spitch + lpad + 4 * j;
+                    safe = safe && (pp[i] - ((uintptr_t)pp[i] & 3u) + 16 <= buf_end);
                 }
-                slot[0 * TTW + lane * TPX + i] = a0;
-                slot[1 * TTW + lane * TPX + i] = a1;
-                slot[2 * TTW + lane * TPX + i] = a2;
+                if (safe) {
+                    u32x4_a4 t[4];
+                    uint32_t ph[4];
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        ph[i] = (uint32_t)((uintptr_t)pp[i] & 3u);
+                        t[i] = *reinterpret_cast<const u32x4_a4 *>(pp[i] - ph[i]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; i++) {
+                        w[i][0] = __builtin_amdgcn_alignbyte(t[i].y, t[i].x, ph[i]);
+                        w[i][1] = __builtin_amdgcn_alignbyte(t[i].z, t[i].y, ph[i]);
+                        w[i][2] = __builtin_amdgcn_alignbyte(t[i].w, t[i].z, ph[i]);
+                    }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) load_realigned<4>(pp[i], buf_end, w[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint4 px;
+                    px.x = w[i][0];
+                    px.y = __builtin_amdgcn_alignbyte(w[i][1], w[i][0], 3);
+                    px.z = __builtin_amdgcn_alignbyte(w[i][2], w[i][1], 2);
+                    px.w = w[i][2] >> 8;
+                    if (base + i * RMX_WAVE + lane < total) *reinterpret_cast<uint4 *>(srcrow + dsto[i]) = px;
+                }
             }
             wave_sync();
+            if (nrep_l + nrep_r > 0) {
+                const int per_row = nrep_l + nrep_r;
+                for (int e = lane; e < nb * per_row; e += RMX_WAVE) {
+                    const int q = e / per_row, z = e - q * per_row;
+                    uint32_t *srow = srcrow + q * spitch + lpad;
+                    if (z < nrep_l) srow[-1 - z] = srow[0];
+                    else srow[(ce - cs) + 1 + (z - nrep_l)] = srow[ce - cs];
+                }
+                wave_sync();
+            }
+            for (int q = 0; q < nb; q++) {
+                const uint32_t *srow = srcrow + q * spitch + lpad;
+                float *slot = ring + ((next_row + q) & ring_mask) * 3 * TTW;
+#pragma unroll
+                for (int i = 0; i < TPX; i++) {
+                    float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+                    if (short_taps) {
+                        // up to 8 taps: fixed offsets from one address, coefficients from registers, unrolled
+                        // for 4, 6 or 8 taps. Taps beyond kx carry coefficient 0 (fma(p, 0, a) == a for the
+                        // finite p an unpacked byte always is), so no bound test is needed inside.
+                        const uint32_t *p0 = srow + (locx[i] - cs);
+                        auto run = [&](auto nt) {
+#pragma unroll
+                            for (int k = 0; k < decltype(nt)::value; k++) {
+                                const uint32_t p = p0[k];
+                                a0 = __builtin_fmaf(ubyte0(p), creg[i][k], a0);
+                                a1 = __builtin_fmaf(ubyte1(p), creg[i][k], a1);
+                                a2 = __builtin_fmaf(ubyte2(p), creg[i][k], a2);
+                            }
+                        };
+                        if (kx <= 4) run(std::integral_constant<int, 4>{});
+                        else if (kx <= 6) run(std::integral_constant<int, 6>{});
+                        else run(std::integral_constant<int, 8>{});
+                    } else {
+                        for (int k = 0; k < kx; k++) {
+                            const uint32_t p = srow[locx[i] + k - cs];
+                            const float c = coef[k * TTW + lane * TPX + i];
+                            a0 = __builtin_fmaf(ubyte0(p), c, a0);
+                            a1 = __builtin_fmaf(ubyte1(p), c, a1);
+                            a2 = __builtin_fmaf(ubyte2(p), c, a2);
+                        }
+                    }
+                    slot[0 * TTW + lane * TPX + i] = a0;
+                    slot[1 * TTW + lane * TPX + i] = a1;
+                    slot[2 * TTW + lane * TPX + i] = a2;
+                }
+            }
+            wave_sync();
+            next_row += nb;
         }
         // ---- vertical pass (each lane reads only ring entries it wrote itself)
         if (cnt > 0) {
             float rsum = 0.0f;
             for (int j = 0; j < ky; j++) rsum += tri_coeff(w0y, ay.radius, j, ay.fscale);
             rsum = (rsum == 0.0f) ? 1.0f : rsum;
+            float acc[3][TPX];
+#pragma unroll
+            for (int c = 0; c < 3; c++)
+#pragma unroll
+                for (int i = 0; i < TPX; i++) acc[c][i] = 0.0f;
+            // taps in ascending order; coefficient and ring row are found once per tap for both columns
+            for (int j = 0; j < ky; j++) {
+                const int rr = max(min(locy + j, yhi), ylo);
+                const float *slot = ring + (rr & ring_mask) * 3 * TTW + lane * TPX;
+                const float c = tri_coeff(w0y, ay.radius, j, ay.fscale);
+#pragma unroll
+                for (int i = 0; i < TPX; i++) {
+                    acc[0][i] = __builtin_fmaf(slot[0 * TTW + i], c, acc[0][i]);
+                    acc[1][i] = __builtin_fmaf(slot[1 * TTW + i], c, acc[1][i]);
+                    acc[2][i] = __builtin_fmaf(slot[2 * TTW + i], c, acc[2][i]);
+                }
+            }
             float v[3][TPX];
 #pragma unroll
             for (int i = 0; i < TPX; i++) {
-                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
-                for (int j = 0; j < ky; j++) {
-                    const int rr = max(min(locy + j, yhi), ylo);
-                    const float *slot = ring + (rr & ring_mask) * 3 * TTW + lane * TPX + i;
-                    const float c = tri_coeff(w0y, ay.radius, j, ay.fscale);
-                    a0 = __builtin_fmaf(slot[0 * TTW], c, a0);
-                    a1 = __builtin_fmaf(slot[1 * TTW], c, a1);
-                    a2 = __builtin_fmaf(slot[2 * TTW], c, a2);
-                }
                 const float inv = 1 / (rsum * colsum[i]);
-                v[0][i] = a0 * inv;
-                v[1][i] = a1 * inv;
-                v[2][i] = a2 * inv;
+                v[0][i] = acc[0][i] * inv;
+                v[1][i] = acc[1][i] * inv;
+                v[2][i] = acc[2][i] * inv;
             }
 #pragma unroll
             for (int c = 0; c < 3; c++)

@@ -120,11 +120,14 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
             if (use_lds) {
                 const int cx0 = min(max(ix0 - bx0, 0), bw - 1), cx1 = min(max(ix1 - bx0, 0), bw - 1);
                 const int cy0 = min(max(iy0 - by0, 0), bh - 1), cy1 = min(max(iy1 - by0, 0), bh - 1);
-                tl = lds[cy0 * pitch + cx0];
+                // one multiply for the four taps: the right / lower neighbour is 0 or 1 column / row away
+                const uint32_t *t0p = lds + __mul24(cy0, pitch) + cx0;
+                const int dx = cx1 - cx0, dy = (cy1 - cy0) ? pitch : 0;
+                tl = t0p[0];
                 if constexpr (!NEAREST) {
-                    tr = lds[cy0 * pitch + cx1];
-                    bl = lds[cy1 * pitch + cx0];
-                    br = lds[cy1 * pitch + cx1];
+                    tr = t0p[dx];
+                    bl = t0p[dy];
+                    br = t0p[dy + dx];
                 }
             } else {
                 tl = load_px_global(simg + (size_t)iy0 * row_stride + (size_t)ix0 * 3);
@@ -147,7 +150,15 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
         }
         v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
     }
-    store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
+    // whole group into 16-byte aligned destination rows: packed stores (a.aux1 is set by the host when every
+    // written width and the padded width are multiples of 8 and the destination base is 16-byte aligned)
+    if (a.aux1 && cnt == PX) {
+        PackedGroup<T> packed;
+        pack_group_dir<T, LAYOUT, false>(v, packed);
+        store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
+    } else {
+        store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
+    }
 }
 
 template <bool NEAREST>
