@@ -50,7 +50,17 @@ struct rmx_ctx {
     bool owns_stream = false;
     int num_cus = 256;
     int max_lds_per_block = 65536;
+    // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
+    // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
+    // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
+    int k1_rows = 8, k3_rows = 8, tri_rows = 12, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1;
 };
+
+static int tune_env(const char *name, int def, int lo, int hi) {
+    const char *e = getenv(name);
+    if (!e || !*e) return def;
+    return std::max(lo, std::min(hi, atoi(e)));
+}
 
 struct rmx_op {
     rmx_ctx *ctx = nullptr;
@@ -202,6 +212,13 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
     if (hipGetDeviceProperties(&prop, device) == hipSuccess) {
         ctx->num_cus = prop.multiProcessorCount;
         ctx->max_lds_per_block = (int)prop.sharedMemPerBlock;
+        ctx->k1_rows = tune_env("RMX_TUNE_CMN_ROWS", ctx->k1_rows, 1, 64);
+        ctx->k3_rows = tune_env("RMX_TUNE_COLOR_ROWS", ctx->k3_rows, 1, 64);
+        ctx->tri_rows = tune_env("RMX_TUNE_TRI_ROWS", ctx->tri_rows, 1, 64);
+        ctx->gen_rows = tune_env("RMX_TUNE_RESIZE_ROWS", ctx->gen_rows, 1, 64);
+        ctx->fast_rows = tune_env("RMX_TUNE_FAST_ROWS", ctx->fast_rows, 1, 64);
+        ctx->fast_lds = tune_env("RMX_TUNE_FAST_LDS", ctx->fast_lds, 2048, 48 * 1024);
+        ctx->fast_wpb = tune_env("RMX_TUNE_FAST_WPB", ctx->fast_wpb, 1, 4);
     }
     *out = ctx;
     return RMX_OK;
@@ -281,7 +298,6 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
         a.lds_bytes = op->fast_lds;
         a.aux0 = op->fast_rows;
         wpb = op->fast_wpb;
-        if (const char *e = getenv("RMX_EXP_WPB")) wpb = atoi(e);
     }
     const uint64_t waves = (uint64_t)op->n * (uint64_t)a.strips;
     const uint64_t blocks = (waves + wpb - 1) / wpb;
@@ -330,8 +346,7 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
         max_rows = std::max(max_rows, (int)s.dst_h);
     }
     op->algo_bytes = bytes;
-    int rows = 8;
-    if (const char *e = getenv("RMX_EXP_K1_ROWS")) rows = std::max(1, atoi(e));
+    const int rows = op->ctx->k1_rows;
     plan_streaming(op, max_rows, rows);
     // aligned specialisation: whole 8-pixel groups everywhere and 16-byte aligned destination rows
     bool aligned = op->dst.w % 8 == 0;
@@ -438,8 +453,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         op->tile_w = tile_w;
         const int xtiles = (max_dw + tile_w - 1) / tile_w;
         op->aux1 = xtiles;
-        op->strip_rows = 12;
-        if (const char *e = getenv("RMX_EXP_TRI_ROWS")) op->strip_rows = std::max(1, atoi(e));
+        op->strip_rows = op->ctx->tri_rows;
         op->aux0 = op->strip_rows;
         const int ystrips = (max_dh + op->strip_rows - 1) / op->strip_rows;
         op->strips = xtiles * ystrips;
@@ -507,10 +521,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     // waves (several residency rounds) overlap better than one long-lived wave per slot; the
     // price is one extra window of source rows per strip. 8 rows measured best on MI355X.
     {
-        int rows = 8;
-        if (const char *e = getenv("RMX_EXP_STRIP_ROWS")) rows = atoi(e);
-        if (const char *e = getenv("RMX_EXP_WPB")) op->waves_per_block = atoi(e);
-        if (const char *e = getenv("RMX_EXP_LDS")) op->lds_per_wave = atoi(e);
+        const int rows = op->ctx->gen_rows;
         op->strip_rows = rows;
         op->aux0 = rows;
         op->strips = std::max(1, (max_dh + rows - 1) / rows);
@@ -525,9 +536,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         bool ok = op->src.w * 3u < (1u << 23) && op->src.h < (1u << 23);
         for (int i = 0; i < op->n && ok; i++) ok = (t[i].dst_w % 8 == 0);
         // 4 rows and a 10 KB slice measured best on MI355X (more, shorter-lived wavefronts per CU)
-        int rows = 4, cap = 10 * 1024;
-        if (const char *e = getenv("RMX_EXP_FAST_ROWS")) rows = std::max(1, atoi(e));
-        if (const char *e = getenv("RMX_EXP_FAST_LDS")) cap = atoi(e);
+        const int rows = op->ctx->fast_rows, cap = op->ctx->fast_lds;
         int need_max = 64;
         for (int i = 0; i < op->n && ok; i++) {
             RmxSample &s = t[i];
@@ -571,7 +580,8 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             op->fast_lds = (need_max + 15) / 16 * 16;
             op->fast_rows = rows;
             op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
-            op->fast_wpb = 1;  // a workgroup's LDS is released only when its last wavefront ends: one-wave groups keep the CU full
+            // (default 1: a workgroup's LDS is released only when its last wavefront ends, one-wave groups keep the CU full)
+            op->fast_wpb = std::max(1, std::min(op->ctx->fast_wpb, op->ctx->max_lds_per_block / std::max(1, op->fast_lds)));
             op->fast_needs_src16 = false;  // its loads only need dword alignment
         }
     }
@@ -695,8 +705,7 @@ static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const 
         max_rows = std::max(max_rows, (int)s.dst_h);
     }
     op->algo_bytes = bytes;
-    int rows = 8;
-    if (const char *e = getenv("RMX_EXP_K3_ROWS")) rows = std::max(1, atoi(e));
+    const int rows = op->ctx->k3_rows;
     plan_streaming(op, max_rows, rows);
     // aligned specialisation: whole 8-pixel groups everywhere and 16-byte aligned destination rows
     bool aligned = op->dst.w % 8 == 0;

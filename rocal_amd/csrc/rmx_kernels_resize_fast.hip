@@ -16,8 +16,11 @@
 // The arithmetic is the general kernel's, operation for operation. Wavefronts never wait for each
 // other; latency is hidden by the other wavefronts resident on the CU (the LDS slice is kept small,
 // per sample, by narrowing the x-tile when the source window is large). The kernel is bound by
-// vector-ALU issue (about 40 instructions per destination pixel, 4 cycles each per SIMD), not by
-// memory: instruction count is what every choice above minimises.
+// vector-ALU issue (about 43 instructions per destination pixel; a wavefront issues one every ~5 cycles
+// and a SIMD sustained one every ~6 here), not by memory: instruction count is what every choice above
+// minimises. Two variants that were tried and measured slower: taps kept packed and widened inside
+// v_fma_mix_f32 (bit-exact through the fp16-subnormal trick, fewer instructions, but each costs more
+// issue time), and tighter register budgets for 20-24 wavefronts per CU.
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
