@@ -104,6 +104,13 @@ RMX_API int rmx_create_flip(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_
 RMX_API int rmx_update_flip(rmx_op *op, const uint32_t *src_roi, const uint32_t *horizontal,
                             const uint32_t *vertical);
 
+/* ---- ToTensor: replaces the second normalise/transpose/cast pass MasterGraph::to_tensor runs on a u8 output
+ *      (rocAL/source/pipeline/master_graph.cpp:514-856) and its device kernels Hip_CopyInt8ToNCHW/NHWC
+ *      (rocAL/rocAL_hip/rocal_hip_kernels.cpp:40-308): out[n,k,y,x] = fmaf(in[n,y,x,rev? 2-k : k],
+ *      multiplier[k], offset[k]) over the whole padded image. multiplier and offset hold 3 floats. ---- */
+RMX_API int rmx_create_to_tensor(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, rmx_op **out);
+RMX_API int rmx_update_to_tensor(rmx_op *op, const float *multiplier /*[3]*/, const float *offset /*[3]*/, int reverse_channels);
+
 /* ---- Resize family: replaces vxExtRppResize (node_resize.cpp:56-57, node_crop_resize.cpp:60-61),
  *      vxExtRppResizeCropMirror (node_resize_crop_mirror.cpp:59-60) and
  *      vxExtRppResizeMirrorNormalize (node_resize_mirror_normalize.cpp:90-92).

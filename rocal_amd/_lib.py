@@ -60,6 +60,8 @@ _SIGS = {
     "rmx_update_warp_affine": [_vp, _vp, _vp, _vp, _vp],
     "rmx_create_rotate": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.POINTER(_vp)],
     "rmx_update_rotate": [_vp, _vp, _vp, _vp, _vp],
+    "rmx_create_to_tensor": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.POINTER(_vp)],
+    "rmx_update_to_tensor": [_vp, _vp, _vp, C.c_int],
     "rmx_copy_bytes": [_vp, _vp, _vp, C.c_size_t],
 }
 _RESTYPES = {"rmx_last_error": C.c_char_p, "rmx_version": C.c_char_p, "rmx_ctx_stream": _vp,

@@ -37,7 +37,7 @@ int fail(int code, const char *fmt, ...) {
 
 enum OpKind {
     OP_CMN = 1, OP_CROP, OP_FLIP, OP_RESIZE, OP_COLOR_TWIST, OP_BRIGHTNESS, OP_CONTRAST, OP_HUE,
-    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE
+    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE, OP_TO_TENSOR
 };
 
 constexpr int TABLE_RING = 4;  // updates in flight before the host has to wait on an old upload
@@ -323,7 +323,8 @@ static int create_k1(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const r
     return RMX_OK;
 }
 
-static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const float *bias, const uint32_t *hflip, const uint32_t *vflip) {
+static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const float *bias, const uint32_t *hflip, const uint32_t *vflip,
+                     bool per_sample_scale = true, bool channel_reverse = false) {
     RmxSample *t;
     int slot = next_slot(op, &t);
     if (slot < 0) return RMX_ERR_HIP;
@@ -331,16 +332,23 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
     int max_rows = 1;
     for (int i = 0; i < op->n; i++) {
         RmxSample &s = t[i];
-        int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
-        if (rc) return rc;
+        if (roi) {
+            int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+            if (rc) return rc;
+        } else {  // whole padded image
+            s.src_x = s.src_y = 0;
+            s.src_w = (int32_t)op->src.w;
+            s.src_h = (int32_t)op->src.h;
+        }
         s.dst_w = std::min<int32_t>(s.src_w, (int32_t)op->dst.w);
         s.dst_h = std::min<int32_t>(s.src_h, (int32_t)op->dst.h);
         s.src_w = s.dst_w;
         s.src_h = s.dst_h;
-        s.flags = ((hflip && hflip[i]) ? RMX_S_HFLIP : 0u) | ((vflip && vflip[i]) ? RMX_S_VFLIP : 0u);
+        s.flags = ((hflip && hflip[i]) ? RMX_S_HFLIP : 0u) | ((vflip && vflip[i]) ? RMX_S_VFLIP : 0u) | (channel_reverse ? RMX_S_CHREV : 0u);
         for (int c = 0; c < 3; c++) {
-            s.scale[c] = scale ? scale[i * 3 + c] : 1.0f;
-            s.bias[c] = bias ? bias[i * 3 + c] : 0.0f;
+            const int k = per_sample_scale ? i * 3 + c : c;
+            s.scale[c] = scale ? scale[k] : 1.0f;
+            s.bias[c] = bias ? bias[k] : 0.0f;
         }
         bytes += (uint64_t)s.dst_w * s.dst_h * 3 * (1 + dtype_size(op->dst.dtype));
         max_rows = std::max(max_rows, (int)s.dst_h);
@@ -390,6 +398,16 @@ int rmx_create_flip(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_d
 int rmx_update_flip(rmx_op *op, const uint32_t *src_roi, const uint32_t *horizontal, const uint32_t *vertical) {
     if (!op || op->kind != OP_FLIP) return fail(RMX_ERR_INVALID, "op is not a Flip node");
     return update_k1(op, src_roi, nullptr, nullptr, horizontal, vertical);
+}
+
+int rmx_create_to_tensor(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, rmx_op **out) {
+    return create_k1(ctx, OP_TO_TENSOR, src, dst, RMX_ROI_XYWH, true, out);
+}
+
+int rmx_update_to_tensor(rmx_op *op, const float *multiplier, const float *offset, int reverse_channels) {
+    if (!op || op->kind != OP_TO_TENSOR) return fail(RMX_ERR_INVALID, "op is not a ToTensor node");
+    if (!multiplier || !offset) return fail(RMX_ERR_INVALID, "multiplier and offset (3 floats each) are required");
+    return update_k1(op, nullptr, multiplier, offset, nullptr, nullptr, false, reverse_channels != 0);
 }
 
 /* ------------------------------------------------------------------ K2 family */

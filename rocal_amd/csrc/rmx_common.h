@@ -27,7 +27,7 @@ struct __attribute__((aligned(16))) RmxSample {
 };
 static_assert(sizeof(RmxSample) == 128, "parameter table row must stay 128 bytes");
 
-enum : uint32_t { RMX_S_HFLIP = 1u, RMX_S_VFLIP = 2u };
+enum : uint32_t { RMX_S_HFLIP = 1u, RMX_S_VFLIP = 2u, RMX_S_CHREV = 4u /* output channel k reads source channel 2-k */ };
 
 struct RmxKArgs {
     const uint8_t *src;      // batch base, u8 NHWC

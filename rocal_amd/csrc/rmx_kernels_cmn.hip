@@ -1,5 +1,5 @@
 // K1: crop + horizontal/vertical flip + per-channel FMA + layout transpose + cast, one pass.
-// Serves CropMirrorNormalize, Crop and Flip (u8 NHWC in; f32/f16/u8, NCHW/NHWC out).
+// Serves CropMirrorNormalize, Crop, Flip and ToTensor (u8 NHWC in; f32/f16/u8, NCHW/NHWC out).
 //
 // Scheduling: one wavefront owns a strip of output rows of one sample. Inside a step the
 // wave covers G = 64/L rows at once, L = lanes per row, each lane producing 8 adjacent
@@ -35,6 +35,7 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
     const int r1 = min(r0 + srows, ch);
     const bool hf = (P.flags & RMX_S_HFLIP) != 0;
     const bool vf = (P.flags & RMX_S_VFLIP) != 0;
+    const bool chrev = (P.flags & RMX_S_CHREV) != 0;
     const int x1 = P.src_x, y1 = P.src_y;
 
     const size_t row_stride = (size_t)a.src_w * 3;
@@ -102,6 +103,14 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
                     if (r < r1) {
                         float v[3][PX];
                         unpack8(w[i], v);
+                        if (chrev) {
+#pragma unroll
+                            for (int k = 0; k < PX; k++) {
+                                const float t = v[0][k];
+                                v[0][k] = v[2][k];
+                                v[2][k] = t;
+                            }
+                        }
                         if constexpr (NORM) {
 #pragma unroll
                             for (int c = 0; c < 3; c++)
@@ -122,6 +131,14 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
                 load_realigned<7>(p, buf_end, w);
                 float v[3][PX];
                 unpack8(w, v);
+                if (chrev) {
+#pragma unroll
+                    for (int k = 0; k < PX; k++) {
+                        const float t = v[0][k];
+                        v[0][k] = v[2][k];
+                        v[2][k] = t;
+                    }
+                }
                 if constexpr (NORM) {
 #pragma unroll
                     for (int c = 0; c < 3; c++)

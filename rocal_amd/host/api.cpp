@@ -136,6 +136,28 @@ void *rocalTensorBuffer(RocalTensor t) { return t ? static_cast<Tensor *>(t)->bu
 const unsigned *rocalTensorRoi(RocalTensor t) { return t ? reinterpret_cast<const unsigned *>(static_cast<Tensor *>(t)->info().roi()) : nullptr; }
 size_t rocalTensorDataSize(RocalTensor t) { return t ? static_cast<Tensor *>(t)->info().data_size() : 0; }
 
+/* ------------------------------------------------------------------ output conversion (rocal_api_data_transfer.cpp:30-52) */
+
+RocalStatus rocalToTensor(RocalContext p_context, void *out_ptr, RocalTensorLayout tensor_format, RocalTensorOutputType tensor_output_type,
+                          float multiplier0, float multiplier1, float multiplier2, float offset0, float offset1, float offset2, bool reverse_channels,
+                          RocalOutputMemType output_mem_type, int max_roi_height, int max_roi_width) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        if (tensor_format != ROCAL_NHWC && tensor_format != ROCAL_NCHW) THROW("Supported only for NHWC and NCHW tensor layout")
+        if (tensor_output_type != ROCAL_FP32 && tensor_output_type != ROCAL_FP16) THROW("Supported only for FP32 and FP16 tensor data types")
+        if (output_mem_type != ROCAL_MEMCPY_GPU) THROW("only ROCAL_MEMCPY_GPU is available: this build has no host path")
+        if (max_roi_height < 0 || max_roi_width < 0) THROW("max_roi_height and max_roi_width cannot be negative")
+        context->master_graph->to_tensor(out_ptr, static_cast<RocalTensorlayout>(tensor_format), multiplier0, multiplier1, multiplier2, offset0, offset1,
+                                         offset2, reverse_channels, static_cast<RocalTensorDataType>(tensor_output_type), (unsigned)max_roi_height,
+                                         (unsigned)max_roi_width);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
 /* ------------------------------------------------------------------ parameters */
 
 void rocalSetSeed(unsigned seed) { ParameterFactory::instance()->set_seed(seed); }

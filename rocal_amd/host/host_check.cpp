@@ -196,6 +196,8 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         outs.push_back(rocalResizeCropMirrorFixed(ctx, src, 36, 28, true, 40, 50, rocalCreateIntParameter(1)));
         outs.push_back(rocalBrightnessFixed(ctx, src, 1.2f, 10.0f, true));
         outs.push_back(rocalContrastFixed(ctx, src, 1.3f, 70.0f, true));
+    } else if (scenario == "to_tensor") {
+        outs.push_back(rocalResize(ctx, src, 40, 32, true));
     } else if (scenario == "errors") {
         // every line must fail the way the reference's API does: null tensor / runtime error + a message
         std::vector<float> zero_std{58.0f, 0.0f, 57.0f};
@@ -241,6 +243,22 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
             std::ofstream r(dir + "/roi" + std::to_string(k) + "_b" + std::to_string(b) + ".txt");
             for (unsigned i = 0; i < n; i++) r << roi[4 * i] << " " << roi[4 * i + 1] << " " << roi[4 * i + 2] << " " << roi[4 * i + 3] << "\n";
         }
+    }
+    if (scenario == "to_tensor") {
+        // the u8 output (32 rows of 40) to a planar fp16 tensor with reversed channels, then its top-left
+        // 24x32 corner to an interleaved fp32 tensor; a host destination must be refused
+        void *tt = nullptr;
+        HIPCHK(hipMalloc(&tt, (size_t)n * 3 * 32 * 40 * 4));
+        std::vector<char> out((size_t)n * 3 * 32 * 40 * 2);
+        if (rocalToTensor(ctx, tt, ROCAL_NCHW, ROCAL_FP16, 1 / 58.395f, 1 / 57.12f, 1 / 57.375f, -2.0f, -1.5f, -1.0f, true, ROCAL_MEMCPY_GPU) != ROCAL_OK) return 9;
+        HIPCHK(hipMemcpy(out.data(), tt, out.size(), hipMemcpyDeviceToHost));
+        std::ofstream(dir + "/tt0.bin", std::ios::binary).write(out.data(), out.size());
+        out.resize((size_t)n * 3 * 24 * 32 * 4);
+        if (rocalToTensor(ctx, tt, ROCAL_NHWC, ROCAL_FP32, 0.5f, 0.25f, 2.0f, 1.0f, 0.0f, -3.0f, false, ROCAL_MEMCPY_GPU, 24, 32) != ROCAL_OK) return 9;
+        HIPCHK(hipMemcpy(out.data(), tt, out.size(), hipMemcpyDeviceToHost));
+        std::ofstream(dir + "/tt1.bin", std::ios::binary).write(out.data(), out.size());
+        if (rocalToTensor(ctx, out.data(), ROCAL_NCHW, ROCAL_FP32, 1, 1, 1, 0, 0, 0, false, ROCAL_MEMCPY_HOST) != ROCAL_RUNTIME_ERROR) return 10;
+        (void)hipFree(tt);
     }
     rocalRelease(ctx);
     (void)hipFree(dev);

@@ -170,6 +170,7 @@ std::vector<uint32_t> Node::roi_as_array(const Roi2DCords *roi) const {
 MasterGraph::MasterGraph(size_t batch_size, int gpu_id, void *stream) : _batch_size(batch_size), _graph(std::make_shared<Graph>(gpu_id, stream)) {}
 
 MasterGraph::~MasterGraph() {
+    if (_to_tensor_op) rmx_op_destroy(_to_tensor_op);
     _nodes.clear();
     for (void *p : _owned_buffers) (void)hipFree(p);
 }
@@ -207,4 +208,42 @@ void MasterGraph::run() {
     ParameterFactory::instance()->renew_parameters();
     for (auto &n : _nodes) n->update_parameters();
     _graph->process();
+}
+
+// master_graph.cpp:514-535 (checks) and :612-632 (device branch). The reference walks the read buffers of its
+// ring and launches Hip_CopyInt8ToNHWC/NCHW once per buffer; here the output tensor is one buffer and the
+// conversion is one launch of the library's ToTensor op on the graph's stream, followed by a wait, so that
+// out_ptr is complete when the call returns.
+void MasterGraph::to_tensor(void *out_ptr, RocalTensorlayout format, float multiplier0, float multiplier1, float multiplier2, float offset0,
+                            float offset1, float offset2, bool reverse_channels, RocalTensorDataType output_data_type, unsigned max_roi_height,
+                            unsigned max_roi_width) {
+    if (!_built) THROW("rocalVerify must be called before rocalToTensor")
+    if (_outputs.size() != 1) THROW("Cannot copy, Multiple output tensors present in the list")
+    Tensor *src = _outputs[0];
+    const TensorInfo &info = src->info();
+    if (info.data_type() != RocalTensorDataType::UINT8) THROW("The output tensor is not of UINT8 type")
+    if (info.layout() != RocalTensorlayout::NHWC) THROW("The output tensor is not interleaved RGB")
+    if (!out_ptr) THROW("rocalToTensor needs a device output pointer")
+    if (!src->buffer()) THROW("The output tensor has no buffer yet")
+    rmx_tensor_desc s = info.desc(), d = s;
+    if (max_roi_height == 0 || max_roi_width == 0) {
+        max_roi_height = s.h;
+        max_roi_width = s.w;
+    }
+    if (max_roi_height > s.h || max_roi_width > s.w) THROW("max_roi_height/max_roi_width exceed the output tensor")
+    d.h = max_roi_height;
+    d.w = max_roi_width;
+    d.layout = (int32_t)format;
+    d.dtype = (int32_t)output_data_type;
+    const unsigned key[4] = {(unsigned)d.layout, (unsigned)d.dtype, d.h, d.w};
+    if (!_to_tensor_op || !std::equal(key, key + 4, _to_tensor_key)) {
+        if (_to_tensor_op) rmx_op_destroy(_to_tensor_op);
+        _to_tensor_op = nullptr;
+        if (rmx_create_to_tensor(_graph->get(), &s, &d, &_to_tensor_op) != RMX_OK) THROW("rmx_create_to_tensor: " + std::string(rmx_last_error()))
+        std::copy(key, key + 4, _to_tensor_key);
+    }
+    const float mul[3] = {multiplier0, multiplier1, multiplier2}, add[3] = {offset0, offset1, offset2};
+    if (rmx_update_to_tensor(_to_tensor_op, mul, add, reverse_channels ? 1 : 0) != RMX_OK) THROW("rmx_update_to_tensor: " + std::string(rmx_last_error()))
+    if (rmx_op_launch(_to_tensor_op, src->buffer(), out_ptr) != RMX_OK) THROW("rmx_op_launch: " + std::string(rmx_last_error()))
+    if (rmx_ctx_sync(_graph->get()) != RMX_OK) THROW("rmx_ctx_sync: " + std::string(rmx_last_error()))
 }

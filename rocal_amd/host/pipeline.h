@@ -145,6 +145,9 @@ class MasterGraph {
     }
     void build();
     void run();
+    // master_graph.cpp:514-856: converts the single u8 output tensor into a float tensor in caller memory
+    void to_tensor(void *out_ptr, RocalTensorlayout format, float multiplier0, float multiplier1, float multiplier2, float offset0, float offset1,
+                   float offset2, bool reverse_channels, RocalTensorDataType output_data_type, unsigned max_roi_height, unsigned max_roi_width);
     size_t batch_size() const { return _batch_size; }
     const std::vector<Tensor *> &outputs() const { return _outputs; }
     bool built() const { return _built; }
@@ -157,6 +160,9 @@ class MasterGraph {
     std::vector<Tensor *> _outputs;
     std::vector<void *> _owned_buffers;
     bool _built = false;
+    // the conversion op of to_tensor(), rebuilt when the requested format changes
+    rmx_op *_to_tensor_op = nullptr;
+    unsigned _to_tensor_key[4] = {0, 0, 0, 0};
 };
 
 struct Context {

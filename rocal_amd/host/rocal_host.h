@@ -26,6 +26,7 @@ enum RocalStatus { ROCAL_OK = 0, ROCAL_CONTEXT_INVALID, ROCAL_RUNTIME_ERROR, ROC
 enum RocalProcessMode { ROCAL_PROCESS_GPU = 0, ROCAL_PROCESS_CPU = 1 };
 enum RocalTensorLayout { ROCAL_NHWC = 0, ROCAL_NCHW = 1, ROCAL_NONE = 9 };
 enum RocalTensorOutputType { ROCAL_FP32 = 0, ROCAL_FP16 = 1, ROCAL_UINT8 = 2 };
+enum RocalOutputMemType { ROCAL_MEMCPY_HOST = 0, ROCAL_MEMCPY_GPU = 1, ROCAL_MEMCPY_PINNED = 2 };
 
 /* ---- context (rocal_api.h:83-110). Only ROCAL_PROCESS_GPU exists: there is no CPU path. ---- */
 extern "C" RocalContext ROCAL_API_CALL rocalCreate(size_t batch_size, RocalProcessMode affinity, int gpu_id = 0, size_t cpu_thread_count = 1,
@@ -43,6 +44,12 @@ extern "C" void *ROCAL_API_CALL rocalTensorBuffer(RocalTensor tensor);
 // x,y,w,h per sample
 extern "C" const unsigned *ROCAL_API_CALL rocalTensorRoi(RocalTensor tensor);
 extern "C" size_t ROCAL_API_CALL rocalTensorDataSize(RocalTensor tensor);
+
+/* ---- u8 output -> float tensor (rocal_api_data_transfer.h:45-66). out_ptr is device memory: only ROCAL_MEMCPY_GPU exists. ---- */
+extern "C" RocalStatus ROCAL_API_CALL rocalToTensor(RocalContext rocal_context, void *out_ptr, RocalTensorLayout tensor_format,
+                                                    RocalTensorOutputType tensor_output_type, float multiplier0, float multiplier1, float multiplier2,
+                                                    float offset0, float offset1, float offset2, bool reverse_channels,
+                                                    RocalOutputMemType output_mem_type, int max_roi_height = 0, int max_roi_width = 0);
 
 /* ---- parameters (rocal_api_parameters.h:39-161) ---- */
 extern "C" void ROCAL_API_CALL rocalSetSeed(unsigned seed);

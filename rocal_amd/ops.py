@@ -163,6 +163,22 @@ class Flip(Op):
         self._update("rmx_update_flip", (src_roi, _U), (horizontal, _U), (vertical, _U))
 
 
+class ToTensor(Op):
+    """MasterGraph::to_tensor / Hip_CopyInt8ToNCHW: whole image, per-channel multiplier/offset, optional RGB<->BGR."""
+
+    def __init__(self, ctx, src_desc, dst_desc):
+        self.ctx = ctx
+        self.src_desc, self.dst_desc = src_desc, dst_desc
+        self._h = C.c_void_p()
+        check(_lib.lib().rmx_create_to_tensor(ctx._h, C.byref(src_desc), C.byref(dst_desc), C.byref(self._h)))
+
+    def update(self, multiplier, offset, reverse_channels=False):
+        m, pm = _arr(multiplier, _F)
+        o, po = _arr(offset, _F)
+        assert m.size == 3 and o.size == 3
+        check(_lib.lib().rmx_update_to_tensor(self._h, pm, po, int(bool(reverse_channels))))
+
+
 class Resize(Op):
     _create = "rmx_create_resize"
     _n_pre = 1

@@ -1,0 +1,126 @@
+"""Parity at the full sizes of the five benchmark configurations (the CPU checker needs well under a
+second for each), size-independent properties of the fused resize path, and the corner cases of the
+aligned fast paths (windows that end on the last byte of the batch buffer, degenerate samples)."""
+import numpy as np
+import pytest
+
+import bench
+from oracle import orc
+from rocal_amd import ops, workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(a):
+    return a.view(np.uint8)
+
+
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
+def test_full_size_configuration_is_bit_identical_to_the_oracle(ctx, cfg):
+    op, src, dst, n, cpu = bench.build_case(cfg, ctx)
+    dst.zero_()
+    op.launch(src, dst)
+    ctx.sync()
+    got = dst.cpu().numpy()
+    exp = cpu(n)
+    assert got.shape == exp.shape
+    assert np.array_equal(_bits(got), _bits(exp)), "config %d: %d values differ" % (cfg, int((got != exp).sum()))
+
+
+def test_fast_and_general_resize_kernels_agree_at_full_size(ctx):
+    """A destination that is not 16-byte aligned sends the same batch through the general kernel."""
+    import torch
+    op, src, dst, n, _ = bench.build_case(1, ctx)
+    assert "fast=1" in op.plan
+    op.launch(src, dst)
+    big = torch.zeros(dst.numel() + 8, dtype=dst.dtype, device="cuda")
+    shifted = big[1:1 + dst.numel()].view(dst.shape)  # 2 bytes off: contiguous, unaligned
+    assert shifted.data_ptr() % 16 != 0
+    op.launch(src, shifted)
+    ctx.sync()
+    assert torch.equal(dst.view(torch.int16), shifted.view(torch.int16))
+
+
+def test_mirror_is_an_involution_on_the_fused_path(ctx):
+    import torch
+    n = 64
+    c = wl.config1(n)
+    inv = (1 / wl.STD).astype(np.float32)
+    scale, bias = np.tile(inv, n), np.tile(-(wl.MEAN * inv), n)
+    dw = np.full(n, 224, np.uint32)
+    op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+    src = torch.from_numpy(c["img"]).cuda()
+    outs = []
+    for mirror in (c["mirror"], 1 - c["mirror"]):
+        op.update_cmn(c["roi"], dw, dw, scale, bias, mirror.astype(np.uint32))
+        out = op.alloc_output()
+        op.launch(src, out)
+        ctx.sync()
+        outs.append(out)
+    assert torch.equal(outs[0].view(torch.int16), torch.flip(outs[1], dims=[3]).view(torch.int16))
+
+
+def test_windows_that_end_on_the_last_bytes_of_the_batch(ctx):
+    """The last sample's window reaches the last pixel of the buffer: the wide loads of the aligned
+    kernels must fall back to their bounds-checked loaders there (and nowhere read past the end)."""
+    import torch
+    rng = np.random.default_rng(9)
+    n, H, W = 3, 37, 53
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    # an exact-size allocation: nothing behind the last pixel belongs to the tensor
+    src = torch.from_numpy(img.reshape(-1).copy()).cuda()
+    roi = np.array([[5, 3, 48, 34], [0, 0, 53, 37], [21, 13, 32, 24]], np.uint32)  # the last two end at (52, 36)
+    dw, dh = np.array([40, 64, 24], np.uint32), np.array([32, 48, 16], np.uint32)
+    inv = (1 / wl.STD).astype(np.float32)
+    scale, bias = np.tile(inv, n), np.tile(-(wl.MEAN * inv), n)
+    mirror = np.array([1, 0, 1], np.uint32)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 48, 64, ops.NCHW, ops.FP16), ops.LINEAR)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert "fast=1" in op.plan
+    out = op.alloc_output()
+    op.launch(src.view(n, H, W, 3), out)
+    ctx.sync()
+    exp = orc.resize(img, roi, dw, dh, 48, 64, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=orc.NCHW, dtype=orc.FP16)
+    assert np.array_equal(_bits(out.cpu().numpy()), _bits(exp))
+    # CropMirrorNormalize and ColorTwist on windows ending at the last pixel (widths multiples of 8: aligned variants)
+    crop = np.array([[5, 5, 48, 32], [13, 0, 40, 37], [29, 21, 24, 16]], np.uint32)
+    cmn = ops.CropMirrorNormalize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 40, 48, ops.NCHW, ops.FP32))
+    cmn.update(crop, scale, bias, mirror)
+    assert "fast=1" in cmn.plan
+    o2 = cmn.alloc_output()
+    cmn.launch(src.view(n, H, W, 3), o2)
+    ctx.sync()
+    e2 = orc.crop_mirror_normalize(img, crop, scale, bias, mirror, 40, 48, orc.NCHW, orc.FP32)
+    assert np.array_equal(_bits(o2.cpu().numpy()), _bits(e2))
+    tw = ops.ColorTwist(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 40, 48, ops.NHWC, ops.UINT8))
+    one = lambda v: np.full(n, v, np.float32)
+    tw.update(crop, one(1.3), one(7.0), one(40.0), one(1.4))
+    o3 = tw.alloc_output()
+    tw.launch(src.view(n, H, W, 3), o3)
+    ctx.sync()
+    sub = np.zeros((n, 40, 48, 3), np.uint8)
+    full = orc.color_twist(img, np.array([[0, 0, W, H]] * n, np.uint32), one(1.3), one(7.0), one(40.0), one(1.4))
+    for i, (x, y, w, h) in enumerate(crop):
+        sub[i, :h, :w] = full[i, y:y + h, x:x + w]
+    assert np.array_equal(o3.cpu().numpy(), sub)
+
+
+def test_degenerate_samples(ctx):
+    """A 1x1 source, a sample with an empty destination (skipped, output untouched) and a 1-row source."""
+    import torch
+    n, H, W = 3, 16, 24
+    img = np.zeros((n, H, W, 3), np.uint8)
+    img[0, 0, 0] = (10, 200, 77)
+    img[2, 0, :, :] = np.arange(W)[:, None] * 3
+    roi = np.array([[0, 0, 1, 1], [0, 0, 8, 8], [0, 0, 24, 1]], np.uint32)
+    dw, dh = np.array([8, 0, 16], np.uint32), np.array([8, 8, 8], np.uint32)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 8, 16, ops.NHWC, ops.UINT8), ops.LINEAR)
+    op.update(roi, dw, dh)
+    out = op.alloc_output(fill=9)
+    op.launch(torch.from_numpy(img).cuda(), out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    exp = orc.resize(img, roi, dw, dh, 8, 16, interp=orc.LINEAR)
+    assert (got[0, :8, :8] == np.array([10, 200, 77], np.uint8)).all()  # a 1x1 source is a constant image
+    assert (got[1] == 9).all()                                            # nothing is written for an empty destination
+    assert np.array_equal(got[0, :8, :8], exp[0, :8, :8]) and np.array_equal(got[2, :8, :16], exp[2, :8, :16])

@@ -162,3 +162,52 @@ def test_hip_path_reproduces_golden_vectors(ctx):
     size = (np.full(n, W, np.uint32), np.full(n, H, np.uint32))
     same(run(ops.Rotate(ctx, sd, sd, ops.LINEAR), full, one(45.0), *size), g["rotate45"], "rotate")
     same(run(ops.WarpAffine(ctx, sd, sd, ops.LINEAR), full, g["warp_rocal_params"], *size), g["warp_affine"], "warp affine")
+
+
+@pytest.mark.parametrize("nchw,fp16,reverse", [(1, 0, 0), (1, 1, 1), (0, 0, 0), (0, 0, 1), (1, 1, 0)])
+def test_hip_to_tensor_matches_reference_hip_kernel(ctx, ref, nchw, fp16, reverse):
+    """The ToTensor op of the library against the reference's own device kernel for the same step
+    (rocal_hip_kernels.cpp:40-308), bit for bit, and against the oracle. The interleaved fp16 variant
+    of the reference is left out: it addresses destination rows at y*W + 3x (rocal_hip_kernels.cpp:112),
+    so its rows overwrite one another; that combination is checked against the oracle below."""
+    import torch
+    rng = np.random.default_rng(34)
+    n, H, W = 4, 40, 56
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    mul = np.array([1 / 58.395, 1 / 57.12, 1 / 57.375], np.float32)
+    add = np.array([-123.675 / 58.395, -116.28 / 57.12, -103.53 / 57.375], np.float32)
+    src = torch.from_numpy(img).cuda()
+    layout, dtype = (ops.NCHW if nchw else ops.NHWC), (ops.FP16 if fp16 else ops.FP32)
+    op = ops.ToTensor(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, H, W, layout, dtype))
+    op.update(mul, add, reverse_channels=bool(reverse))
+    out = op.alloc_output()
+    op.launch(src, out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    dst = torch.zeros(n * 3 * H * W, dtype=torch.float16 if fp16 else torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    rc = ref.ref_copy_int8_to_tensor(None, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), nchw, n, 3, H, W,
+                                     mul.ctypes.data_as(C.c_void_p), add.ctypes.data_as(C.c_void_p), reverse, fp16)
+    assert rc == 0
+    theirs = dst.cpu().numpy().reshape(got.shape)
+    bits = np.uint16 if fp16 else np.uint32
+    assert np.array_equal(got.view(bits), theirs.view(bits))
+    exp = orc.to_tensor(img, mul, add, reverse_channels=bool(reverse), layout=orc.NCHW if nchw else orc.NHWC, dtype=orc.FP16 if fp16 else orc.FP32)
+    assert np.array_equal(got.view(bits), exp.view(bits))
+
+
+@pytest.mark.parametrize("reverse", [0, 1])
+def test_hip_to_tensor_interleaved_fp16_matches_oracle(ctx, reverse):
+    import torch
+    rng = np.random.default_rng(35)
+    n, H, W = 3, 21, 43   # odd width: the byte-wise loaders, not the aligned variant
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    mul = np.array([1 / 255.0, 0.5, 2.0], np.float32)
+    add = np.array([0.0, -1.0, 0.25], np.float32)
+    op = ops.ToTensor(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, H, W, ops.NHWC, ops.FP16))
+    op.update(mul, add, reverse_channels=bool(reverse))
+    out = op.alloc_output()
+    op.launch(torch.from_numpy(img).cuda(), out)
+    ctx.sync()
+    exp = orc.to_tensor(img, mul, add, reverse_channels=bool(reverse), layout=orc.NHWC, dtype=orc.FP16)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), exp.view(np.uint16))

@@ -158,6 +158,22 @@ def test_crop_variants_and_point_ops(tmp_path):
     _same(o[4][0], orc.contrast(img, _roi(), one(1.3), one(70.0)), "contrast")
 
 
+def test_to_tensor_of_the_u8_output(tmp_path):
+    """rocalToTensor (rocal_api_data_transfer.cpp:30-52 -> MasterGraph::to_tensor): planar fp16 with reversed
+    channels of the whole output, then an interleaved fp32 tensor of its top-left max_roi corner."""
+    img, outs, _ = _run("to_tensor", tmp_path, 1, [(np.uint8, (N, 32, 40, 3))])
+    dw, dh = np.full(N, 40, np.uint32), np.full(N, 32, np.uint32)
+    a = orc.resize(img, _roi(), dw, dh, 32, 40, interp=orc.LINEAR)
+    _same(outs[1][0][0], a, "resized u8 output")
+    f32 = lambda *v: np.array(v, np.float32)
+    t0 = np.fromfile(tmp_path / "tt0.bin", dtype=np.float16).reshape(N, 3, 32, 40)
+    _same(t0, orc.to_tensor(a, f32(1 / f32(58.395)[0], 1 / f32(57.12)[0], 1 / f32(57.375)[0]), f32(-2.0, -1.5, -1.0), reverse_channels=True,
+                            layout=orc.NCHW, dtype=orc.FP16), "planar fp16 tensor")
+    t1 = np.fromfile(tmp_path / "tt1.bin", dtype=np.float32).reshape(N, 24, 32, 3)
+    _same(t1, orc.to_tensor(np.ascontiguousarray(a[:, :24, :32]), f32(0.5, 0.25, 2.0), f32(1.0, 0.0, -3.0), layout=orc.NHWC, dtype=orc.FP32),
+          "interleaved fp32 tensor of the 24x32 corner")
+
+
 def test_api_errors_follow_the_reference(tmp_path):
     _image().tofile(tmp_path / "input.bin")
     with open(tmp_path / "meta.txt", "w") as f:
