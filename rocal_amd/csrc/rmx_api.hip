@@ -53,7 +53,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 8, k3_rows = 8, tri_rows = 12, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1;
+    int k1_rows = 8, k3_rows = 8, tri_rows = 12, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, tri_wpb = 4, tri_ring = 0;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -219,6 +219,8 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->fast_rows = tune_env("RMX_TUNE_FAST_ROWS", ctx->fast_rows, 1, 64);
         ctx->fast_lds = tune_env("RMX_TUNE_FAST_LDS", ctx->fast_lds, 2048, 48 * 1024);
         ctx->fast_wpb = tune_env("RMX_TUNE_FAST_WPB", ctx->fast_wpb, 1, 4);
+        ctx->tri_wpb = tune_env("RMX_TUNE_TRI_WPB", ctx->tri_wpb, 1, 4);
+        ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
     }
     *out = ctx;
     return RMX_OK;
@@ -467,7 +469,38 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             return fail(RMX_ERR_UNSUPPORTED, "triangular resize: a source sample of %u x %u pixels is beyond the kernel's 32-bit offsets", op->src.w, op->src.h);
         if (op->lds_per_wave > op->ctx->max_lds_per_block || kx_cap > 0xffff)
             return fail(RMX_ERR_UNSUPPORTED, "triangular resize with scale %.1f x %.1f needs %d bytes of LDS per wave", max_rx, max_ry, op->lds_per_wave);
-        op->waves_per_block = std::max(1, std::min(4, op->ctx->max_lds_per_block / op->lds_per_wave));
+        // Downscaling variant: no ring. Usable when every sample shrinks vertically, has at most 8 horizontal
+        // taps, and no source row is read by output rows more than three apart (four rows are in flight):
+        // first row of r+4 strictly below the last row of r, evaluated with the kernel's own fp32 law.
+        bool down = kx_cap <= 8 && !op->ctx->tri_ring;
+        for (int i = 0; i < op->n && down; i++) {
+            const RmxSample &s = t[i];
+            if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+            if (!(s.ry >= 1.0f)) {
+                down = false;
+                break;
+            }
+            const float radius = s.ry > 1.0f ? s.ry : 1.0f;
+            const float offset = (s.ry - 1) * 0.5f - radius;
+            const int ksz = (int)std::ceil(radius * 2);
+            const int ylo = s.src_y, yhi = s.src_y + s.src_h - 1;
+            auto loc_of = [&](int r) {
+                float raw = (float)(s.pc_y + r) * s.ry;
+                raw = raw + offset;
+                raw = raw + (float)ylo;
+                return (int)std::ceil(raw);
+            };
+            for (int r = 0; r + 4 < s.dst_h && down; r++) {
+                const int last = std::max(std::min(loc_of(r) + ksz - 1, yhi), ylo);
+                const int first = std::max(std::min(loc_of(r + 4), yhi), ylo);
+                down = first > last;
+            }
+        }
+        if (down) {
+            op->fn = rmx::select_resize_tri_down_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
+            op->lds_per_wave = (int)((3 * (size_t)src_pitch * 4 + 15) / 16 * 16);  // the staged source rows only
+        }
+        op->waves_per_block = std::max(1, std::min(op->ctx->tri_wpb, op->ctx->max_lds_per_block / op->lds_per_wave));
         op->tile_w = tile_w;
         const int xtiles = (max_dw + tile_w - 1) / tile_w;
         op->aux1 = xtiles;

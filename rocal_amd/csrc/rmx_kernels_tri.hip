@@ -305,6 +305,256 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
     }
 }
 
+// Downscaling variant (vertical ratio >= 1, at most 8 horizontal taps): the vertical pass keeps no ring of
+// filtered rows. Source rows are filtered horizontally in ascending order and each filtered row is added,
+// straight from registers, to the output rows whose windows contain it; at a ratio >= 1 a source row belongs
+// to the windows of at most four consecutive output rows (the host checks this per sample), so four sets of
+// accumulators in a shift register are enough. Every output row still receives its taps in ascending order
+// with the same coefficients, so the result is bit-identical to the ring kernel's, and the LDS slice shrinks
+// to the staged source rows. A lane owns columns lane and lane + 64 of the tile: neighbouring lanes read
+// source pixels `ratio` dwords apart, half the bank stride of adjacent column pairs.
+constexpr int TDM = 4;  // output rows in flight
+
+template <typename T, int LAYOUT, bool NORM, bool QUANT>
+__global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
+    const int lane = threadIdx.x & (RMX_WAVE - 1);
+    const int wib = threadIdx.x / RMX_WAVE;
+    const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
+    uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
+    wave = __builtin_amdgcn_readfirstlane(wave);
+    if (wave >= nwaves) return;
+    const int s = (int)(wave / (uint32_t)a.strips);
+    const int part = (int)(wave % (uint32_t)a.strips);
+    const int tiles_x = a.aux1;
+    const int strip = part / tiles_x, tx = part - strip * tiles_x;
+    // the whole table row in one round trip
+    const RmxSample P = a.table[s];
+    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.fsx));
+
+    const int dw = P.dst_w, dh = P.dst_h;
+    const int srows = a.aux0;
+    const int r0 = strip * srows, xt = tx * TTW;
+    if (r0 >= dh || xt >= dw) return;
+    const int r1 = min(r0 + srows, dh);
+    const int tw = min(TTW, dw - xt);
+    const bool hf = (P.flags & RMX_S_HFLIP) != 0;
+    const int xlo = P.src_x, ylo = P.src_y;
+    const int xhi = xlo + P.src_w - 1, yhi = ylo + P.src_h - 1;
+    const int pcx = P.pc_x, pcy = P.pc_y;
+    const TriAxis ax = tri_axis(P.rx, P.fsx), ay = tri_axis(P.ry, P.fsy);
+    const int kx = ax.ksize, ky = ay.ksize;
+
+    const size_t row_stride = (size_t)a.src_w * 3;
+    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    const uint8_t *buf_end = a.src + a.src_bytes;
+    T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
+    uint32_t *srcrow = rmx_lds_tri + (size_t)wib * (a.lds_bytes >> 2);
+
+    float sc[3], bi[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        sc[c] = P.scale[c];
+        bi[c] = P.bias[c];
+    }
+
+    // ---- per-lane columns: taps, coefficients (registers), column sums
+    int locx[TPX];
+    bool col_on[TPX];
+    float colsum[TPX], creg[TPX][8];
+#pragma unroll
+    for (int i = 0; i < TPX; i++) {
+        const int col = xt + lane + RMX_WAVE * i;
+        col_on[i] = col < dw;
+        const int u = pcx + min(col, dw - 1);
+        float w0;
+        tri_loc(ax, u, (float)xlo, locx[i], w0);
+        float sum = 0.0f;
+        for (int k = 0; k < kx; k++) sum += tri_coeff(w0, ax.radius, k, ax.fscale);
+        colsum[i] = (sum == 0.0f) ? 1.0f : sum;
+#pragma unroll
+        for (int k = 0; k < 8; k++) creg[i][k] = (k < kx) ? tri_coeff(w0, ax.radius, k, ax.fscale) : 0.0f;
+    }
+    // tile-wide staged source column range (wave-uniform)
+    int l_first, l_last;
+    {
+        float w0;
+        tri_loc(ax, pcx + xt, (float)xlo, l_first, w0);
+        tri_loc(ax, pcx + xt + tw - 1, (float)xlo, l_last, w0);
+    }
+    const int cs = max(min(l_first, xhi), xlo);
+    const int ce = max(min(l_last + kx - 1, xhi), xlo);
+    const int items = (ce - cs + 4) >> 2;
+    // staged row: [lpad: copies of the first column][items*4 pixels from column cs][copies of the last column]
+    const int nrep_l = max(cs - l_first, 0), nrep_r = max(l_last + kx - 1 - ce, 0);
+    const int lpad = (nrep_l + 3) & ~3;
+    const int spitch = lpad + items * 4 + ((nrep_r + 3) & ~3);  // dwords per staged row
+
+    // ---- output rows in flight: rq .. rq+TDM-1 (wave-uniform state), slot 0 is the oldest
+    int rq = r0;
+    int qloc[TDM];
+    float qw0[TDM];
+    float acc[TDM][3][TPX];
+#pragma unroll
+    for (int m = 0; m < TDM; m++) {
+        tri_loc(ay, pcy + min(rq + m, r1 - 1), (float)ylo, qloc[m], qw0[m]);
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+#pragma unroll
+            for (int i = 0; i < TPX; i++) acc[m][c][i] = 0.0f;
+    }
+    int y_last;
+    {
+        int loc;
+        float w0;
+        tri_loc(ay, pcy + r1 - 1, (float)ylo, loc, w0);
+        y_last = max(min(loc + ky - 1, yhi), ylo);
+    }
+
+    for (int y = max(min(qloc[0], yhi), ylo); y <= y_last;) {
+        // stage up to TRB rows with one round trip: (row, item) pairs form one flat index space, four
+        // loads per lane are issued back to back before the first is consumed
+        const int nb = min(TRB, y_last - y + 1);
+        const int total = nb * items;
+        const float inv_items = 1.0f / (float)items;
+        for (int base = 0; base < total; base += 4 * RMX_WAVE) {
+            uint32_t w[4][3];
+            int dsto[4];
+            const uint8_t *pp[4];
+            bool safe = true;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int idx = min(base + i * RMX_WAVE + lane, total - 1);
+                const int q = (int)(((float)idx + 0.5f) * inv_items);  // idx / items (exact: see the bilinear kernel)
+                const int j = idx - q * items;
+                pp[i] = simg + ((uint32_t)__mul24(y + q, (int)row_stride) + (uint32_t)(cs + 4 * j) * 3u);
+                dsto[i] = q * spitch + lpad + 4 * j;
+                safe = safe && (pp[i] - ((uintptr_t)pp[i] & 3u) + 16 <= buf_end);
+            }
+            if (safe) {
+                u32x4_a4 t[4];
+                uint32_t ph[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    ph[i] = (uint32_t)((uintptr_t)pp[i] & 3u);
+                    t[i] = *reinterpret_cast<const u32x4_a4 *>(pp[i] - ph[i]);
+                }
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    w[i][0] = __builtin_amdgcn_alignbyte(t[i].y, t[i].x, ph[i]);
+                    w[i][1] = __builtin_amdgcn_alignbyte(t[i].z, t[i].y, ph[i]);
+                    w[i][2] = __builtin_amdgcn_alignbyte(t[i].w, t[i].z, ph[i]);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) load_realigned<4>(pp[i], buf_end, w[i]);
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint4 px;
+                px.x = w[i][0];
+                px.y = __builtin_amdgcn_alignbyte(w[i][1], w[i][0], 3);
+                px.z = __builtin_amdgcn_alignbyte(w[i][2], w[i][1], 2);
+                px.w = w[i][2] >> 8;
+                if (base + i * RMX_WAVE + lane < total) *reinterpret_cast<uint4 *>(srcrow + dsto[i]) = px;
+            }
+        }
+        wave_sync();
+        if (nrep_l + nrep_r > 0) {
+            const int per_row = nrep_l + nrep_r;
+            for (int e = lane; e < nb * per_row; e += RMX_WAVE) {
+                const int q = e / per_row, z = e - q * per_row;
+                uint32_t *srow = srcrow + q * spitch + lpad;
+                if (z < nrep_l) srow[-1 - z] = srow[0];
+                else srow[(ce - cs) + 1 + (z - nrep_l)] = srow[ce - cs];
+            }
+            wave_sync();
+        }
+        for (int q = 0; q < nb; q++) {
+            const int yy = y + q;
+            // ---- horizontal pass of source row yy: up to 8 taps at fixed offsets from one address, coefficients
+            // from registers, unrolled for 4, 6 or 8 taps. Taps beyond kx carry coefficient 0 (fma(p, 0, a) == a
+            // for the finite p an unpacked byte always is), so no bound test is needed inside.
+            const uint32_t *srow = srcrow + q * spitch + lpad;
+            float h[3][TPX];
+#pragma unroll
+            for (int i = 0; i < TPX; i++) {
+                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+                const uint32_t *p0 = srow + (locx[i] - cs);
+                auto run = [&](auto nt) {
+#pragma unroll
+                    for (int k = 0; k < decltype(nt)::value; k++) {
+                        const uint32_t p = p0[k];
+                        a0 = __builtin_fmaf(ubyte0(p), creg[i][k], a0);
+                        a1 = __builtin_fmaf(ubyte1(p), creg[i][k], a1);
+                        a2 = __builtin_fmaf(ubyte2(p), creg[i][k], a2);
+                    }
+                };
+                if (kx <= 4) run(std::integral_constant<int, 4>{});
+                else if (kx <= 6) run(std::integral_constant<int, 6>{});
+                else run(std::integral_constant<int, 8>{});
+                h[0][i] = a0;
+                h[1][i] = a1;
+                h[2][i] = a2;
+            }
+            // ---- vertical pass: the taps of the rows in flight that read source row yy (a tap index that
+            // leaves the window reads its first / last row, so the border rows can serve several taps)
+#pragma unroll
+            for (int m = 0; m < TDM; m++) {
+                if (rq + m < r1) {
+                    int jlo = (yy == ylo) ? 0 : yy - qloc[m];
+                    int jhi = (yy == yhi) ? ky - 1 : yy - qloc[m];
+                    jlo = max(jlo, 0);
+                    jhi = min(jhi, ky - 1);
+                    for (int j = jlo; j <= jhi; j++) {
+                        const float c = tri_coeff(qw0[m], ay.radius, j, ay.fscale);
+#pragma unroll
+                        for (int ch = 0; ch < 3; ch++)
+#pragma unroll
+                            for (int i = 0; i < TPX; i++) acc[m][ch][i] = __builtin_fmaf(h[ch][i], c, acc[m][ch][i]);
+                    }
+                }
+            }
+            // ---- rows whose last tap was this source row: normalise, epilogue, store, shift the queue
+            while (rq < r1 && max(min(qloc[0] + ky - 1, yhi), ylo) <= yy) {
+                float rsum = 0.0f;
+                for (int j = 0; j < ky; j++) rsum += tri_coeff(qw0[0], ay.radius, j, ay.fscale);
+                rsum = (rsum == 0.0f) ? 1.0f : rsum;
+#pragma unroll
+                for (int i = 0; i < TPX; i++) {
+                    const float inv = 1 / (rsum * colsum[i]);
+                    float v[3][1];
+#pragma unroll
+                    for (int ch = 0; ch < 3; ch++) {
+                        float t = acc[0][ch][i] * inv;
+                        if constexpr (QUANT) t = round_u8(t);
+                        if constexpr (NORM) t = __builtin_fmaf(t, sc[ch], bi[ch]);
+                        v[ch][0] = t;
+                    }
+                    const int col = xt + lane + RMX_WAVE * i;
+                    store_group<T, LAYOUT, 1>(dimg, a.dst_h, a.dst_w, rq, hf ? (dw - 1 - col) : col, col_on[i] ? 1 : 0, v, false);
+                }
+#pragma unroll
+                for (int m = 0; m + 1 < TDM; m++) {
+                    qloc[m] = qloc[m + 1];
+                    qw0[m] = qw0[m + 1];
+#pragma unroll
+                    for (int ch = 0; ch < 3; ch++)
+#pragma unroll
+                        for (int i = 0; i < TPX; i++) acc[m][ch][i] = acc[m + 1][ch][i];
+                }
+                rq++;
+                tri_loc(ay, pcy + min(rq + TDM - 1, r1 - 1), (float)ylo, qloc[TDM - 1], qw0[TDM - 1]);
+#pragma unroll
+                for (int ch = 0; ch < 3; ch++)
+#pragma unroll
+                    for (int i = 0; i < TPX; i++) acc[TDM - 1][ch][i] = 0.0f;
+            }
+        }
+        wave_sync();  // the next batch overwrites the staged rows
+        y += nb;
+    }
+}
+
 template <typename T, int LAYOUT>
 static KernelFn pick3(bool norm, bool quant) {
     if (norm && quant) return (KernelFn)rmx_resize_tri_kernel<T, LAYOUT, true, true>;
@@ -325,6 +575,29 @@ KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, 
         case RMX_FP32: return pick3<float, RMX_NHWC>(norm, quant);
         case RMX_FP16: return pick3<__half, RMX_NHWC>(norm, quant);
         default: return pick3<uint8_t, RMX_NHWC>(norm, quant);
+    }
+}
+
+template <typename T, int LAYOUT>
+static KernelFn pick3_down(bool norm, bool quant) {
+    if (norm && quant) return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, true, true>;
+    if (norm) return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, true, false>;
+    return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, false, false>;
+}
+
+KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
+    *name = "rmx_resize_tri_down_kernel";
+    if (layout == RMX_NCHW) {
+        switch (dtype) {
+            case RMX_FP32: return pick3_down<float, RMX_NCHW>(norm, quant);
+            case RMX_FP16: return pick3_down<__half, RMX_NCHW>(norm, quant);
+            default: return pick3_down<uint8_t, RMX_NCHW>(norm, quant);
+        }
+    }
+    switch (dtype) {
+        case RMX_FP32: return pick3_down<float, RMX_NHWC>(norm, quant);
+        case RMX_FP16: return pick3_down<__half, RMX_NHWC>(norm, quant);
+        default: return pick3_down<uint8_t, RMX_NHWC>(norm, quant);
     }
 }
 
