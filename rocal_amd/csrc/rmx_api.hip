@@ -53,7 +53,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 8, k3_rows = 8, tri_rows = 12, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, tri_wpb = 4, tri_ring = 0;
+    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, tri_wpb = 1, tri_ring = 0;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -214,7 +214,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->max_lds_per_block = (int)prop.sharedMemPerBlock;
         ctx->k1_rows = tune_env("RMX_TUNE_CMN_ROWS", ctx->k1_rows, 1, 64);
         ctx->k3_rows = tune_env("RMX_TUNE_COLOR_ROWS", ctx->k3_rows, 1, 64);
-        ctx->tri_rows = tune_env("RMX_TUNE_TRI_ROWS", ctx->tri_rows, 1, 64);
+        ctx->tri_rows = tune_env("RMX_TUNE_TRI_ROWS", ctx->tri_rows, 0, 64);  // 0: chosen per batch
         ctx->gen_rows = tune_env("RMX_TUNE_RESIZE_ROWS", ctx->gen_rows, 1, 64);
         ctx->fast_rows = tune_env("RMX_TUNE_FAST_ROWS", ctx->fast_rows, 1, 64);
         ctx->fast_lds = tune_env("RMX_TUNE_FAST_LDS", ctx->fast_lds, 2048, 48 * 1024);
@@ -496,15 +496,48 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 down = first > last;
             }
         }
+        int rows = op->ctx->tri_rows > 0 ? op->ctx->tri_rows : 12;
         if (down) {
             op->fn = rmx::select_resize_tri_down_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
-            op->lds_per_wave = (int)((3 * (size_t)src_pitch * 4 + 15) / 16 * 16);  // the staged source rows only
+            // LDS slice: the rows of one staging round (four 16-byte loads per lane = 4, 2 or 1 rows, by row length)
+            size_t lds = 0;
+            for (int i = 0; i < op->n; i++) {
+                const RmxSample &s = t[i];
+                if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+                const int kxi = (int)std::ceil(2.0f * std::max(s.rx, 1.0f));
+                const int cols = std::min<int>((int)op->src.w, (int)std::ceil(tile_w * (double)std::max(s.rx, 1.0f)) + kxi + 4);
+                const int pitch = ((cols + 3) / 4) * 4 + 8 + 2 * ((kxi + 3) / 4 * 4);
+                const int items = (cols + 3) / 4 + 1;
+                const int rows_per_round = items <= 64 ? 4 : (items <= 128 ? 2 : 1);
+                lds = std::max(lds, (size_t)rows_per_round * pitch * 4);
+            }
+            op->lds_per_wave = (int)((std::max<size_t>(lds, 64) + 15) / 16 * 16);  // the staged source rows only
+            if (op->lds_per_wave > op->ctx->max_lds_per_block)
+                return fail(RMX_ERR_UNSUPPORTED, "triangular resize needs %d bytes of LDS per wave", op->lds_per_wave);
+            // Rows per strip: a strip of R rows filters R*ratio + taps source rows, and the device runs the strips in
+            // rounds of (wavefront slots) at a time; pick the R with the least rounds x rows-per-strip.
+            if (op->ctx->tri_rows == 0) {
+                const int per_cu = std::max(1, std::min(16, (160 * 1024) / op->lds_per_wave));
+                const long slots = (long)op->ctx->num_cus * per_cu;
+                double best_cost = 0.0;
+                for (int r = 4; r <= 64; r++) {
+                    long waves = 0;
+                    for (int i = 0; i < op->n; i++)
+                        if (t[i].dst_w > 0 && t[i].dst_h > 0) waves += (long)((t[i].dst_w + tile_w - 1) / tile_w) * ((t[i].dst_h + r - 1) / r);
+                    const long rounds = std::max(1L, (waves + slots - 1) / slots);
+                    const double cost = (double)rounds * (r * (double)max_ry + ky);
+                    if (best_cost == 0.0 || cost < best_cost) {
+                        best_cost = cost;
+                        rows = r;
+                    }
+                }
+            }
         }
         op->waves_per_block = std::max(1, std::min(op->ctx->tri_wpb, op->ctx->max_lds_per_block / op->lds_per_wave));
         op->tile_w = tile_w;
         const int xtiles = (max_dw + tile_w - 1) / tile_w;
         op->aux1 = xtiles;
-        op->strip_rows = op->ctx->tri_rows;
+        op->strip_rows = rows;
         op->aux0 = op->strip_rows;
         const int ystrips = (max_dh + op->strip_rows - 1) / op->strip_rows;
         op->strips = xtiles * ystrips;

@@ -311,8 +311,8 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
 // to the windows of at most four consecutive output rows (the host checks this per sample), so four sets of
 // accumulators in a shift register are enough. Every output row still receives its taps in ascending order
 // with the same coefficients, so the result is bit-identical to the ring kernel's, and the LDS slice shrinks
-// to the staged source rows. A lane owns columns lane and lane + 64 of the tile: neighbouring lanes read
-// source pixels `ratio` dwords apart, half the bank stride of adjacent column pairs.
+// to the staged source rows of one round of loads. A lane owns columns lane and lane + 64 of the tile:
+// neighbouring lanes read source pixels `ratio` dwords apart, half the bank stride of adjacent column pairs.
 constexpr int TDM = 4;  // output rows in flight
 
 template <typename T, int LAYOUT, bool NORM, bool QUANT>
@@ -357,17 +357,19 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
         bi[c] = P.bias[c];
     }
 
-    // ---- per-lane columns: taps, coefficients (registers), column sums
+    // ---- per-lane columns: taps, coefficients (registers), column sums, destination column (mirrored if asked)
     int locx[TPX];
     bool col_on[TPX];
+    uint32_t xcol[TPX];
     float colsum[TPX], creg[TPX][8];
 #pragma unroll
     for (int i = 0; i < TPX; i++) {
         const int col = xt + lane + RMX_WAVE * i;
         col_on[i] = col < dw;
-        const int u = pcx + min(col, dw - 1);
+        const int colc = min(col, dw - 1);
+        xcol[i] = (uint32_t)(hf ? (dw - 1 - colc) : colc);
         float w0;
-        tri_loc(ax, u, (float)xlo, locx[i], w0);
+        tri_loc(ax, pcx + colc, (float)xlo, locx[i], w0);
         float sum = 0.0f;
         for (int k = 0; k < kx; k++) sum += tri_coeff(w0, ax.radius, k, ax.fscale);
         colsum[i] = (sum == 0.0f) ? 1.0f : sum;
@@ -384,7 +386,8 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
     const int cs = max(min(l_first, xhi), xlo);
     const int ce = max(min(l_last + kx - 1, xhi), xlo);
     const int items = (ce - cs + 4) >> 2;
-    // staged row: [lpad: copies of the first column][items*4 pixels from column cs][copies of the last column]
+    // staged row: [lpad: copies of the first column][items*4 pixels from column cs][copies of the last column].
+    // With the border columns repeated in LDS no tap index needs clamping in the horizontal pass.
     const int nrep_l = max(cs - l_first, 0), nrep_r = max(l_last + kx - 1 - ce, 0);
     const int lpad = (nrep_l + 3) & ~3;
     const int spitch = lpad + items * 4 + ((nrep_r + 3) & ~3);  // dwords per staged row
@@ -409,59 +412,35 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
         tri_loc(ay, pcy + r1 - 1, (float)ylo, loc, w0);
         y_last = max(min(loc + ky - 1, yhi), ylo);
     }
+    const int y_first = max(min(qloc[0], yhi), ylo);
 
-    for (int y = max(min(qloc[0], yhi), ylo); y <= y_last;) {
-        // stage up to TRB rows with one round trip: (row, item) pairs form one flat index space, four
-        // loads per lane are issued back to back before the first is consumed
-        const int nb = min(TRB, y_last - y + 1);
-        const int total = nb * items;
-        const float inv_items = 1.0f / (float)items;
-        for (int base = 0; base < total; base += 4 * RMX_WAVE) {
-            uint32_t w[4][3];
-            int dsto[4];
-            const uint8_t *pp[4];
-            bool safe = true;
+    // ---- staging plan of the tile. A row is `items` four-pixel items; a round is four 16-byte loads per lane:
+    // 4 rows of one slot, 2 rows of two slots or 1 row of up to four slots (a row has at most 3 x 64 items at up
+    // to 8 taps; spare slots repeat the last one). Everything that does not depend on the row is computed here:
+    // the dword-aligned byte offset of the slot's item inside a row, the byte phase (the same for all items of a
+    // lane, they are 12 bytes apart) and the item's place in the staged row.
+    const int spr = (items + RMX_WAVE - 1) / RMX_WAVE;
+    const int sh = spr == 1 ? 0 : (spr == 2 ? 1 : 2);  // log2(slots per row)
+    const int rpr = 4 >> sh;                           // rows per round
+    uint32_t sl_al[4], sl_lds[4];
+    bool sl_on[4];
+    const uint32_t low = ((uint32_t)(cs + 4 * min(lane, items - 1)) * 3u) & 3u;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int idx = min(base + i * RMX_WAVE + lane, total - 1);
-                const int q = (int)(((float)idx + 0.5f) * inv_items);  // idx / items (exact: see the bilinear kernel)
-                const int j = idx - q * items;
-                pp[i] = simg + ((uint32_t)__mul24(y + q, (int)row_stride) + (uint32_t)(cs + 4 * j) * 3u);
-                dsto[i] = q * spitch + lpad + 4 * j;
-                safe = safe && (pp[i] - ((uintptr_t)pp[i] & 3u) + 16 <= buf_end);
-            }
-            if (safe) {
-                u32x4_a4 t[4];
-                uint32_t ph[4];
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    ph[i] = (uint32_t)((uintptr_t)pp[i] & 3u);
-                    t[i] = *reinterpret_cast<const u32x4_a4 *>(pp[i] - ph[i]);
-                }
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    w[i][0] = __builtin_amdgcn_alignbyte(t[i].y, t[i].x, ph[i]);
-                    w[i][1] = __builtin_amdgcn_alignbyte(t[i].z, t[i].y, ph[i]);
-                    w[i][2] = __builtin_amdgcn_alignbyte(t[i].w, t[i].z, ph[i]);
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 4; i++) load_realigned<4>(pp[i], buf_end, w[i]);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                uint4 px;
-                px.x = w[i][0];
-                px.y = __builtin_amdgcn_alignbyte(w[i][1], w[i][0], 3);
-                px.z = __builtin_amdgcn_alignbyte(w[i][2], w[i][1], 2);
-                px.w = w[i][2] >> 8;
-                if (base + i * RMX_WAVE + lane < total) *reinterpret_cast<uint4 *>(srcrow + dsto[i]) = px;
-            }
-        }
-        wave_sync();
+    for (int i = 0; i < 4; i++) {
+        const int k = min(i & ((1 << sh) - 1), spr - 1);
+        const int j = min(lane + RMX_WAVE * k, items - 1);
+        sl_al[i] = ((uint32_t)(cs + 4 * j) * 3u) & ~3u;
+        sl_lds[i] = (uint32_t)(lpad + 4 * j);
+        sl_on[i] = lane + RMX_WAVE * k < items;
+    }
+    // every wide load of this wavefront stays inside the batch buffer (last row, last item, carry and load width)
+    const bool safe = simg + (size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16 <= buf_end;
+
+    // clamp-to-edge columns of the nr staged rows
+    auto replicate = [&](int nr) {
         if (nrep_l + nrep_r > 0) {
             const int per_row = nrep_l + nrep_r;
-            for (int e = lane; e < nb * per_row; e += RMX_WAVE) {
+            for (int e = lane; e < nr * per_row; e += RMX_WAVE) {
                 const int q = e / per_row, z = e - q * per_row;
                 uint32_t *srow = srcrow + q * spitch + lpad;
                 if (z < nrep_l) srow[-1 - z] = srow[0];
@@ -469,90 +448,152 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
             }
             wave_sync();
         }
-        for (int q = 0; q < nb; q++) {
-            const int yy = y + q;
-            // ---- horizontal pass of source row yy: up to 8 taps at fixed offsets from one address, coefficients
-            // from registers, unrolled for 4, 6 or 8 taps. Taps beyond kx carry coefficient 0 (fma(p, 0, a) == a
-            // for the finite p an unpacked byte always is), so no bound test is needed inside.
-            const uint32_t *srow = srcrow + q * spitch + lpad;
-            float h[3][TPX];
+    };
+
+    // staged row q is source row yy: filter it and add it to the output rows in flight. NT = taps of the unrolled
+    // horizontal pass (4, 6 or 8 >= kx): taps beyond kx carry coefficient 0 (fma(p, 0, a) == a for the finite p
+    // an unpacked byte always is), so no bound test is needed inside; all LDS reads go out before the arithmetic.
+    auto process_row = [&](auto nt, int q, int yy) {
+        constexpr int NT = decltype(nt)::value;
+        const uint32_t *srow = srcrow + q * spitch + lpad;
+        uint32_t px[TPX][NT];
 #pragma unroll
-            for (int i = 0; i < TPX; i++) {
-                float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
-                const uint32_t *p0 = srow + (locx[i] - cs);
-                auto run = [&](auto nt) {
+        for (int i = 0; i < TPX; i++) {
+            const uint32_t *p0 = srow + (locx[i] - cs);
 #pragma unroll
-                    for (int k = 0; k < decltype(nt)::value; k++) {
-                        const uint32_t p = p0[k];
-                        a0 = __builtin_fmaf(ubyte0(p), creg[i][k], a0);
-                        a1 = __builtin_fmaf(ubyte1(p), creg[i][k], a1);
-                        a2 = __builtin_fmaf(ubyte2(p), creg[i][k], a2);
-                    }
-                };
-                if (kx <= 4) run(std::integral_constant<int, 4>{});
-                else if (kx <= 6) run(std::integral_constant<int, 6>{});
-                else run(std::integral_constant<int, 8>{});
-                h[0][i] = a0;
-                h[1][i] = a1;
-                h[2][i] = a2;
+            for (int k = 0; k < NT; k++) px[i][k] = p0[k];
+        }
+        float h[3][TPX];
+#pragma unroll
+        for (int i = 0; i < TPX; i++) {
+            float a0 = 0.0f, a1 = 0.0f, a2 = 0.0f;
+#pragma unroll
+            for (int k = 0; k < NT; k++) {
+                a0 = __builtin_fmaf(ubyte0(px[i][k]), creg[i][k], a0);
+                a1 = __builtin_fmaf(ubyte1(px[i][k]), creg[i][k], a1);
+                a2 = __builtin_fmaf(ubyte2(px[i][k]), creg[i][k], a2);
             }
-            // ---- vertical pass: the taps of the rows in flight that read source row yy (a tap index that
-            // leaves the window reads its first / last row, so the border rows can serve several taps)
+            h[0][i] = a0;
+            h[1][i] = a1;
+            h[2][i] = a2;
+        }
+        // ---- vertical pass: the taps of the rows in flight that read source row yy (a tap index that
+        // leaves the window reads its first / last row, so the border rows can serve several taps)
 #pragma unroll
-            for (int m = 0; m < TDM; m++) {
-                if (rq + m < r1) {
-                    int jlo = (yy == ylo) ? 0 : yy - qloc[m];
-                    int jhi = (yy == yhi) ? ky - 1 : yy - qloc[m];
-                    jlo = max(jlo, 0);
-                    jhi = min(jhi, ky - 1);
-                    for (int j = jlo; j <= jhi; j++) {
-                        const float c = tri_coeff(qw0[m], ay.radius, j, ay.fscale);
-#pragma unroll
-                        for (int ch = 0; ch < 3; ch++)
-#pragma unroll
-                            for (int i = 0; i < TPX; i++) acc[m][ch][i] = __builtin_fmaf(h[ch][i], c, acc[m][ch][i]);
-                    }
-                }
-            }
-            // ---- rows whose last tap was this source row: normalise, epilogue, store, shift the queue
-            while (rq < r1 && max(min(qloc[0] + ky - 1, yhi), ylo) <= yy) {
-                float rsum = 0.0f;
-                for (int j = 0; j < ky; j++) rsum += tri_coeff(qw0[0], ay.radius, j, ay.fscale);
-                rsum = (rsum == 0.0f) ? 1.0f : rsum;
-#pragma unroll
-                for (int i = 0; i < TPX; i++) {
-                    const float inv = 1 / (rsum * colsum[i]);
-                    float v[3][1];
-#pragma unroll
-                    for (int ch = 0; ch < 3; ch++) {
-                        float t = acc[0][ch][i] * inv;
-                        if constexpr (QUANT) t = round_u8(t);
-                        if constexpr (NORM) t = __builtin_fmaf(t, sc[ch], bi[ch]);
-                        v[ch][0] = t;
-                    }
-                    const int col = xt + lane + RMX_WAVE * i;
-                    store_group<T, LAYOUT, 1>(dimg, a.dst_h, a.dst_w, rq, hf ? (dw - 1 - col) : col, col_on[i] ? 1 : 0, v, false);
-                }
-#pragma unroll
-                for (int m = 0; m + 1 < TDM; m++) {
-                    qloc[m] = qloc[m + 1];
-                    qw0[m] = qw0[m + 1];
+        for (int m = 0; m < TDM; m++) {
+            if (rq + m < r1) {
+                int jlo = (yy == ylo) ? 0 : yy - qloc[m];
+                int jhi = (yy == yhi) ? ky - 1 : yy - qloc[m];
+                jlo = max(jlo, 0);
+                jhi = min(jhi, ky - 1);
+                for (int j = jlo; j <= jhi; j++) {
+                    const float c = tri_coeff(qw0[m], ay.radius, j, ay.fscale);
 #pragma unroll
                     for (int ch = 0; ch < 3; ch++)
 #pragma unroll
-                        for (int i = 0; i < TPX; i++) acc[m][ch][i] = acc[m + 1][ch][i];
+                        for (int i = 0; i < TPX; i++) acc[m][ch][i] = __builtin_fmaf(h[ch][i], c, acc[m][ch][i]);
                 }
-                rq++;
-                tri_loc(ay, pcy + min(rq + TDM - 1, r1 - 1), (float)ylo, qloc[TDM - 1], qw0[TDM - 1]);
+            }
+        }
+        // ---- rows whose last tap was this source row: normalise, epilogue, store, shift the queue
+        while (rq < r1 && max(min(qloc[0] + ky - 1, yhi), ylo) <= yy) {
+            float rsum = 0.0f;
+            for (int j = 0; j < ky; j++) rsum += tri_coeff(qw0[0], ay.radius, j, ay.fscale);
+            rsum = (rsum == 0.0f) ? 1.0f : rsum;
+#pragma unroll
+            for (int i = 0; i < TPX; i++) {
+                const float inv = 1 / (rsum * colsum[i]);
+#pragma unroll
+                for (int ch = 0; ch < 3; ch++) {
+                    float t = acc[0][ch][i] * inv;
+                    if constexpr (QUANT) t = round_u8(t);
+                    if constexpr (NORM) t = __builtin_fmaf(t, sc[ch], bi[ch]);
+                    // wave-uniform row pointer + the lane's column offset
+                    if constexpr (LAYOUT == RMX_NCHW) {
+                        T *rowp = dimg + ((size_t)ch * a.dst_h + rq) * a.dst_w;
+                        if (col_on[i]) rowp[xcol[i]] = OutCvt<T>::cvt(t);
+                    } else {
+                        T *rowp = dimg + (size_t)rq * a.dst_w * 3 + ch;
+                        if (col_on[i]) rowp[xcol[i] * 3u] = OutCvt<T>::cvt(t);
+                    }
+                }
+            }
+#pragma unroll
+            for (int m = 0; m + 1 < TDM; m++) {
+                qloc[m] = qloc[m + 1];
+                qw0[m] = qw0[m + 1];
 #pragma unroll
                 for (int ch = 0; ch < 3; ch++)
 #pragma unroll
-                    for (int i = 0; i < TPX; i++) acc[TDM - 1][ch][i] = 0.0f;
+                    for (int i = 0; i < TPX; i++) acc[m][ch][i] = acc[m + 1][ch][i];
             }
+            rq++;
+            tri_loc(ay, pcy + min(rq + TDM - 1, r1 - 1), (float)ylo, qloc[TDM - 1], qw0[TDM - 1]);
+#pragma unroll
+            for (int ch = 0; ch < 3; ch++)
+#pragma unroll
+                for (int i = 0; i < TPX; i++) acc[TDM - 1][ch][i] = 0.0f;
         }
-        wave_sync();  // the next batch overwrites the staged rows
-        y += nb;
-    }
+    };
+
+    auto run = [&](auto nt) {
+        if (!safe) {
+            // the wavefront's rows touch the last bytes of the batch buffer: row by row, bounds-checked loads
+            for (int y = y_first; y <= y_last; y++) {
+                for (int j = lane; j < items; j += RMX_WAVE) {
+                    const uint8_t *pp = simg + (size_t)y * row_stride + (size_t)(cs + 4 * j) * 3;
+                    uint32_t w[3];
+                    load_realigned<4>(pp, buf_end, w);
+                    uint4 px;
+                    px.x = w[0];
+                    px.y = __builtin_amdgcn_alignbyte(w[1], w[0], 3);
+                    px.z = __builtin_amdgcn_alignbyte(w[2], w[1], 2);
+                    px.w = w[2] >> 8;
+                    *reinterpret_cast<uint4 *>(srcrow + lpad + 4 * j) = px;
+                }
+                wave_sync();
+                replicate(1);
+                process_row(nt, 0, y);
+                wave_sync();  // the next row overwrites the staged one
+            }
+            return;
+        }
+        // Software pipeline over the rounds: the loads of the next round are issued before the rows of the current
+        // one are filtered and wait in registers, so a round trip to memory runs under the arithmetic of the
+        // previous round. The four loads are straight-line and unconditional (rows beyond the last repeat it).
+        u32x4_a4 t[4];
+        auto issue = [&](int yb, int nr) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int q = min(i >> sh, nr - 1);
+                const uint8_t *rowp = simg + (size_t)(yb + q) * row_stride;  // wave-uniform
+                const uint32_t r = (uint32_t)((uintptr_t)rowp & 3u);
+                t[i] = *reinterpret_cast<const u32x4_a4 *>((rowp - r) + (sl_al[i] + ((low + r) & 4u)));
+            }
+        };
+        issue(y_first, min(rpr, y_last - y_first + 1));
+        for (int y = y_first; y <= y_last;) {
+            const int nr = min(rpr, y_last - y + 1);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int q = min(i >> sh, nr - 1);
+                const uint32_t r = (uint32_t)((uintptr_t)(simg + (size_t)(y + q) * row_stride) & 3u);
+                const uint32_t d[4] = {t[i].x, t[i].y, t[i].z, t[i].w};
+                const uint4 px = expand4(d, (low + r) & 3u);
+                if (sl_on[i]) *reinterpret_cast<uint4 *>(srcrow + (uint32_t)(q * spitch) + sl_lds[i]) = px;
+            }
+            wave_sync();
+            const int yn = y + nr;
+            issue(min(yn, y_last), max(1, min(rpr, y_last - yn + 1)));
+            replicate(nr);
+            for (int q = 0; q < nr; q++) process_row(nt, q, y + q);
+            wave_sync();  // the next round overwrites the staged rows
+            y = yn;
+        }
+    };
+    if (kx <= 4) run(std::integral_constant<int, 4>{});
+    else if (kx <= 6) run(std::integral_constant<int, 6>{});
+    else run(std::integral_constant<int, 8>{});
 }
 
 template <typename T, int LAYOUT>
