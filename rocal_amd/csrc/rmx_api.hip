@@ -515,7 +515,9 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             if (op->lds_per_wave > op->ctx->max_lds_per_block)
                 return fail(RMX_ERR_UNSUPPORTED, "triangular resize needs %d bytes of LDS per wave", op->lds_per_wave);
             // Rows per strip: a strip of R rows filters R*ratio + taps source rows, and the device runs the strips in
-            // rounds of (wavefront slots) at a time; pick the R with the least rounds x rows-per-strip.
+            // rounds of (wavefront slots) at a time; pick the R with the least rounds x rows-per-strip. Measured on
+            // MI355X: a batch of equal strips that march in step runs 10-20 % slower than one whose last strip of each
+            // image is a short one, so an R that leaves a remainder of at most R/2 rows is preferred.
             if (op->ctx->tri_rows == 0) {
                 const int per_cu = std::max(1, std::min(16, (160 * 1024) / op->lds_per_wave));
                 const long slots = (long)op->ctx->num_cus * per_cu;
@@ -525,7 +527,8 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                     for (int i = 0; i < op->n; i++)
                         if (t[i].dst_w > 0 && t[i].dst_h > 0) waves += (long)((t[i].dst_w + tile_w - 1) / tile_w) * ((t[i].dst_h + r - 1) / r);
                     const long rounds = std::max(1L, (waves + slots - 1) / slots);
-                    const double cost = (double)rounds * (r * (double)max_ry + ky);
+                    const int rem = max_dh % r;
+                    const double cost = (double)rounds * (r * (double)max_ry + ky) * ((rem == 0 || 2 * rem > r) ? 1.15 : 1.0);
                     if (best_cost == 0.0 || cost < best_cost) {
                         best_cost = cost;
                         rows = r;

@@ -344,8 +344,11 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
     const TriAxis ax = tri_axis(P.rx, P.fsx), ay = tri_axis(P.ry, P.fsy);
     const int kx = ax.ksize, ky = ay.ksize;
 
-    const size_t row_stride = (size_t)a.src_w * 3;
+    // (a sample is smaller than 4 GiB: the host checks it, so offsets inside a sample are 32-bit)
+    const uint32_t row_stride = (uint32_t)a.src_w * 3u;
     const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
+    const uint8_t *base4 = simg - skew;  // dword-aligned base below the sample
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
     uint32_t *srcrow = rmx_lds_tri + (size_t)wib * (a.lds_bytes >> 2);
@@ -413,6 +416,16 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
         y_last = max(min(loc + ky - 1, yhi), ylo);
     }
     const int y_first = max(min(qloc[0], yhi), ylo);
+    // sum of the vertical coefficients of output row r0 + lane (a strip has at most 64 rows), taps ascending;
+    // the row that completes fetches its sum from the lane that holds it
+    float rsum_v = 0.0f;
+    {
+        int loc;
+        float w0;
+        tri_loc(ay, pcy + min(r0 + lane, r1 - 1), (float)ylo, loc, w0);
+        for (int j = 0; j < ky; j++) rsum_v += tri_coeff(w0, ay.radius, j, ay.fscale);
+        rsum_v = (rsum_v == 0.0f) ? 1.0f : rsum_v;
+    }
 
     // ---- staging plan of the tile. A row is `items` four-pixel items; a round is four 16-byte loads per lane:
     // 4 rows of one slot, 2 rows of two slots or 1 row of up to four slots (a row has at most 3 x 64 items at up
@@ -434,7 +447,7 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
         sl_on[i] = lane + RMX_WAVE * k < items;
     }
     // every wide load of this wavefront stays inside the batch buffer (last row, last item, carry and load width)
-    const bool safe = simg + (size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16 <= buf_end;
+    const bool safe = simg + ((size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16) <= buf_end;
 
     // clamp-to-edge columns of the nr staged rows
     auto replicate = [&](int nr) {
@@ -497,9 +510,7 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
         }
         // ---- rows whose last tap was this source row: normalise, epilogue, store, shift the queue
         while (rq < r1 && max(min(qloc[0] + ky - 1, yhi), ylo) <= yy) {
-            float rsum = 0.0f;
-            for (int j = 0; j < ky; j++) rsum += tri_coeff(qw0[0], ay.radius, j, ay.fscale);
-            rsum = (rsum == 0.0f) ? 1.0f : rsum;
+            const float rsum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rq - r0));
 #pragma unroll
             for (int i = 0; i < TPX; i++) {
                 const float inv = 1 / (rsum * colsum[i]);
@@ -566,9 +577,9 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int q = min(i >> sh, nr - 1);
-                const uint8_t *rowp = simg + (size_t)(yb + q) * row_stride;  // wave-uniform
-                const uint32_t r = (uint32_t)((uintptr_t)rowp & 3u);
-                t[i] = *reinterpret_cast<const u32x4_a4 *>((rowp - r) + (sl_al[i] + ((low + r) & 4u)));
+                const uint32_t ro = (uint32_t)(yb + q) * row_stride + skew;  // wave-uniform: row start from base4
+                const uint32_t r = ro & 3u;
+                t[i] = *reinterpret_cast<const u32x4_a4 *>(base4 + ((ro - r) + sl_al[i] + ((low + r) & 4u)));
             }
         };
         issue(y_first, min(rpr, y_last - y_first + 1));
@@ -577,7 +588,7 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int q = min(i >> sh, nr - 1);
-                const uint32_t r = (uint32_t)((uintptr_t)(simg + (size_t)(y + q) * row_stride) & 3u);
+                const uint32_t r = ((uint32_t)(y + q) * row_stride + skew) & 3u;
                 const uint32_t d[4] = {t[i].x, t[i].y, t[i].z, t[i].w};
                 const uint4 px = expand4(d, (low + r) & 3u);
                 if (sl_on[i]) *reinterpret_cast<uint4 *>(srcrow + (uint32_t)(q * spitch) + sl_lds[i]) = px;
