@@ -53,7 +53,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, tri_wpb = 1, tri_ring = 0;
+    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -220,6 +220,8 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->fast_lds = tune_env("RMX_TUNE_FAST_LDS", ctx->fast_lds, 2048, 48 * 1024);
         ctx->fast_wpb = tune_env("RMX_TUNE_FAST_WPB", ctx->fast_wpb, 1, 4);
         ctx->tri_wpb = tune_env("RMX_TUNE_TRI_WPB", ctx->tri_wpb, 1, 4);
+        ctx->warp_passes = tune_env("RMX_TUNE_WARP_PASSES", ctx->warp_passes, 1, 8);
+        ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
         ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
     }
     *out = ctx;
@@ -291,7 +293,7 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.aux0 = op->aux0;
     a.aux1 = op->aux1;
     if (((uintptr_t)src) & 3u) return fail(RMX_ERR_INVALID, "the source batch must start at a 4-byte aligned address");
-    if ((op->kind == OP_WARP_AFFINE || op->kind == OP_ROTATE) && (((uintptr_t)dst) & 15u)) a.aux1 = 0;  // packed stores need an aligned base
+    if ((op->kind == OP_WARP_AFFINE || op->kind == OP_ROTATE) && (((uintptr_t)dst) & 15u)) a.aux1 &= ~1;  // packed stores need an aligned base
     // the fast specialisation wants 16-byte aligned batch bases (rows of both sides are then aligned too)
     const bool fast = op->fn_fast && (((uintptr_t)dst) & 15u) == 0 && (!op->fast_needs_src16 || (((uintptr_t)src) & 15u) == 0);
     int wpb = op->waves_per_block;
@@ -895,27 +897,31 @@ static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, con
         bytes += (uint64_t)s.src_w * s.src_h * 3 + (uint64_t)s.dst_w * s.dst_h * 3 * dtype_size(op->dst.dtype);
         max_dw = std::max(max_dw, (int)s.dst_w);
         max_dh = std::max(max_dh, (int)s.dst_h);
-        // LDS need of a 32x16 destination tile: bounding box of its image under M, plus margins
-        double bw = 32.0 * std::fabs(s.m[0]) + 16.0 * std::fabs(s.m[1]) + 5.0;
-        double bh = 32.0 * std::fabs(s.m[3]) + 16.0 * std::fabs(s.m[4]) + 5.0;
+        // LDS need of a destination tile (32 x 16*passes): bounding box of its image under M, margins, and the
+        // repeated column and row
+        const double th = 16.0 * op->ctx->warp_passes;
+        double bw = 32.0 * std::fabs(s.m[0]) + th * std::fabs(s.m[1]) + 6.0;
+        double bh = 32.0 * std::fabs(s.m[3]) + th * std::fabs(s.m[4]) + 6.0;
         if (std::isfinite(bw) && std::isfinite(bh)) {
-            bw = std::min(bw, (double)s.src_w);
-            bh = std::min(bh, (double)s.src_h);
+            bw = std::min(bw, (double)s.src_w + 1);
+            bh = std::min(bh, (double)s.src_h + 1);
             worst_box = std::max(worst_box, (std::ceil(bw / 4) * 4 + 4) * bh);
         }
     }
     op->algo_bytes = bytes;
-    const int cap = 16 * 1024;  // per wave; bigger boxes fall back to global gathers inside the kernel
+    const int cap = 16 * 1024;  // per wave (16 loads per lane); bigger boxes fall back to global gathers inside the kernel
     int need = (int)std::min<double>(worst_box * 4, (double)cap);
     op->lds_per_wave = std::max(256, (need + 15) / 16 * 16);
-    op->waves_per_block = 4;
-    const int tiles_x = (max_dw + 31) / 32, tiles_y = (max_dh + 15) / 16;
+    op->waves_per_block = std::max(1, std::min(op->ctx->warp_wpb, op->ctx->max_lds_per_block / op->lds_per_wave));
+    const int passes = op->ctx->warp_passes;
+    const int tiles_x = (max_dw + 31) / 32, tiles_y = (max_dh + 16 * passes - 1) / (16 * passes);
     op->strips = tiles_x * tiles_y;
     op->aux0 = tiles_x;
-    // aux1: the shapes allow packed 16-byte stores (whole 8-pixel groups, rows a multiple of 8 pixels wide)
+    // aux1 bit 0: the shapes allow packed 16-byte stores (whole 8-pixel groups, rows a multiple of 8 pixels wide);
+    // bits 8..: passes of 16 rows per tile
     bool aligned = op->dst.w % 8 == 0;
     for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
-    op->aux1 = aligned ? 1 : 0;
+    op->aux1 = (aligned ? 1 : 0) | (passes << 8);
     return commit_slot(op, slot);
 }
 

@@ -1,23 +1,35 @@
 // K4: inverse-map affine warp (WarpAffine / Rotate), bilinear or nearest, constant-0 outside
 // the source ROI; u8 NHWC in, T/LAYOUT out.
 //
-// A wavefront owns one 32x16 destination tile. The tile's corners are pushed through the
-// affine map to get the source bounding box, which is staged into the wave's private LDS slice
-// (dword per pixel, dword-aligned 128-bit global loads) and then gathered from LDS: source
-// pixels that several destination pixels touch are fetched from HBM/L2 once per tile. When
-// the box does not fit the slice (strong minification) the wave gathers from global memory.
-// Each lane produces 8 adjacent destination pixels of one row and writes them with wide stores.
+// A wavefront owns a destination tile of 32 columns x (16 x passes) rows. The tile's corners are pushed
+// through the affine map to get the source bounding box (every pixel of the tile maps inside it: each
+// step of the coordinate law is monotone in x and in y, also after rounding), which is staged into the
+// wavefront's LDS slice, one dword per pixel, with all loads of the box in flight together; one extra
+// column and row repeat the ROI's last column / row, so the right and lower neighbours of a tap are always
+// at +1 and +pitch. Each lane then produces 8 adjacent destination pixels of one row per pass, branch-free:
+// taps of pixels that fall outside the ROI are read from wherever their (meaningless) address points inside
+// the slice and the result is replaced by 0. When the box does not fit the slice (strong minification) the
+// wavefront gathers from global memory instead.
 #include "rmx_device.h"
 #include "rmx_launch.h"
+
+#include <type_traits>
 
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_warp[];
 
-constexpr int WTW = 32, WTH = 16;  // destination tile: 4 lanes x 8 px wide, 16 rows
+constexpr int WTW = 32, WTH = 16;  // destination tile: 4 lanes x 8 px wide, 16 rows per pass
 
 RMX_DEV uint32_t load_px_global(const uint8_t *p) {
     return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
+}
+
+// floor(x) as an integer in one instruction (saturating; 0 for NaN)
+RMX_DEV int floor_i32(float x) {
+    int r;
+    asm("v_cvt_flr_i32_f32 %0, %1" : "=v"(r) : "v"(x));
+    return r;
 }
 
 template <typename T, int LAYOUT, bool NEAREST>
@@ -25,16 +37,20 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const int wib = threadIdx.x / RMX_WAVE;
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
-    uint32_t wave = xcd_swizzle(blockIdx.x, gridDim.x) * (blockDim.x / RMX_WAVE) + wib;
+    uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
     const int s = (int)(wave / (uint32_t)a.strips);
     const int tile = (int)(wave % (uint32_t)a.strips);
     const int tiles_x = a.aux0;
+    const int passes = a.aux1 >> 8;
+    const bool packed_ok = (a.aux1 & 1) != 0;
     const int ty = tile / tiles_x, tx = tile - ty * tiles_x;
-    const RmxSample &P = a.table[s];
+    // the whole table row in one round trip
+    const RmxSample P = a.table[s];
+    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.flags), "s"(P.m[0]), "s"(P.m[5]));
     const int dw = P.dst_w, dh = P.dst_h;
-    const int X0 = tx * WTW, Y0 = ty * WTH;
+    const int X0 = tx * WTW, Y0 = ty * (WTH * passes);
     if (X0 >= dw || Y0 >= dh) return;
 
     const int xlo = P.src_x, ylo = P.src_y;
@@ -43,14 +59,14 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const float dcx = (float)(dw >> 1), dcy = (float)(dh >> 1);
     const float scx = (float)(xlo + (P.src_w >> 1)), scy = (float)(ylo + (P.src_h >> 1));
 
-    const size_t row_stride = (size_t)a.src_w * 3;
+    const uint32_t row_stride = (uint32_t)a.src_w * 3u;
     const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
     uint32_t *lds = rmx_lds_warp + (size_t)wib * (a.lds_bytes >> 2);
 
     // source bounding box of the tile (wave-uniform), one pixel of margin, clipped to the ROI
-    const int X1 = min(X0 + WTW, dw) - 1, Y1 = min(Y0 + WTH, dh) - 1;
+    const int X1 = min(X0 + WTW, dw) - 1, Y1 = min(Y0 + WTH * passes, dh) - 1;
     float bxmin = 3.0e38f, bxmax = -3.0e38f, bymin = 3.0e38f, bymax = -3.0e38f;
 #pragma unroll
     for (int cy = 0; cy < 2; cy++)
@@ -59,6 +75,10 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
             float xr = (float)(cx ? X1 : X0) - dcx, yr = (float)(cy ? Y1 : Y0) - dcy;
             float sx = __builtin_fmaf(xr, m0, __builtin_fmaf(yr, m1, m2)) + scx;
             float sy = __builtin_fmaf(xr, m3, __builtin_fmaf(yr, m4, m5)) + scy;
+            if constexpr (NEAREST) {
+                sx += 0.5f;
+                sy += 0.5f;
+            }
             bxmin = __builtin_fminf(bxmin, sx); bxmax = __builtin_fmaxf(bxmax, sx);
             bymin = __builtin_fminf(bymin, sy); bymax = __builtin_fmaxf(bymax, sy);
         }
@@ -69,95 +89,172 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const int by0 = max((int)floorf(bymin) - 1, ylo), by1 = min((int)floorf(bymax) + 2, yhi);
     const int bw = bx1 - bx0 + 1, bh = by1 - by0 + 1;
     const bool empty = bw <= 0 || bh <= 0;
-    const int items = (max(bw, 0) + 3) >> 2;
+    // staged box: bw columns + the repeated last one, bh rows + the repeated last one
+    const int items = (max(bw, 0) + 1 + 3) >> 2;
     const int pitch = items * 4;
-    const bool use_lds = !empty && (size_t)bh * pitch * 4 <= (size_t)a.lds_bytes;
+    const int total = (bh + 1) * items;
+    const bool use_lds = !empty && total <= 16 * RMX_WAVE && (size_t)(bh + 1) * pitch * 4 <= (size_t)a.lds_bytes;
 
-    if (use_lds) {
-        int q = 0, j = lane;
-        while (j >= items) { j -= items; q++; }
-        while (q < bh) {
-            const uint8_t *p = simg + (size_t)(by0 + q) * row_stride + (size_t)(bx0 + 4 * j) * 3;
-            uint32_t w[3];
-            load_realigned<4>(p, buf_end, w);
-            uint4 px;
-            px.x = w[0];
-            px.y = __builtin_amdgcn_alignbyte(w[1], w[0], 3);
-            px.z = __builtin_amdgcn_alignbyte(w[2], w[1], 2);
-            px.w = w[2] >> 8;
-            *reinterpret_cast<uint4 *>(lds + q * pitch + 4 * j) = px;
-            j += RMX_WAVE;
-            while (j >= items) { j -= items; q++; }
+    const int lr = lane >> 2, g = lane & 3;
+    const int x0 = X0 + g * PX;
+    const int cnt = min(PX, dw - x0);
+    const float xr0 = (float)x0 - dcx;
+
+    if (!use_lds) {
+        // empty box (every pixel is outside the ROI) or a box too large for the slice: per-pixel gathers from global memory
+        for (int pass = 0; pass < passes; pass++) {
+            const int y = Y0 + pass * WTH + lr;
+            if (y >= dh || cnt <= 0) continue;
+            const float yr = (float)y - dcy;
+            float v[3][PX];
+#pragma unroll
+            for (int k = 0; k < PX; k++) {
+                const float xr = (float)(x0 + k) - dcx;
+                const float sx = __builtin_fmaf(xr, m0, __builtin_fmaf(yr, m1, m2)) + scx;
+                const float sy = __builtin_fmaf(xr, m3, __builtin_fmaf(yr, m4, m5)) + scy;
+                float fx, fy;
+                if constexpr (NEAREST) {
+                    fx = floorf(sx + 0.5f);
+                    fy = floorf(sy + 0.5f);
+                } else {
+                    fx = floorf(sx);
+                    fy = floorf(sy);
+                }
+                const bool oob = empty || fx < (float)xlo || fy < (float)ylo || fx > (float)xhi || fy > (float)yhi || !(fx == fx) || !(fy == fy);
+                float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f;
+                if (!oob) {
+                    const int ix0 = (int)fx, iy0 = (int)fy;
+                    const int ix1 = min(ix0 + 1, xhi), iy1 = min(iy0 + 1, yhi);
+                    const uint32_t tl = load_px_global(simg + (size_t)iy0 * row_stride + (size_t)ix0 * 3);
+                    if constexpr (NEAREST) {
+                        o0 = ubyte0(tl); o1 = ubyte1(tl); o2 = ubyte2(tl);
+                    } else {
+                        const uint32_t tr = load_px_global(simg + (size_t)iy0 * row_stride + (size_t)ix1 * 3);
+                        const uint32_t bl = load_px_global(simg + (size_t)iy1 * row_stride + (size_t)ix0 * 3);
+                        const uint32_t br = load_px_global(simg + (size_t)iy1 * row_stride + (size_t)ix1 * 3);
+                        const float wx = sx - fx, wy = sy - fy;
+                        const float omx = 1.0f - wx, omy = 1.0f - wy;
+                        const float w00 = omy * omx, w01 = omy * wx, w10 = wy * omx;
+                        o0 = __builtin_fmaf(ubyte0(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte0(bl), w10, ubyte0(br) * wy * wx)));
+                        o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte1(br) * wy * wx)));
+                        o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte2(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte2(br) * wy * wx)));
+                    }
+                }
+                v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
+            }
+            store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
         }
+        return;
+    }
+
+    // ---- stage the box: (row, 4-pixel item) pairs form one flat index space dealt to the lanes; rows beyond
+    // the box repeat the ROI's last row (the clamp does it); all loads go out before the first is consumed
+    {
+        const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
+        const uint8_t *base4 = simg - skew;
+        const uint32_t col0 = (uint32_t)bx0 * 3u + skew;
+        const float inv_items = 1.0f / (float)items;
+        // the last load of the box stays inside the batch buffer
+        const bool safe = simg + ((size_t)min(by1 + 1, yhi) * row_stride + (size_t)bx0 * 3 + 12 * (size_t)items + 4) <= buf_end;
+        auto stage = [&](auto nsc) {
+            constexpr int NS = decltype(nsc)::value;
+            u32x4_a4 v[NS];
+            uint32_t dst_off[NS], ph[NS];
+#pragma unroll
+            for (int j = 0; j < NS; j++) {
+                const int idx = min(j * RMX_WAVE + lane, total - 1);
+                // idx / items: (idx + 0.5) / items is at least 0.5/items away from an integer, so the truncation is exact
+                const int r = (int)(((float)idx + 0.5f) * inv_items);
+                const int c = idx - __mul24(r, items);
+                const int ysrc = min(by0 + r, yhi);
+                const uint32_t off = (uint32_t)ysrc * row_stride + col0 + 12u * (uint32_t)c;
+                v[j] = *reinterpret_cast<const u32x4_a4 *>(base4 + (off & ~3u));
+                dst_off[j] = (uint32_t)(__mul24(r, pitch) + 4 * c);
+                ph[j] = off & 3u;
+            }
+#pragma unroll
+            for (int j = 0; j < NS; j++) {
+                const uint32_t d[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+                const uint4 px = expand4(d, ph[j]);
+                if (j * RMX_WAVE + lane < total) *reinterpret_cast<uint4 *>(lds + dst_off[j]) = px;
+            }
+        };
+        if (safe) {
+            if (total <= 4 * RMX_WAVE) stage(std::integral_constant<int, 4>{});
+            else if (total <= 8 * RMX_WAVE) stage(std::integral_constant<int, 8>{});
+            else stage(std::integral_constant<int, 16>{});
+        } else {
+            // the box touches the last bytes of the batch buffer: bounds-checked loads
+            for (int idx = lane; idx < total; idx += RMX_WAVE) {
+                const int r = idx / items, c = idx - r * items;
+                const uint8_t *p = simg + (size_t)min(by0 + r, yhi) * row_stride + (size_t)(bx0 + 4 * c) * 3;
+                uint32_t w[3];
+                load_realigned<4>(p, buf_end, w);
+                uint4 px;
+                px.x = w[0];
+                px.y = __builtin_amdgcn_alignbyte(w[1], w[0], 3);
+                px.z = __builtin_amdgcn_alignbyte(w[2], w[1], 2);
+                px.w = w[2] >> 8;
+                *reinterpret_cast<uint4 *>(lds + r * pitch + 4 * c) = px;
+            }
+        }
+        wave_sync();
+        // the column behind the box repeats its last column (it is read only when that is the ROI's last column)
+        for (int r = lane; r <= bh; r += RMX_WAVE) lds[r * pitch + bw] = lds[r * pitch + bw - 1];
         wave_sync();
     }
 
-    const int lr = lane >> 2, g = lane & 3;
-    const int y = Y0 + lr, x0 = X0 + g * PX;
-    const int cnt = min(PX, dw - x0);
-    if (y >= dh || cnt <= 0) return;
-    const float yr = (float)y - dcy;
-    float v[3][PX];
+    // ---- gather and blend, branch-free
+    const int boff = by0 * pitch + bx0;  // dword offset of source pixel (0, 0) relative to the slice (may be "negative")
+    const uint32_t xspan = (uint32_t)(xhi - xlo), yspan = (uint32_t)(yhi - ylo);
+    for (int pass = 0; pass < passes; pass++) {
+        const int y = Y0 + pass * WTH + lr;
+        if (y >= dh || cnt <= 0) continue;
+        const float yr = (float)y - dcy;
+        const float cxy = __builtin_fmaf(yr, m1, m2), cyy = __builtin_fmaf(yr, m4, m5);
+        float v[3][PX];
 #pragma unroll
-    for (int k = 0; k < PX; k++) {
-        const float xr = (float)(x0 + k) - dcx;
-        const float sx = __builtin_fmaf(xr, m0, __builtin_fmaf(yr, m1, m2)) + scx;
-        const float sy = __builtin_fmaf(xr, m3, __builtin_fmaf(yr, m4, m5)) + scy;
-        float fx, fy;
-        if constexpr (NEAREST) {
-            fx = floorf(sx + 0.5f);
-            fy = floorf(sy + 0.5f);
-        } else {
-            fx = floorf(sx);
-            fy = floorf(sy);
-        }
-        const bool oob = empty || fx < (float)xlo || fy < (float)ylo || fx > (float)xhi || fy > (float)yhi || !(fx == fx) || !(fy == fy);
-        float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f;
-        if (!oob) {
-            const int ix0 = (int)fx, iy0 = (int)fy;
-            const int ix1 = min(ix0 + 1, xhi), iy1 = min(iy0 + 1, yhi);
-            uint32_t tl, tr, bl, br;
-            if (use_lds) {
-                const int cx0 = min(max(ix0 - bx0, 0), bw - 1), cx1 = min(max(ix1 - bx0, 0), bw - 1);
-                const int cy0 = min(max(iy0 - by0, 0), bh - 1), cy1 = min(max(iy1 - by0, 0), bh - 1);
-                // one multiply for the four taps: the right / lower neighbour is 0 or 1 column / row away
-                const uint32_t *t0p = lds + __mul24(cy0, pitch) + cx0;
-                const int dx = cx1 - cx0, dy = (cy1 - cy0) ? pitch : 0;
-                tl = t0p[0];
-                if constexpr (!NEAREST) {
-                    tr = t0p[dx];
-                    bl = t0p[dy];
-                    br = t0p[dy + dx];
-                }
-            } else {
-                tl = load_px_global(simg + (size_t)iy0 * row_stride + (size_t)ix0 * 3);
-                if constexpr (!NEAREST) {
-                    tr = load_px_global(simg + (size_t)iy0 * row_stride + (size_t)ix1 * 3);
-                    bl = load_px_global(simg + (size_t)iy1 * row_stride + (size_t)ix0 * 3);
-                    br = load_px_global(simg + (size_t)iy1 * row_stride + (size_t)ix1 * 3);
-                }
-            }
+        for (int k = 0; k < PX; k++) {
+            const float xr = xr0 + (float)k;  // == (float)(x0 + k) - dcx: small integers, exact
+            float sx = __builtin_fmaf(xr, m0, cxy) + scx;
+            float sy = __builtin_fmaf(xr, m3, cyy) + scy;
             if constexpr (NEAREST) {
+                sx += 0.5f;
+                sy += 0.5f;
+            }
+            const int ix0 = floor_i32(sx), iy0 = floor_i32(sy);
+            const bool inb = (uint32_t)(ix0 - xlo) <= xspan && (uint32_t)(iy0 - ylo) <= yspan && sx == sx && sy == sy;
+            // (an address inside the slice also for pixels outside the ROI, whose coordinates can be anything)
+            const uint32_t *t0p = lds + (inb ? (__mul24(iy0, pitch) + ix0 - boff) : 0);
+            float o0, o1, o2;
+            if constexpr (NEAREST) {
+                const uint32_t tl = t0p[0];
                 o0 = ubyte0(tl); o1 = ubyte1(tl); o2 = ubyte2(tl);
             } else {
-                const float wx = sx - fx, wy = sy - fy;
+                const uint32_t tl = t0p[0], tr = t0p[1];
+                const uint32_t *t1p = t0p + pitch;
+                const uint32_t bl = t1p[0], br = t1p[1];
+                // sx - floor(sx): exact for the non-negative coordinates of pixels inside the ROI
+                const float wx = __builtin_amdgcn_fractf(sx), wy = __builtin_amdgcn_fractf(sy);
                 const float omx = 1.0f - wx, omy = 1.0f - wy;
                 const float w00 = omy * omx, w01 = omy * wx, w10 = wy * omx;
                 o0 = __builtin_fmaf(ubyte0(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte0(bl), w10, ubyte0(br) * wy * wx)));
                 o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte1(br) * wy * wx)));
                 o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte2(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte2(br) * wy * wx)));
             }
+            v[0][k] = inb ? o0 : 0.0f;
+            v[1][k] = inb ? o1 : 0.0f;
+            v[2][k] = inb ? o2 : 0.0f;
         }
-        v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
-    }
-    // whole group into 16-byte aligned destination rows: packed stores (a.aux1 is set by the host when every
-    // written width and the padded width are multiples of 8 and the destination base is 16-byte aligned)
-    if (a.aux1 && cnt == PX) {
-        PackedGroup<T> packed;
-        pack_group_dir<T, LAYOUT, false>(v, packed);
-        store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
-    } else {
-        store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
+        // whole group into 16-byte aligned destination rows: packed stores (the host sets the flag when every
+        // written width and the padded width are multiples of 8 and the destination base is 16-byte aligned)
+        if (packed_ok && cnt == PX) {
+            PackedGroup<T> packed;
+            pack_group_dir<T, LAYOUT, false>(v, packed);
+            store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
+        } else {
+            store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
+        }
     }
 }
 
