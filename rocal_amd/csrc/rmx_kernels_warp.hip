@@ -68,6 +68,7 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     // source bounding box of the tile (wave-uniform), one pixel of margin, clipped to the ROI
     const int X1 = min(X0 + WTW, dw) - 1, Y1 = min(Y0 + WTH * passes, dh) - 1;
     float bxmin = 3.0e38f, bxmax = -3.0e38f, bymin = 3.0e38f, bymax = -3.0e38f;
+    bool corners_ok = true;
 #pragma unroll
     for (int cy = 0; cy < 2; cy++)
 #pragma unroll
@@ -81,7 +82,10 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
             }
             bxmin = __builtin_fminf(bxmin, sx); bxmax = __builtin_fmaxf(bxmax, sx);
             bymin = __builtin_fminf(bymin, sy); bymax = __builtin_fmaxf(bymax, sy);
+            corners_ok = corners_ok && sx == sx && sy == sy;
         }
+    // every pixel of the tile maps between the corner extremes: when those lie inside the ROI no pixel needs a test
+    const bool all_in = corners_ok && bxmin >= (float)xlo && bymin >= (float)ylo && bxmax < (float)(xhi + 1) && bymax < (float)(yhi + 1);
     // keep the float->int conversions in range for degenerate matrices
     bxmin = __builtin_fmaxf(bxmin, -1.0e6f); bxmax = __builtin_fminf(bxmax, 1.0e6f);
     bymin = __builtin_fmaxf(bymin, -1.0e6f); bymax = __builtin_fminf(bymax, 1.0e6f);
@@ -207,55 +211,60 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     // ---- gather and blend, branch-free
     const int boff = by0 * pitch + bx0;  // dword offset of source pixel (0, 0) relative to the slice (may be "negative")
     const uint32_t xspan = (uint32_t)(xhi - xlo), yspan = (uint32_t)(yhi - ylo);
-    for (int pass = 0; pass < passes; pass++) {
-        const int y = Y0 + pass * WTH + lr;
-        if (y >= dh || cnt <= 0) continue;
-        const float yr = (float)y - dcy;
-        const float cxy = __builtin_fmaf(yr, m1, m2), cyy = __builtin_fmaf(yr, m4, m5);
-        float v[3][PX];
+    auto gather = [&](auto chk) {
+        constexpr bool CHECK = decltype(chk)::value;
+        for (int pass = 0; pass < passes; pass++) {
+            const int y = Y0 + pass * WTH + lr;
+            if (y >= dh || cnt <= 0) continue;
+            const float yr = (float)y - dcy;
+            const float cxy = __builtin_fmaf(yr, m1, m2), cyy = __builtin_fmaf(yr, m4, m5);
+            float v[3][PX];
 #pragma unroll
-        for (int k = 0; k < PX; k++) {
-            const float xr = xr0 + (float)k;  // == (float)(x0 + k) - dcx: small integers, exact
-            float sx = __builtin_fmaf(xr, m0, cxy) + scx;
-            float sy = __builtin_fmaf(xr, m3, cyy) + scy;
-            if constexpr (NEAREST) {
-                sx += 0.5f;
-                sy += 0.5f;
+            for (int k = 0; k < PX; k++) {
+                const float xr = xr0 + (float)k;  // == (float)(x0 + k) - dcx: small integers, exact
+                float sx = __builtin_fmaf(xr, m0, cxy) + scx;
+                float sy = __builtin_fmaf(xr, m3, cyy) + scy;
+                if constexpr (NEAREST) {
+                    sx += 0.5f;
+                    sy += 0.5f;
+                }
+                const int ix0 = floor_i32(sx), iy0 = floor_i32(sy);
+                const bool inb = !CHECK || ((uint32_t)(ix0 - xlo) <= xspan && (uint32_t)(iy0 - ylo) <= yspan && sx == sx && sy == sy);
+                // (an address inside the slice also for pixels outside the ROI, whose coordinates can be anything)
+                const uint32_t *t0p = lds + (inb ? (__mul24(iy0, pitch) + ix0 - boff) : 0);
+                float o0, o1, o2;
+                if constexpr (NEAREST) {
+                    const uint32_t tl = t0p[0];
+                    o0 = ubyte0(tl); o1 = ubyte1(tl); o2 = ubyte2(tl);
+                } else {
+                    const uint32_t tl = t0p[0], tr = t0p[1];
+                    const uint32_t *t1p = t0p + pitch;
+                    const uint32_t bl = t1p[0], br = t1p[1];
+                    // sx - floor(sx): exact for the non-negative coordinates of pixels inside the ROI
+                    const float wx = __builtin_amdgcn_fractf(sx), wy = __builtin_amdgcn_fractf(sy);
+                    const float omx = 1.0f - wx, omy = 1.0f - wy;
+                    const float w00 = omy * omx, w01 = omy * wx, w10 = wy * omx;
+                    o0 = __builtin_fmaf(ubyte0(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte0(bl), w10, ubyte0(br) * wy * wx)));
+                    o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte1(br) * wy * wx)));
+                    o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte2(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte2(br) * wy * wx)));
+                }
+                v[0][k] = inb ? o0 : 0.0f;
+                v[1][k] = inb ? o1 : 0.0f;
+                v[2][k] = inb ? o2 : 0.0f;
             }
-            const int ix0 = floor_i32(sx), iy0 = floor_i32(sy);
-            const bool inb = (uint32_t)(ix0 - xlo) <= xspan && (uint32_t)(iy0 - ylo) <= yspan && sx == sx && sy == sy;
-            // (an address inside the slice also for pixels outside the ROI, whose coordinates can be anything)
-            const uint32_t *t0p = lds + (inb ? (__mul24(iy0, pitch) + ix0 - boff) : 0);
-            float o0, o1, o2;
-            if constexpr (NEAREST) {
-                const uint32_t tl = t0p[0];
-                o0 = ubyte0(tl); o1 = ubyte1(tl); o2 = ubyte2(tl);
+            // whole group into 16-byte aligned destination rows: packed stores (the host sets the flag when every
+            // written width and the padded width are multiples of 8 and the destination base is 16-byte aligned)
+            if (packed_ok && cnt == PX) {
+                PackedGroup<T> packed;
+                pack_group_dir<T, LAYOUT, false>(v, packed);
+                store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
             } else {
-                const uint32_t tl = t0p[0], tr = t0p[1];
-                const uint32_t *t1p = t0p + pitch;
-                const uint32_t bl = t1p[0], br = t1p[1];
-                // sx - floor(sx): exact for the non-negative coordinates of pixels inside the ROI
-                const float wx = __builtin_amdgcn_fractf(sx), wy = __builtin_amdgcn_fractf(sy);
-                const float omx = 1.0f - wx, omy = 1.0f - wy;
-                const float w00 = omy * omx, w01 = omy * wx, w10 = wy * omx;
-                o0 = __builtin_fmaf(ubyte0(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte0(bl), w10, ubyte0(br) * wy * wx)));
-                o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte1(br) * wy * wx)));
-                o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte2(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte2(br) * wy * wx)));
+                store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
             }
-            v[0][k] = inb ? o0 : 0.0f;
-            v[1][k] = inb ? o1 : 0.0f;
-            v[2][k] = inb ? o2 : 0.0f;
         }
-        // whole group into 16-byte aligned destination rows: packed stores (the host sets the flag when every
-        // written width and the padded width are multiples of 8 and the destination base is 16-byte aligned)
-        if (packed_ok && cnt == PX) {
-            PackedGroup<T> packed;
-            pack_group_dir<T, LAYOUT, false>(v, packed);
-            store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
-        } else {
-            store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
-        }
-    }
+    };
+    if (all_in) gather(std::false_type{});
+    else gather(std::true_type{});
 }
 
 template <bool NEAREST>
