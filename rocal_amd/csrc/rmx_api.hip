@@ -509,9 +509,10 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 const int kxi = (int)std::ceil(2.0f * std::max(s.rx, 1.0f));
                 const int cols = std::min<int>((int)op->src.w, (int)std::ceil(tile_w * (double)std::max(s.rx, 1.0f)) + kxi + 4);
                 const int pitch = ((cols + 3) / 4) * 4 + 8 + 2 * ((kxi + 3) / 4 * 4);
-                const int items = (cols + 3) / 4 + 1;
-                const int rows_per_round = items <= 64 ? 4 : (items <= 128 ? 2 : 1);
-                lds = std::max(lds, (size_t)rows_per_round * pitch * 4);
+                // (a tile's own row can be shorter than this bound: then more rows go into a round)
+                const int pads = 8 + 2 * ((kxi + 3) / 4 * 4);
+                const int need = std::max(pitch, std::max(2 * std::min(pitch, 512 + pads), 4 * std::min(pitch, 256 + pads)));
+                lds = std::max(lds, (size_t)need * 4);
             }
             op->lds_per_wave = (int)((std::max<size_t>(lds, 64) + 15) / 16 * 16);  // the staged source rows only
             if (op->lds_per_wave > op->ctx->max_lds_per_block)

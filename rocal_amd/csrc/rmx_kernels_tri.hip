@@ -434,7 +434,8 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
     // lane, they are 12 bytes apart) and the item's place in the staged row.
     const int spr = (items + RMX_WAVE - 1) / RMX_WAVE;
     const int sh = spr == 1 ? 0 : (spr == 2 ? 1 : 2);  // log2(slots per row)
-    const int rpr = 4 >> sh;                           // rows per round
+    // rows per round, never more than the slice holds (then the spare slots repeat a row)
+    const int rpr = min(4 >> sh, max(1, (a.lds_bytes >> 2) / spitch));
     uint32_t sl_al[4], sl_lds[4];
     bool sl_on[4];
     const uint32_t low = ((uint32_t)(cs + 4 * min(lane, items - 1)) * 3u) & 3u;
@@ -447,7 +448,8 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
         sl_on[i] = lane + RMX_WAVE * k < items;
     }
     // every wide load of this wavefront stays inside the batch buffer (last row, last item, carry and load width)
-    const bool safe = simg + ((size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16) <= buf_end;
+    // (rows longer than the three slots of a round take the row-by-row path as well)
+    const bool safe = items <= 3 * RMX_WAVE && simg + ((size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16) <= buf_end;
 
     // clamp-to-edge columns of the nr staged rows
     auto replicate = [&](int nr) {

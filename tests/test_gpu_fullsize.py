@@ -124,3 +124,88 @@ def test_degenerate_samples(ctx):
     assert (got[0, :8, :8] == np.array([10, 200, 77], np.uint8)).all()  # a 1x1 source is a constant image
     assert (got[1] == 9).all()                                            # nothing is written for an empty destination
     assert np.array_equal(got[0, :8, :8], exp[0, :8, :8]) and np.array_equal(got[2, :8, :16], exp[2, :8, :16])
+
+
+@pytest.mark.parametrize("rx,ry", [(1.3, 1.0), (1.9, 2.4), (3.0, 3.0), (3.7, 3.7), (2.5, 1.2)])
+def test_triangular_downscale_tap_and_row_length_classes(ctx, rx, ry):
+    """The downscaling triangular kernel: 4/6/8-tap specialisations, 1/2/3 load slots per source row, partial
+    last tile, per-sample windows, mirror, and an exact-size source whose last rows take the bounds-checked
+    loader. (rx, ry) are the ratios of the first sample; the others shrink a little more or less."""
+    import torch
+    rng = np.random.default_rng(int(rx * 100 + ry * 10))
+    n, dw0, dh0 = 3, 200, 37
+    W, H = int(round(dw0 * rx)) + 9, int(round(dh0 * ry)) + 5
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.array([[0, 0, W - 9, H - 5], [4, 3, W - 4, H - 3], [9, 5, W - 9, H - 5]], np.uint32)  # the last two end at (W-1, H-1)
+    dw = np.array([dw0, dw0 - 8, dw0 - 7], np.uint32)
+    dh = np.array([dh0, dh0 - 1, dh0], np.uint32)
+    mirror = np.array([0, 1, 1], np.uint32)
+    inv = (1 / wl.STD).astype(np.float32)
+    scale, bias = np.tile(inv, n), np.tile(-(wl.MEAN * inv), n)
+    src = torch.from_numpy(img.reshape(-1).copy()).cuda()  # nothing behind the last pixel belongs to the tensor
+    for dtype, layout in ((ops.FP16, ops.NCHW), (ops.UINT8, ops.NHWC)):
+        op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, dh0, dw0, layout, dtype), ops.TRIANGULAR)
+        if dtype == ops.UINT8:
+            op.update(roi, dw, dh, mirror)
+            exp = orc.resize(img, roi, dw, dh, dh0, dw0, interp=orc.TRIANGULAR, mirror=mirror, layout=layout, dtype=dtype)
+        else:
+            op.update_cmn(roi, dw, dh, scale, bias, mirror)
+            exp = orc.resize(img, roi, dw, dh, dh0, dw0, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=layout, dtype=dtype)
+        assert op.kernel_name == "rmx_resize_tri_down_kernel"
+        out = op.alloc_output()
+        op.launch(src.view(n, H, W, 3), out)
+        ctx.sync()
+        got = out.cpu().numpy()
+        assert np.array_equal(_bits(got), _bits(exp)), "%d values differ" % int((got != exp).sum())
+
+
+def test_triangular_ring_and_downscale_kernels_agree(ctx, monkeypatch):
+    """The same downscaling batch through the ring kernel (forced) and through the register kernel."""
+    import torch
+    rng = np.random.default_rng(77)
+    n, H, W = 2, 150, 260
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.array([[0, 0, W, H], [10, 6, 240, 140]], np.uint32)
+    dw, dh = np.array([96, 88], np.uint32), np.array([64, 50], np.uint32)
+    outs = []
+    for ring in ("0", "1"):
+        monkeypatch.setenv("RMX_TUNE_TRI_RING", ring)
+        c2 = ops.Context()
+        op = ops.Resize(c2, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 64, 96, ops.NCHW, ops.FP32), ops.TRIANGULAR)
+        op.update(roi, dw, dh)
+        assert op.kernel_name == ("rmx_resize_tri_kernel" if ring == "1" else "rmx_resize_tri_down_kernel")
+        out = op.alloc_output()
+        op.launch(torch.from_numpy(img).cuda(), out)
+        c2.sync()
+        outs.append(out.cpu().numpy())
+    assert np.array_equal(_bits(outs[0]), _bits(outs[1]))
+
+
+@pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST])
+def test_warp_on_an_exact_size_source_and_tiny_windows(ctx, interp):
+    """Boxes that reach the last bytes of the batch buffer (bounds-checked staging), a 1x1 and a 2x3 ROI, ROIs away
+    from the origin (repeated edge column / row), destinations that are not multiples of 8 or of the tile."""
+    import torch
+    rng = np.random.default_rng(21)
+    n, H, W = 5, 67, 83
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.array([[0, 0, W, H], [40, 30, 1, 1], [20, 10, 2, 3], [11, 7, 72, 60], [0, 0, W, H]], np.uint32)
+    dw = np.array([83, 40, 33, 77, 83], np.uint32)
+    dh = np.array([67, 20, 41, 50, 67], np.uint32)
+    affine = np.array([[1.0, 0.0, 0.0, 1.0, 0.0, 0.0],          # identity: reads up to the last pixel
+                       [0.1, 0.0, 0.0, 0.1, 0.0, 0.0],
+                       [0.05, 0.02, -0.02, 0.05, 0.3, 0.2],
+                       [0.9, 0.25, -0.2, 1.1, 3.5, -2.25],
+                       [1.2, -0.4, 0.5, 0.8, -9.0, 12.0]], np.float32)  # rocAL order x0,y0,x1,y1,o0,o1
+    m = np.stack([orc.affine_from_rocal(a) for a in affine])
+    exp = orc.warp_affine(img, roi, m, dw, dh, H, W, interp=interp)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    op = ops.WarpAffine(ctx, sd, sd, interp)
+    op.update(roi, affine, dw, dh)
+    out = op.alloc_output()
+    src = torch.from_numpy(img.reshape(-1).copy()).cuda()
+    op.launch(src.view(n, H, W, 3), out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    for i in range(n):
+        assert np.array_equal(got[i, :dh[i], :dw[i]], exp[i, :dh[i], :dw[i]]), "sample %d: %d values differ" % (i, int((got[i, :dh[i], :dw[i]] != exp[i, :dh[i], :dw[i]]).sum()))
