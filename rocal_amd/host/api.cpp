@@ -4,7 +4,10 @@
 // stored in the context, printed, and turned into a null tensor / ROCAL_RUNTIME_ERROR.
 #include "rocal_host.h"
 
+#include "meta.h"
+
 #include <iostream>
+#include <type_traits>
 
 namespace {
 
@@ -12,6 +15,27 @@ void report(Context *context, const std::exception &e) {
     context->capture_error(e.what());
     std::cerr << e.what() << std::endl;
 }
+
+// MasterGraph::meta_add_node (master_graph.h:265-273): the metadata twin of an augmentation node
+template <typename MetaT, typename NodeT>
+void meta_add_node(Context *context, std::shared_ptr<NodeT> node) {
+    if (!context->master_graph->meta_data_enabled()) return;
+    auto meta_node = std::make_shared<MetaT>();
+    meta_node->_node = node;
+    meta_node->_batch_size = (int)context->master_graph->batch_size();
+    context->master_graph->meta_graph()->_meta_nodes.push_back(meta_node);
+}
+
+// which metadata node follows which augmentation node (rocal_api_augmentation.cpp: the meta_add_node calls)
+template <typename NodeT> struct MetaOf { using type = void; };
+template <> struct MetaOf<CropNode> { using type = CropMetaNode; };
+template <> struct MetaOf<CropMirrorNormalizeNode> { using type = CropMirrorNormalizeMetaNode; };
+template <> struct MetaOf<CropResizeNode> { using type = CropResizeMetaNode; };
+template <> struct MetaOf<ResizeNode> { using type = ResizeMetaNode; };
+template <> struct MetaOf<ResizeCropMirrorNode> { using type = ResizeCropMirrorMetaNode; };
+template <> struct MetaOf<ResizeMirrorNormalizeNode> { using type = ResizeMirrorNormalizeMetaNode; };
+template <> struct MetaOf<FlipNode> { using type = FlipMetaNode; };
+template <> struct MetaOf<RotateNode> { using type = RotateMetaNode; };
 
 enum class Dims { KEEP, SET };
 
@@ -44,6 +68,7 @@ Tensor *add_op(RocalContext p_context, RocalTensor p_input, bool is_output, Roca
         output = context->master_graph->create_tensor(output_info, is_output);
         auto node = context->master_graph->add_node<NodeT>({input}, {output});
         init(*node);
+        if constexpr (!std::is_void<typename MetaOf<NodeT>::type>::value) meta_add_node<typename MetaOf<NodeT>::type, NodeT>(context, node);
     } catch (const std::exception &e) {
         report(context, e);
         output = nullptr;
@@ -154,6 +179,84 @@ RocalStatus rocalToTensor(RocalContext p_context, void *out_ptr, RocalTensorLayo
     } catch (const std::exception &e) {
         report(context, e);
         return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+/* ------------------------------------------------------------------ bounding boxes */
+
+RocalStatus rocalEnableBoundingBoxes(RocalContext p_context) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->enable_meta_data();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+RocalStatus rocalSetBoundingBoxes(RocalContext p_context, const unsigned *counts, const float *ltrb, const int *labels) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        if (!context->master_graph->meta_data_enabled()) THROW("rocalEnableBoundingBoxes was not called")
+        if (!counts || !ltrb || !labels) THROW("counts, box and label arrays are required")
+        const size_t n = context->master_graph->batch_size();
+        auto batch = std::make_shared<MetaDataBatch>(n);
+        size_t k = 0;
+        for (size_t i = 0; i < n; i++)
+            for (unsigned j = 0; j < counts[i]; j++, k++) {
+                batch->get_bb_cords_batch()[i].push_back({ltrb[4 * k], ltrb[4 * k + 1], ltrb[4 * k + 2], ltrb[4 * k + 3]});
+                batch->get_labels_batch()[i].push_back(labels[k]);
+            }
+        context->master_graph->set_input_meta_data(batch);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+unsigned rocalGetBoundingBoxCount(RocalContext p_context, unsigned *counts) {
+    if (!p_context) return 0;
+    auto meta = static_cast<Context *>(p_context)->master_graph->output_meta_data();
+    if (!meta) return 0;
+    unsigned total = 0;
+    for (size_t i = 0; i < meta->size(); i++) {
+        const unsigned c = (unsigned)meta->get_bb_cords_batch()[i].size();
+        if (counts) counts[i] = c;
+        total += c;
+    }
+    return total;
+}
+
+RocalStatus rocalGetBoundingBoxCords(RocalContext p_context, float *ltrb) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto meta = static_cast<Context *>(p_context)->master_graph->output_meta_data();
+    if (!meta || !ltrb) return ROCAL_RUNTIME_ERROR;
+    size_t k = 0;
+    for (size_t i = 0; i < meta->size(); i++)
+        for (const auto &b : meta->get_bb_cords_batch()[i]) {
+            ltrb[k++] = b.l;
+            ltrb[k++] = b.t;
+            ltrb[k++] = b.r;
+            ltrb[k++] = b.b;
+        }
+    return ROCAL_OK;
+}
+
+// one label per box of rocalGetBoundingBoxCords (a node that pads an empty sample with a zero box adds label 0, except
+// the plain resize, which adds the box only: there the label is reported as 0 too)
+RocalStatus rocalGetBoundingBoxLabel(RocalContext p_context, int *labels) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto meta = static_cast<Context *>(p_context)->master_graph->output_meta_data();
+    if (!meta || !labels) return ROCAL_RUNTIME_ERROR;
+    size_t k = 0;
+    for (size_t i = 0; i < meta->size(); i++) {
+        const auto &l = meta->get_labels_batch()[i];
+        for (size_t j = 0; j < meta->get_bb_cords_batch()[i].size(); j++) labels[k++] = j < l.size() ? l[j] : 0;
     }
     return ROCAL_OK;
 }

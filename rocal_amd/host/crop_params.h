@@ -35,6 +35,8 @@ class CropParam {
     const std::vector<uint32_t> &get_y1_arr_val() const { return y1_arr_val; }
     const std::vector<uint32_t> &get_croph_arr_val() const { return croph_arr_val; }
     const std::vector<uint32_t> &get_cropw_arr_val() const { return cropw_arr_val; }
+    const std::vector<uint32_t> &get_x2_arr_val() const { return x2_arr_val; }
+    const std::vector<uint32_t> &get_y2_arr_val() const { return y2_arr_val; }
     void get_crop_dimensions(std::vector<uint32_t> &crop_w_dim, std::vector<uint32_t> &crop_h_dim) const {
         crop_w_dim = cropw_arr_val;
         crop_h_dim = croph_arr_val;

@@ -170,7 +170,41 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
     const int coin_v[2] = {0, 1};
     const double coin_f[2] = {0.5, 0.5};
     RocalIntParam coin = rocalCreateIntRand(coin_v, coin_f, 2);
-    if (scenario == "cmn") {
+    // bounding boxes (scenarios meta_*): <dir>/boxes.txt holds, per sample, a count and then "l t r b label" lines
+    const bool with_boxes = scenario.rfind("meta_", 0) == 0;
+    std::vector<unsigned> box_counts(n, 0);
+    std::vector<float> box_ltrb;
+    std::vector<int> box_labels;
+    if (with_boxes) {
+        std::ifstream bf(dir + "/boxes.txt");
+        for (unsigned i = 0; i < n; i++) {
+            if (!(bf >> box_counts[i])) return 2;
+            for (unsigned j = 0; j < box_counts[i]; j++) {
+                float l, t, r, b;
+                int label;
+                bf >> l >> t >> r >> b >> label;
+                box_ltrb.insert(box_ltrb.end(), {l, t, r, b});
+                box_labels.push_back(label);
+            }
+        }
+        if (rocalEnableBoundingBoxes(ctx) != ROCAL_OK) return 11;
+    }
+    if (scenario == "meta_cmn") {
+        outs.push_back(rocalCropMirrorNormalize(ctx, src, 40, 48, 0.5f, 0.5f, mean, stdv, true, coin, ROCAL_NCHW, ROCAL_FP32));
+    } else if (scenario == "meta_resize_flip") {
+        RocalTensor a = rocalResize(ctx, src, 40, 32, false);
+        outs.push_back(rocalFlipFixed(ctx, a, 1, 1, true));
+    } else if (scenario == "meta_rotate") {
+        outs.push_back(rocalRotateFixed(ctx, src, 30.0f, true));
+    } else if (scenario == "meta_rcm") {
+        outs.push_back(rocalResizeCropMirrorFixed(ctx, src, 36, 28, true, 40, 50, rocalCreateIntParameter(1)));
+    } else if (scenario == "meta_crop_then_rmn") {
+        RocalTensor a = rocalCropFixed(ctx, src, 30, 20, 1, false, 5, 7, 0);
+        outs.push_back(rocalResizeMirrorNormalize(ctx, a, 60, 40, mean, stdv, true, ROCAL_SCALING_MODE_STRETCH, {}, 0, 0, ROCAL_LINEAR_INTERPOLATION,
+                                                  rocalCreateIntParameter(1), ROCAL_NCHW, ROCAL_FP16));
+    } else if (scenario == "meta_crop_resize") {
+        outs.push_back(rocalCropResizeFixed(ctx, src, 64, 64, true, 0.5f, 1.2f, 0.3f, 0.7f));
+    } else if (scenario == "cmn") {
         RocalIntParam mirror = coin;
         outs.push_back(rocalCropMirrorNormalize(ctx, src, 40, 48, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP32));
     } else if (scenario == "rrc_cmn") {
@@ -229,9 +263,25 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
     }
     if (mid) std::cout << "intermediate_elided " << (rocalTensorBuffer(mid) == nullptr ? 1 : 0) << std::endl;
     for (int b = 0; b < 2; b++) {
+        if (with_boxes && rocalSetBoundingBoxes(ctx, box_counts.data(), box_ltrb.data(), box_labels.data()) != ROCAL_OK) return 12;
         if (rocalDeviceSourceFeed(ctx, src, dev, rw.data(), rh.data()) != ROCAL_OK || rocalRun(ctx) != ROCAL_OK) {
             std::cerr << "run failed: " << rocalGetErrorMessage(ctx) << std::endl;
             return 8;
+        }
+        if (with_boxes) {
+            std::vector<unsigned> counts(n);
+            const unsigned total = rocalGetBoundingBoxCount(ctx, counts.data());
+            std::vector<float> ltrb(4 * (size_t)total);
+            std::vector<int> labels(total);
+            if (rocalGetBoundingBoxCords(ctx, ltrb.data()) != ROCAL_OK || rocalGetBoundingBoxLabel(ctx, labels.data()) != ROCAL_OK) return 13;
+            std::ofstream f(dir + "/boxes_b" + std::to_string(b) + ".txt");
+            f.precision(9);
+            size_t k = 0;
+            for (unsigned i = 0; i < n; i++) {
+                f << counts[i] << "\n";
+                for (unsigned j = 0; j < counts[i]; j++, k++)
+                    f << ltrb[4 * k] << " " << ltrb[4 * k + 1] << " " << ltrb[4 * k + 2] << " " << ltrb[4 * k + 3] << " " << labels[k] << "\n";
+            }
         }
         for (size_t k = 0; k < outs.size(); k++) {
             const size_t bytes = rocalTensorDataSize(outs[k]);

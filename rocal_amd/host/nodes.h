@@ -56,6 +56,7 @@ class CropNode : public Node {
     void init(unsigned crop_h, unsigned crop_w, float x_drift, float y_drift);
     void init(unsigned crop_h, unsigned crop_w);  // centre crop
     void init(FloatParam *crop_h_factor, FloatParam *crop_w_factor, FloatParam *x_drift, FloatParam *y_drift);
+    std::shared_ptr<RocalCropParam> get_crop_param() { return _crop_param; }
 
    protected:
     void create_node() override;
@@ -86,6 +87,8 @@ class FlipNode : public Node {
     FlipNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(int h_flag, int v_flag);
     void init(IntParam *h_flag, IntParam *v_flag);
+    const std::vector<int> &horizontal_values() const { return _horizontal.values(); }
+    const std::vector<int> &vertical_values() const { return _vertical.values(); }
 
    protected:
     void create_node() override;
@@ -103,6 +106,9 @@ class ResizeFamilyNode : public Node {
    public:
     using Node::Node;
     bool try_absorb(Node *next) override;
+    // the resize target (the padded output size), as the reference's metadata nodes read it
+    unsigned get_dst_width() { return (unsigned)_outputs[0]->info().max_shape()[0]; }
+    unsigned get_dst_height() { return (unsigned)_outputs[0]->info().max_shape()[1]; }
 
    protected:
     void create_resize_op(int interpolation);
@@ -141,6 +147,7 @@ class CropResizeNode : public ResizeFamilyNode {
     void init(float area, float aspect_ratio, float x_center_drift, float y_center_drift);
     void init(FloatParam *area, FloatParam *aspect_ratio, FloatParam *x_center_drift, FloatParam *y_center_drift);
     void init(unsigned crop_h, unsigned crop_w, float x_drift, float y_drift, RocalResizeInterpolationType interpolation_type);
+    const CropParam *get_crop_param() const { return _is_random_crop ? static_cast<const CropParam *>(_crop_param.get()) : _crop_fixed_param.get(); }
 
    protected:
     void create_node() override;
@@ -158,6 +165,8 @@ class ResizeCropMirrorNode : public ResizeFamilyNode {
     ResizeCropMirrorNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(unsigned crop_h, unsigned crop_w, IntParam *mirror, RocalResizeInterpolationType interpolation_type);
     void init(FloatParam *crop_h_factor, FloatParam *crop_w_factor, IntParam *mirror, RocalResizeInterpolationType interpolation_type);
+    std::shared_ptr<RocalCropParam> get_crop_param() { return _crop_param; }
+    const std::vector<int> &mirror_values() const { return _mirror.values(); }
 
    protected:
     void create_node() override;
@@ -175,6 +184,7 @@ class ResizeMirrorNormalizeNode : public ResizeFamilyNode {
     ResizeMirrorNormalizeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(unsigned dest_width, unsigned dest_height, RocalResizeScalingMode scaling_mode, std::vector<unsigned> max_size,
               RocalResizeInterpolationType interpolation_type, std::vector<float> &mean, std::vector<float> &std_dev, IntParam *mirror);
+    const std::vector<int> &mirror_values() const { return _mirror.values(); }
 
    protected:
     void create_node() override;
@@ -298,6 +308,9 @@ class RotateNode : public Node {
     RotateNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float angle, RocalResizeInterpolationType interpolation_type);
     void init(FloatParam *angle, RocalResizeInterpolationType interpolation_type);
+    const std::vector<float> &angle_values() const { return _angle.values(); }
+    unsigned get_dst_width() { return (unsigned)_outputs[0]->info().max_shape()[0]; }
+    unsigned get_dst_height() { return (unsigned)_outputs[0]->info().max_shape()[1]; }
 
    protected:
     void create_node() override;

@@ -5,6 +5,7 @@
 #include <algorithm>
 #include <iostream>
 
+#include "meta.h"
 #include "parameters.h"
 
 /* ---------------------------------------------------------------- TensorInfo / Tensor */
@@ -207,7 +208,18 @@ void MasterGraph::run() {
     if (!_built) THROW("rocalVerify must be called before rocalRun")
     ParameterFactory::instance()->renew_parameters();
     for (auto &n : _nodes) n->update_parameters();
+    if (_meta_graph && _input_meta) {
+        if (_input_meta->size() != _batch_size) THROW("bounding boxes were given for " + TOSTR(_input_meta->size()) + " samples, the batch has " + TOSTR(_batch_size))
+        // an empty instance when nodes will fill it, a copy when no node touches the boxes
+        _output_meta = _input_meta->clone(_meta_graph->_meta_nodes.empty());
+        _meta_graph->process(_input_meta, _output_meta);
+    }
     _graph->process();
+}
+
+void MasterGraph::enable_meta_data() {
+    if (!_nodes.empty()) THROW("bounding boxes must be switched on before the first augmentation is added")
+    if (!_meta_graph) _meta_graph = std::make_shared<BoundingBoxGraph>();
 }
 
 // master_graph.cpp:514-535 (checks) and :612-632 (device branch). The reference walks the read buffers of its

@@ -132,6 +132,9 @@ class Node {
 // The part of Context + MasterGraph the hot path needs (rocAL/include/pipeline/master_graph.h:245-263,
 // source/pipeline/master_graph.cpp:247-260,323-335,408,1010-1017): owns tensors and nodes, builds them
 // on verify, and per batch renews parameters, updates every node and processes the graph.
+class BoundingBoxGraph;
+class MetaDataBatch;
+
 class MasterGraph {
    public:
     MasterGraph(size_t batch_size, int gpu_id, void *stream);
@@ -148,6 +151,13 @@ class MasterGraph {
     // master_graph.cpp:514-856: converts the single u8 output tensor into a float tensor in caller memory
     void to_tensor(void *out_ptr, RocalTensorlayout format, float multiplier0, float multiplier1, float multiplier2, float offset0, float offset1,
                    float offset2, bool reverse_channels, RocalTensorDataType output_data_type, unsigned max_roi_height, unsigned max_roi_width);
+    // bounding boxes that follow the images (master_graph.cpp:1004-1013): switched on before nodes are added,
+    // a batch of boxes is handed in before each run and the transformed batch is read back after it
+    void enable_meta_data();
+    bool meta_data_enabled() const { return (bool)_meta_graph; }
+    std::shared_ptr<BoundingBoxGraph> meta_graph() { return _meta_graph; }
+    void set_input_meta_data(std::shared_ptr<MetaDataBatch> m) { _input_meta = m; }
+    std::shared_ptr<MetaDataBatch> output_meta_data() { return _output_meta; }
     size_t batch_size() const { return _batch_size; }
     const std::vector<Tensor *> &outputs() const { return _outputs; }
     bool built() const { return _built; }
@@ -159,6 +169,8 @@ class MasterGraph {
     std::list<std::unique_ptr<Tensor>> _tensors;
     std::vector<Tensor *> _outputs;
     std::vector<void *> _owned_buffers;
+    std::shared_ptr<BoundingBoxGraph> _meta_graph;
+    std::shared_ptr<MetaDataBatch> _input_meta, _output_meta;
     bool _built = false;
     // the conversion op of to_tensor(), rebuilt when the requested format changes
     rmx_op *_to_tensor_op = nullptr;

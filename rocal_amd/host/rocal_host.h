@@ -51,6 +51,16 @@ extern "C" RocalStatus ROCAL_API_CALL rocalToTensor(RocalContext rocal_context, 
                                                     float offset0, float offset1, float offset2, bool reverse_channels,
                                                     RocalOutputMemType output_mem_type, int max_roi_height = 0, int max_roi_width = 0);
 
+/* ---- bounding boxes (rocal_api_meta_data.h). Metadata readers are outside the hot path: rocalEnableBoundingBoxes() stands
+   where rocalCreateCOCOReader() & co. stand (before the augmentations are added); the boxes of a batch (l,t,r,b in pixels
+   of the decoded image, `counts[i]` per sample, all samples back to back) are handed in before rocalRun() and the
+   transformed ones are read back after it, in the same layout. ---- */
+extern "C" RocalStatus ROCAL_API_CALL rocalEnableBoundingBoxes(RocalContext context);
+extern "C" RocalStatus ROCAL_API_CALL rocalSetBoundingBoxes(RocalContext context, const unsigned *counts, const float *ltrb, const int *labels);
+extern "C" unsigned ROCAL_API_CALL rocalGetBoundingBoxCount(RocalContext context, unsigned *counts);  // returns the total
+extern "C" RocalStatus ROCAL_API_CALL rocalGetBoundingBoxCords(RocalContext context, float *ltrb);
+extern "C" RocalStatus ROCAL_API_CALL rocalGetBoundingBoxLabel(RocalContext context, int *labels);
+
 /* ---- parameters (rocal_api_parameters.h:39-161) ---- */
 extern "C" void ROCAL_API_CALL rocalSetSeed(unsigned seed);
 extern "C" unsigned ROCAL_API_CALL rocalGetSeed();

@@ -180,3 +180,121 @@ def test_api_errors_follow_the_reference(tmp_path):
         f.write("%d %d %d\n" % (N, H, W) + "".join("%d %d\n" % r for r in ROIS))
     p = subprocess.run([HOST_CHECK, "pipeline", "errors", str(tmp_path)], capture_output=True, text=True, timeout=110)
     assert p.returncode == 0 and "errors_bad_mask 0" in p.stdout, (p.returncode, p.stdout, p.stderr[-2000:])
+
+
+# ---------------------------------------------------------------- bounding boxes through the metadata nodes
+
+def _boxes():
+    """Per sample: a list of (l, t, r, b) inside the sample's ROI and a list of labels; one sample has no box."""
+    rng = np.random.default_rng(8)
+    boxes, labels = [], []
+    for i, (w, h) in enumerate(ROIS):
+        k = 0 if i == 3 else int(rng.integers(1, 5))
+        bs = []
+        for _ in range(k):
+            l, t = rng.uniform(0, w * 0.7), rng.uniform(0, h * 0.7)
+            bs.append((np.float32(l), np.float32(t), np.float32(min(w, l + rng.uniform(4, w * 0.6))), np.float32(min(h, t + rng.uniform(4, h * 0.6)))))
+        boxes.append(bs)
+        labels.append([int(x) for x in rng.integers(1, 90, k)])
+    return boxes, labels
+
+
+def _run_meta(scenario, tmp_path):
+    from oracle import meta  # noqa: F401  (imported here so that a missing file fails this test only)
+    boxes, labels = _boxes()
+    with open(tmp_path / "boxes.txt", "w") as f:
+        for bs, ls in zip(boxes, labels):
+            f.write("%d\n" % len(bs))
+            for b, l in zip(bs, ls):
+                f.write("%.9g %.9g %.9g %.9g %d\n" % (b[0], b[1], b[2], b[3], l))
+    img = _image()
+    img.tofile(tmp_path / "input.bin")
+    with open(tmp_path / "meta.txt", "w") as f:
+        f.write("%d %d %d\n" % (N, H, W))
+        for w, h in ROIS:
+            f.write("%d %d\n" % (w, h))
+    print("host_check pipeline", scenario, flush=True)
+    p = subprocess.run([HOST_CHECK, "pipeline", scenario, str(tmp_path)], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, (p.returncode, p.stdout, p.stderr)
+    got = []
+    for b in range(2):
+        tok = open(tmp_path / ("boxes_b%d.txt" % b)).read().split()
+        k, batch = 0, []
+        for _ in range(N):
+            c = int(tok[k]); k += 1
+            bs, ls = [], []
+            for _ in range(c):
+                bs.append(tuple(np.float32(float(v)) for v in tok[k:k + 4]))
+                ls.append(int(tok[k + 4]))
+                k += 5
+            batch.append((bs, ls))
+        got.append(batch)
+    return boxes, labels, got
+
+
+def _same_boxes(got, exp, what, rtol=0.0):
+    gb, gl = got
+    eb, el = exp
+    assert len(gb) == len(eb), (what, gb, eb)
+    assert gl[:len(el)] == el and all(v == 0 for v in gl[len(el):]), (what, gl, el)
+    for g, e in zip(gb, eb):
+        if rtol:
+            assert np.allclose(np.array(g, np.float32), np.array(e, np.float32), rtol=rtol, atol=1e-4), (what, g, e)
+        else:
+            assert np.array_equal(np.array(g, np.float32).view(np.uint32), np.array(e, np.float32).view(np.uint32)), (what, g, e)
+
+
+def test_boxes_through_crop_mirror_normalize(tmp_path):
+    from oracle import meta
+    boxes, labels, got = _run_meta("meta_cmn", tmp_path)
+    crop = np.stack([orc.fixed_crop(w, h, 48, 40, anchor=(0.5, 0.5)) for w, h in ROIS])
+    mirrors = _coin_batches(2)
+    for b in range(2):
+        for i in range(N):
+            x1, y1, cw, ch = (int(v) for v in crop[i])
+            _same_boxes(got[b][i], meta.crop_mirror_normalize(boxes[i], labels[i], x1, y1, cw, ch, int(mirrors[b][i])), "cmn boxes, batch %d sample %d" % (b, i))
+
+
+def test_boxes_through_resize_then_flip(tmp_path):
+    from oracle import meta
+    boxes, labels, got = _run_meta("meta_resize_flip", tmp_path)
+    for i, (w, h) in enumerate(ROIS):
+        rb, rl = meta.resize(boxes[i], labels[i], w, h, 40, 32)
+        _same_boxes(got[1][i], meta.flip(rb, rl, 40, 32, 1, 1), "resize+flip boxes, sample %d" % i)
+
+
+def test_boxes_through_rotate(tmp_path):
+    """cos and sin come from the C library on one side and from Python's on the other: compared to 1e-5."""
+    from oracle import meta
+    boxes, labels, got = _run_meta("meta_rotate", tmp_path)
+    for i, (w, h) in enumerate(ROIS):
+        _same_boxes(got[0][i], meta.rotate(boxes[i], labels[i], w, h, W, H, 30.0), "rotate boxes, sample %d" % i, rtol=1e-5)
+
+
+def test_boxes_through_resize_crop_mirror(tmp_path):
+    from oracle import meta
+    boxes, labels, got = _run_meta("meta_rcm", tmp_path)
+    window = np.stack([orc.fixed_crop(w, h, 50, 40) for w, h in ROIS])
+    for i in range(N):
+        x1, y1, cw, ch = (int(v) for v in window[i])
+        _same_boxes(got[1][i], meta.resize_crop_mirror(boxes[i], labels[i], x1, y1, x1 + cw, y1 + ch, 36, 28, 1), "rcm boxes, sample %d" % i)
+
+
+def test_boxes_through_crop_then_resize_mirror_normalize(tmp_path):
+    from oracle import meta
+    boxes, labels, got = _run_meta("meta_crop_then_rmn", tmp_path)
+    placed = np.stack([orc.fixed_crop(w, h, 30, 20, x1=5, y1=7) for w, h in ROIS])
+    for i in range(N):
+        x1, y1, cw, ch = (int(v) for v in placed[i])
+        cb, cl = meta.crop(boxes[i], labels[i], x1, y1, cw, ch)
+        _same_boxes(got[0][i], meta.resize_mirror_normalize(cb, cl, cw, ch, 60, 40, 1), "crop+rmn boxes, sample %d" % i)
+
+
+def test_boxes_through_crop_resize(tmp_path):
+    from oracle import meta
+    boxes, labels, got = _run_meta("meta_crop_resize", tmp_path)
+    s = orc.FParam.simple
+    window = np.stack([orc.random_crop(s(0.5), s(1.2), s(0.3), s(0.7), w, h) for w, h in ROIS])
+    for i in range(N):
+        x1, y1, cw, ch = (int(v) for v in window[i])
+        _same_boxes(got[1][i], meta.crop_resize(boxes[i], labels[i], x1, y1, x1 + cw, y1 + ch, 64, 64), "crop-resize boxes, sample %d" % i)
