@@ -127,3 +127,35 @@ def test_oracle_crop_laws_known_answers():
     assert list(orc.random_crop(s(1.0), s(1.0), s(0.5), s(0.5), 100, 300)) == [0, (300 - 133) // 2, 100, 133]
     # factor crop: trunc(.5*101)=50, trunc(.25*80)=20; drifts trunc(.5*51)=25, trunc(.99*60)=59
     assert list(orc.factor_crop(s(0.25), s(0.5), s(0.5), s(0.99), 101, 80)) == [25, 59, 50, 20]
+
+
+# ---------------------------------------------------------------- metadata laws: the restatement against hand-computed cases
+
+def test_box_laws_known_answers():
+    from oracle import meta
+    f = np.float32
+    boxes, labels = [(10, 10, 50, 40), (0, 0, 5, 5), (28, 20, 60, 60)], [3, 4, 5]
+    # crop window (5,7)+(30x20): box 0 keeps 425/1200 of its area (kept, clipped, shifted); box 1 is outside;
+    # box 2 keeps 7*7/1280 (dropped)
+    assert meta.crop(boxes, labels, 5, 7, 30, 20) == ([(f(5), f(3), f(30), f(20))], [3])
+    # nothing left -> the whole crop with label 0
+    assert meta.crop([(0, 0, 5, 5)], [9], 50, 50, 10, 8) == ([(f(0), f(0), f(10), f(8))], [0])
+    # mirror inside the crop: l' = w - r, r' = w - l
+    assert meta.crop_mirror_normalize(boxes[:1], labels[:1], 5, 7, 30, 20, 1) == ([(f(0), f(3), f(25), f(20))], [3])
+    # crop + resize by exactly 2 in x and 3 in y
+    assert meta.crop_resize(boxes[:1], labels[:1], 5, 7, 35, 27, 60, 60) == ([(f(10), f(9), f(60), f(60))], [3])
+    # resize-crop-mirror: mirror in the crop frame, then scale
+    assert meta.resize_crop_mirror(boxes[:1], labels[:1], 5, 7, 35, 27, 60, 60, 1) == ([(f(0), f(9), f(50), f(60))], [3])
+    # plain resize doubles; an empty sample gets one zero box and no label
+    assert meta.resize([(1, 2, 3, 4)], [7], 10, 10, 20, 20) == ([(f(2), f(4), f(6), f(8))], [7])
+    assert meta.resize([], [], 10, 10, 20, 20) == ([(f(0), f(0), f(0), f(0))], [])
+    # resize-mirror-normalize mirrors with the "- 1" of the reference
+    assert meta.resize_mirror_normalize([(1, 2, 3, 4)], [7], 10, 10, 20, 20, 1) == ([(f(13), f(4), f(17), f(8))], [7])
+    # flipping twice is the identity
+    once = meta.flip([(1, 2, 3, 4)], [7], 10, 8, 1, 1)
+    assert once == ([(f(7), f(4), f(9), f(6))], [7]) and meta.flip(*once, 10, 8, 1, 1) == ([(f(1), f(2), f(3), f(4))], [7])
+    # rotation by 0 degrees about equal centres keeps the box (its left/top are min(0, .) first, then clipped to the image)
+    assert meta.rotate([(10, 10, 50, 40)], [3], 96, 80, 96, 80, 0.0) == ([(f(0), f(0), f(50), f(40))], [3])
+    # overlap measure: intersection over the first box's area, or over the union
+    assert meta.overlap((0, 0, 10, 10), (5, 5, 15, 15)) == 0.25
+    assert abs(meta.overlap((0, 0, 10, 10), (5, 5, 15, 15), True) - 25.0 / 175.0) < 1e-7
