@@ -76,6 +76,14 @@ RMX_API const char *rmx_version(void);
  * (rocAL swaps them every batch, rocAL/source/pipeline/tensor.cpp:478-489). Asynchronous. */
 RMX_API int rmx_op_launch(rmx_op *op, const void *src, void *dst);
 RMX_API int rmx_op_destroy(rmx_op *op);
+/* Ragged source: instead of one padded [N,Hmax,Wmax,3] tensor the images of a batch lie tightly packed (row stride =
+ * width*3) at byte `offsets[i]` of ONE device buffer of `buffer_bytes`, each with its own `widths[i]` x `heights[i]`
+ * (<= the w x h of the source descriptor, which then only bounds the sizes). ROIs of later updates are relative to each
+ * image. Takes effect with the next rmx_update_* of the op and stays until called again; all three arrays NULL go
+ * back to the padded tensor. Stands where rocAL copies every decoded image into the padded batch
+ * (rocAL/source/loaders/image/image_read_and_decode.cpp:165-390, circular_buffer.cpp:88-133): a C1 batch is
+ * 315 MB padded for about 80 MB of pixels. */
+RMX_API int rmx_op_set_ragged_source(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights, uint64_t buffer_bytes);
 /* Algorithmic bytes of the last update: sum of source-window bytes + destination bytes. */
 RMX_API uint64_t rmx_op_algorithmic_bytes(const rmx_op *op);
 /* Launch plan of the last update as text (waves, strips, LDS per wave ...), for logs and benchmarks. */

@@ -72,7 +72,11 @@ struct rmx_op {
     bool norm = false, quant = false;
     int n = 0;
 
-    RmxSample *h_table[TABLE_RING] = {};  // pinned
+    RmxSample *h_table[TABLE_RING] = {};  // pinned; n rows, then n source layout entries
+    std::vector<RmxSrcLayout> layout;     // ragged source (empty: one padded tensor); copied behind the rows on every update
+    uint64_t ragged_bytes = 0;            // extent of the ragged source buffer
+    bool slot_ragged[TABLE_RING] = {};    // what the table slot was committed with
+    uint64_t slot_src_bytes[TABLE_RING] = {};
     RmxSample *d_table[TABLE_RING] = {};
     hipEvent_t uploaded[TABLE_RING] = {};
     int cur = -1;  // slot of the last update, -1 before the first
@@ -120,7 +124,7 @@ int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor
     op->dst = *dst;
     op->roi_type = roi_type;
     op->n = (int)src->n;
-    size_t bytes = sizeof(RmxSample) * (size_t)op->n;
+    size_t bytes = (sizeof(RmxSample) + sizeof(RmxSrcLayout)) * (size_t)op->n;
     for (int i = 0; i < TABLE_RING; i++) {
         hipError_t e = hipHostMalloc((void **)&op->h_table[i], bytes, hipHostMallocDefault);
         if (e == hipSuccess) e = hipMalloc((void **)&op->d_table[i], bytes);
@@ -145,17 +149,28 @@ int next_slot(rmx_op *op, RmxSample **row) {
 }
 
 int commit_slot(rmx_op *op, int slot) {
-    HIP_TRY(hipMemcpyAsync(op->d_table[slot], op->h_table[slot], sizeof(RmxSample) * (size_t)op->n,
-                           hipMemcpyHostToDevice, op->ctx->stream));
+    size_t bytes = sizeof(RmxSample) * (size_t)op->n;
+    if (!op->layout.empty()) {
+        memcpy(reinterpret_cast<char *>(op->h_table[slot]) + bytes, op->layout.data(), sizeof(RmxSrcLayout) * (size_t)op->n);
+        bytes += sizeof(RmxSrcLayout) * (size_t)op->n;
+    }
+    op->slot_ragged[slot] = !op->layout.empty();
+    op->slot_src_bytes[slot] = op->ragged_bytes;
+    HIP_TRY(hipMemcpyAsync(op->d_table[slot], op->h_table[slot], bytes, hipMemcpyHostToDevice, op->ctx->stream));
     HIP_TRY(hipEventRecord(op->uploaded[slot], op->ctx->stream));
     op->cur = slot;
     return RMX_OK;
 }
 
+// image size of sample i: its own when the source is ragged, the padded tensor's otherwise
+inline uint32_t sample_w(const rmx_op *op, int i) { return op->layout.empty() ? op->src.w : op->layout[i].row_stride / 3u; }
+inline uint32_t sample_h(const rmx_op *op, int i) { return op->layout.empty() ? op->src.h : op->layout[i].rows; }
+
 // ROI in the caller's convention -> x,y,w,h clipped to the padded source tensor.
 int read_roi(const rmx_op *op, const uint32_t *roi, int i, int32_t *x, int32_t *y, int32_t *w, int32_t *h) {
+    const uint32_t sw = sample_w(op, i), sh = sample_h(op, i);
     if (!roi) {
-        *x = 0; *y = 0; *w = (int32_t)op->src.w; *h = (int32_t)op->src.h;
+        *x = 0; *y = 0; *w = (int32_t)sw; *h = (int32_t)sh;
         return RMX_OK;
     }
     uint32_t a = roi[i * 4], b = roi[i * 4 + 1], c = roi[i * 4 + 2], d = roi[i * 4 + 3];
@@ -164,9 +179,9 @@ int read_roi(const rmx_op *op, const uint32_t *roi, int i, int32_t *x, int32_t *
         c -= a;
         d -= b;
     }
-    if (a >= op->src.w || b >= op->src.h) return fail(RMX_ERR_INVALID, "sample %d: roi origin (%u,%u) outside the %ux%u source", i, a, b, op->src.w, op->src.h);
-    if (c > op->src.w - a) c = op->src.w - a;
-    if (d > op->src.h - b) d = op->src.h - b;
+    if (a >= sw || b >= sh) return fail(RMX_ERR_INVALID, "sample %d: roi origin (%u,%u) outside the %ux%u source", i, a, b, sw, sh);
+    if (c > sw - a) c = sw - a;
+    if (d > sh - b) d = sh - b;
     *x = (int32_t)a; *y = (int32_t)b; *w = (int32_t)c; *h = (int32_t)d;
     return RMX_OK;
 }
@@ -282,7 +297,8 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.src = (const uint8_t *)src;
     a.dst = dst;
     a.table = op->d_table[op->cur];
-    a.src_bytes = (uint64_t)op->src.n * op->src.h * op->src.w * op->src.c;
+    a.src_bytes = op->slot_ragged[op->cur] ? op->slot_src_bytes[op->cur] : (uint64_t)op->src.n * op->src.h * op->src.w * op->src.c;
+    a.layout = op->slot_ragged[op->cur] ? reinterpret_cast<const RmxSrcLayout *>(op->d_table[op->cur] + op->n) : nullptr;
     a.n = op->n;
     a.src_h = (int)op->src.h;
     a.src_w = (int)op->src.w;
@@ -317,6 +333,33 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     return RMX_OK;
 }
 
+/* ------------------------------------------------------------------ ragged sources */
+
+int rmx_op_set_ragged_source(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights, uint64_t buffer_bytes) {
+    if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
+    if (!offsets && !widths && !heights) {  // back to one padded tensor
+        op->layout.clear();
+        op->ragged_bytes = 0;
+        return RMX_OK;
+    }
+    if (!offsets || !widths || !heights) return fail(RMX_ERR_INVALID, "offsets, widths and heights are required together");
+    std::vector<RmxSrcLayout> l((size_t)op->n);
+    for (int i = 0; i < op->n; i++) {
+        if (widths[i] == 0 || heights[i] == 0 || widths[i] > op->src.w || heights[i] > op->src.h)
+            return fail(RMX_ERR_INVALID, "sample %d: image of %u x %u is empty or exceeds the %u x %u of the source descriptor", i, widths[i], heights[i], op->src.w, op->src.h);
+        const uint64_t bytes = (uint64_t)widths[i] * heights[i] * 3;
+        if (offsets[i] > buffer_bytes || bytes > buffer_bytes - offsets[i])
+            return fail(RMX_ERR_INVALID, "sample %d: %llu bytes at offset %llu do not fit the buffer of %llu bytes", i, (unsigned long long)bytes, (unsigned long long)offsets[i],
+                        (unsigned long long)buffer_bytes);
+        l[i].offset = offsets[i];
+        l[i].row_stride = widths[i] * 3u;
+        l[i].rows = heights[i];
+    }
+    op->layout.swap(l);
+    op->ragged_bytes = buffer_bytes;
+    return RMX_OK;
+}
+
 /* ------------------------------------------------------------------ K1 family */
 
 static int create_k1(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, bool norm, rmx_op **out) {
@@ -341,8 +384,8 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
             if (rc) return rc;
         } else {  // whole padded image
             s.src_x = s.src_y = 0;
-            s.src_w = (int32_t)op->src.w;
-            s.src_h = (int32_t)op->src.h;
+            s.src_w = (int32_t)sample_w(op, i);
+            s.src_h = (int32_t)sample_h(op, i);
         }
         s.dst_w = std::min<int32_t>(s.src_w, (int32_t)op->dst.w);
         s.dst_h = std::min<int32_t>(s.src_h, (int32_t)op->dst.h);

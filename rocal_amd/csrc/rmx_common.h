@@ -27,6 +27,15 @@ struct __attribute__((aligned(16))) RmxSample {
 };
 static_assert(sizeof(RmxSample) == 128, "parameter table row must stay 128 bytes");
 
+// Where a sample's image lies when the source is not one padded [N,Hmax,Wmax,3] tensor: tightly packed images of
+// different sizes, one after the other (or anywhere) in one buffer.
+struct RmxSrcLayout {
+    uint64_t offset;      // bytes from the source base to the sample's first pixel
+    uint32_t row_stride;  // bytes per image row
+    uint32_t rows;        // image height
+};
+static_assert(sizeof(RmxSrcLayout) == 16, "source layout entry must stay 16 bytes");
+
 enum : uint32_t { RMX_S_HFLIP = 1u, RMX_S_VFLIP = 2u, RMX_S_CHREV = 4u /* output channel k reads source channel 2-k */ };
 
 struct RmxKArgs {
@@ -42,6 +51,7 @@ struct RmxKArgs {
     int32_t aux0, aux1;
     int32_t wpb;             // wavefronts per workgroup of this launch
     uint32_t nblocks;        // workgroups of this launch
+    const RmxSrcLayout *layout;  // per-sample source placement, or null: sample s starts at s*src_h*src_w*3
 };
 
 #define RMX_WAVE 64

@@ -24,6 +24,17 @@ RMX_DEV float round_u8(float v) {
     return __builtin_fminf(__builtin_fmaxf(v, 0.0f), 255.0f);
 }
 
+// First pixel and row stride (bytes) of sample s: from the layout table of a ragged source, else the padded batch.
+RMX_DEV const uint8_t *sample_base(const RmxKArgs &a, int s, uint32_t &row_stride) {
+    if (a.layout) {
+        const RmxSrcLayout L = a.layout[s];
+        row_stride = L.row_stride;
+        return a.src + L.offset;
+    }
+    row_stride = (uint32_t)a.src_w * 3u;
+    return a.src + (size_t)s * a.src_h * row_stride;
+}
+
 // Order LDS traffic between the lanes of one wavefront. A wave's DS instructions execute in
 // issue order, so no hardware barrier is needed: this only stops the compiler from moving
 // LDS reads above the writes they depend on.

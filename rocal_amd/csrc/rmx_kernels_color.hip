@@ -73,8 +73,9 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     const int x1 = P.src_x, y1 = P.src_y;
     const float p0 = P.color[0], p1 = P.color[1], p2 = P.color[2], p3 = P.color[3];
 
-    const size_t row_stride = (size_t)a.src_w * 3;
-    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    uint32_t row_stride32;
+    const uint8_t *simg = sample_base(a, s, row_stride32);
+    const size_t row_stride = row_stride32;
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
 

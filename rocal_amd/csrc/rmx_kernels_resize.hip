@@ -136,9 +136,8 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
     }
 
     StageCtx S;
-    S.row_stride = (uint32_t)a.src_w * 3u;
     {
-        const uint8_t *simg = a.src + (size_t)s * a.src_h * S.row_stride;
+        const uint8_t *simg = sample_base(a, s, S.row_stride);
         S.skew = (uint32_t)((uintptr_t)simg & 3u);
         S.base4 = simg - S.skew;
         const uint64_t left = (uint64_t)((a.src + a.src_bytes) - S.base4);

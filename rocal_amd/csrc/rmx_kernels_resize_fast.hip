@@ -81,8 +81,8 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
     }
 
     // source addressing: dword-aligned base below the sample, 32-bit byte offsets from it
-    const uint32_t row_stride = (uint32_t)a.src_w * 3u;
-    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    uint32_t row_stride;
+    const uint8_t *simg = sample_base(a, s, row_stride);
     const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
     const uint8_t *base4 = simg - skew;
     const uint64_t left = (uint64_t)((a.src + a.src_bytes) - base4);

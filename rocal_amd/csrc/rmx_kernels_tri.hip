@@ -81,8 +81,9 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
     const int kx_cap = P.strip_rows & 0xffff;
     const int ring_mask = ring_rows - 1;
 
-    const size_t row_stride = (size_t)a.src_w * 3;
-    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    uint32_t row_stride32;
+    const uint8_t *simg = sample_base(a, s, row_stride32);
+    const size_t row_stride = row_stride32;
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
 
@@ -345,8 +346,8 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
     const int kx = ax.ksize, ky = ay.ksize;
 
     // (a sample is smaller than 4 GiB: the host checks it, so offsets inside a sample are 32-bit)
-    const uint32_t row_stride = (uint32_t)a.src_w * 3u;
-    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    uint32_t row_stride;
+    const uint8_t *simg = sample_base(a, s, row_stride);
     const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
     const uint8_t *base4 = simg - skew;  // dword-aligned base below the sample
     const uint8_t *buf_end = a.src + a.src_bytes;

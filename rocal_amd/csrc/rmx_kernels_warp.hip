@@ -59,8 +59,8 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const float dcx = (float)(dw >> 1), dcy = (float)(dh >> 1);
     const float scx = (float)(xlo + (P.src_w >> 1)), scy = (float)(ylo + (P.src_h >> 1));
 
-    const uint32_t row_stride = (uint32_t)a.src_w * 3u;
-    const uint8_t *simg = a.src + (size_t)s * a.src_h * row_stride;
+    uint32_t row_stride;
+    const uint8_t *simg = sample_base(a, s, row_stride);
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
     uint32_t *lds = rmx_lds_warp + (size_t)wib * (a.lds_bytes >> 2);

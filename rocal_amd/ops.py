@@ -104,7 +104,8 @@ class Op:
         """src/dst: torch CUDA tensors (the batch buffers). Asynchronous on the context's stream."""
         assert src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()
         sd, dd = self.src_desc, self.dst_desc
-        assert src.numel() * src.element_size() >= sd.n * sd.h * sd.w * sd.c, "source buffer smaller than its descriptor"
+        need = getattr(self, "_ragged_bytes", None) or sd.n * sd.h * sd.w * sd.c
+        assert src.numel() * src.element_size() >= need, "source buffer smaller than its descriptor"
         esz = {FP32: 4, FP16: 2, UINT8: 1}[dd.dtype]
         assert dst.numel() * dst.element_size() >= dd.n * dd.h * dd.w * dd.c * esz, "destination buffer smaller than its descriptor"
         check(_lib.lib().rmx_op_launch(self._h, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())))
@@ -114,6 +115,19 @@ class Op:
         d = self.dst_desc
         shape = (d.n, d.c, d.h, d.w) if d.layout == NCHW else (d.n, d.h, d.w, d.c)
         return t.full(shape, fill, dtype=torch_dtype(d.dtype), device="cuda:%d" % self.ctx.device)
+
+    def set_ragged_source(self, offsets, widths, heights, buffer_bytes):
+        """The batch's images lie tightly packed at byte `offsets` of one buffer (None, None, None: padded tensor again)."""
+        if offsets is None:
+            check(_lib.lib().rmx_op_set_ragged_source(self._h, None, None, None, 0))
+            self._ragged_bytes = None
+            return
+        self._ragged_bytes = int(buffer_bytes)
+        o = np.ascontiguousarray(offsets, np.uint64)
+        w = np.ascontiguousarray(widths, np.uint32)
+        h = np.ascontiguousarray(heights, np.uint32)
+        check(_lib.lib().rmx_op_set_ragged_source(self._h, o.ctypes.data_as(C.c_void_p), w.ctypes.data_as(C.c_void_p), h.ctypes.data_as(C.c_void_p),
+                                                  int(buffer_bytes)))
 
     @property
     def algorithmic_bytes(self):

@@ -204,3 +204,103 @@ def test_random_warp(ctx, seed):
     ctx.sync()
     got = out.cpu().numpy()
     assert np.array_equal(got, exp), "seed %d (%s): %d values differ" % (seed, op.plan, int((got != exp).sum()))
+
+
+def _ragged(rng, n, H, W):
+    """n images of their own sizes (<= H x W): packed one after the other at arbitrary byte offsets of one buffer,
+    and the same images in the top-left corners of a padded [n,H,W,3] tensor for the oracle."""
+    import torch
+    ws = rng.integers(max(1, W // 3), W + 1, n).astype(np.uint32)
+    hs = rng.integers(max(1, H // 3), H + 1, n).astype(np.uint32)
+    padded = np.zeros((n, H, W, 3), np.uint8)
+    chunks, offsets, pos = [], [], int(rng.integers(0, 2)) * 4
+    lead = pos
+    for i in range(n):
+        im = rng.integers(0, 256, (hs[i], ws[i], 3), dtype=np.uint8)
+        padded[i, :hs[i], :ws[i]] = im
+        gap = int(rng.integers(0, 6))
+        offsets.append(pos + gap)
+        chunks.append(np.zeros(gap, np.uint8))
+        chunks.append(im.reshape(-1))
+        pos += gap + im.size
+    buf = np.concatenate([np.zeros(lead, np.uint8)] + chunks)
+    return padded, torch.from_numpy(buf).cuda(), np.array(offsets, np.uint64), ws, hs, buf.size
+
+
+def _roi_in(rng, ws, hs):
+    roi = np.empty((len(ws), 4), np.uint32)
+    for i, (w, h) in enumerate(zip(ws, hs)):
+        rw, rh = int(rng.integers(1, w + 1)), int(rng.integers(1, h + 1))
+        roi[i] = (int(rng.integers(0, w - rw + 1)), int(rng.integers(0, h - rh + 1)), rw, rh)
+    return roi
+
+
+@pytest.mark.parametrize("seed", range(30))
+def test_random_ops_on_a_ragged_source(ctx, seed):
+    """Every kernel family reading tightly packed images of different sizes instead of a padded tensor."""
+    rng = np.random.default_rng(6000 + seed)
+    n = int(rng.integers(1, 5))
+    H, W = int(rng.integers(12, 140)), int(rng.integers(12, 180))
+    padded, buf, offsets, ws, hs, nbytes = _ragged(rng, n, H, W)
+    roi = _roi_in(rng, ws, hs)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    family = seed % 5
+    inv = (1 / wl.STD).astype(np.float32)
+    scale, bias = np.tile(inv, n), np.tile(-(wl.MEAN * inv), n)
+    mirror = rng.integers(0, 2, n).astype(np.uint32)
+    if family in (0, 1, 2):  # resize: linear (also the aligned fast path), nearest, triangular
+        interp = [ops.LINEAR, ops.NEAREST, ops.TRIANGULAR][family]
+        dw = (rng.integers(1, 16, n) * 8).astype(np.uint32) if seed % 2 else rng.integers(1, 120, n).astype(np.uint32)
+        dh = rng.integers(1, 100, n).astype(np.uint32)
+        oh, ow = int(dh.max()), int(dw.max())
+        op = ops.Resize(ctx, sd, ops.desc(n, oh, ow, ops.NCHW, ops.FP16), interp)
+        op.set_ragged_source(offsets, ws, hs, nbytes)
+        op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        exp = orc.resize(padded, roi, dw, dh, oh, ow, interp=interp, mirror=mirror, scale=scale, bias=bias, layout=orc.NCHW, dtype=orc.FP16)
+    elif family == 3:
+        if seed % 2:
+            roi[:, 2] = np.maximum(1, roi[:, 2] // 8 * 8)
+        oh, ow = int(roi[:, 3].max()), int(roi[:, 2].max())
+        op = ops.CropMirrorNormalize(ctx, sd, ops.desc(n, oh, ow, ops.NCHW, ops.FP32))
+        op.set_ragged_source(offsets, ws, hs, nbytes)
+        op.update(roi, scale, bias, mirror)
+        exp = orc.crop_mirror_normalize(padded, roi, scale, bias, mirror, oh, ow, orc.NCHW, orc.FP32)
+    else:
+        if seed % 2:
+            f = lambda lo, hi: rng.uniform(lo, hi, n).astype(np.float32)
+            p = (f(0.5, 1.8), f(-30, 30), f(-180, 180), f(0.0, 2.0))
+            op = ops.ColorTwist(ctx, sd, sd)
+            op.set_ragged_source(offsets, ws, hs, nbytes)
+            op.update(roi, *p)
+            exp = orc.color_twist(padded, roi, *p)
+        else:
+            affine = np.empty((n, 6), np.float32)
+            for i in range(n):
+                ang, sc = rng.uniform(-np.pi, np.pi), rng.uniform(0.5, 2.0)
+                affine[i] = (np.cos(ang) * sc, np.sin(ang) * sc, -np.sin(ang) * sc, np.cos(ang) * sc, rng.uniform(-8, 8), rng.uniform(-8, 8))
+            dw = np.minimum(rng.integers(1, 160, n), W).astype(np.uint32)
+            dh = np.minimum(rng.integers(1, 120, n), H).astype(np.uint32)
+            op = ops.WarpAffine(ctx, sd, sd, ops.LINEAR)
+            op.set_ragged_source(offsets, ws, hs, nbytes)
+            op.update(roi, affine, dw, dh)
+            exp = orc.warp_affine(padded, roi, np.stack([orc.affine_from_rocal(a) for a in affine]), dw, dh, H, W, interp=orc.LINEAR)
+    out = op.alloc_output()
+    op.launch(buf, out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    assert np.array_equal(_bits(got), _bits(exp)), "seed %d family %d (%s, %s): %d values differ" % (seed, family, op.kernel_name, op.plan, int((got != exp).sum()))
+    # and back to the padded tensor with the same op
+    import torch
+    op.set_ragged_source(None, None, None, 0)
+    if family in (0, 1, 2):
+        op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    elif family == 3:
+        op.update(roi, scale, bias, mirror)
+    elif seed % 2:
+        op.update(roi, *p)
+    else:
+        op.update(roi, affine, dw, dh)
+    out2 = op.alloc_output()
+    op.launch(torch.from_numpy(padded).cuda(), out2)
+    ctx.sync()
+    assert np.array_equal(_bits(out2.cpu().numpy()), _bits(exp))
