@@ -14,31 +14,32 @@ enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
 
 // Branch-free: every choice is a select. Lanes of a wavefront hold pixels of different hue sectors, so
 // branches would run every case one after the other under changing execution masks.
-RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, float alpha, float beta, float shift, float satf) {
+RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, float alpha, float beta, float shift, float shift2, float shift4, float satf) {
     const float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
     const float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
     const float delta = cmax - cmin;
     const float rd = rcp[(int)delta];      // 0 when delta == 0
     float s = delta * rcp[(int)cmax];
-    const bool is_r = cmax == r, is_g = cmax == g, grey = delta == 0.0f;
-    float num = is_r ? (g - b) : (is_g ? (b - r) : (r - g));
-    float add = is_r ? 0.0f : (is_g ? 2.0f : 4.0f);
-    num = grey ? 0.0f : num;
-    add = grey ? 0.0f : add;
-    float hh = __builtin_fmaf(num, rd, add + shift);
+    // A grey pixel needs no case of its own: r == g == b makes it a "red is largest" pixel with g - b == 0.
+    const bool is_r = cmax == r, is_g = cmax == g;
+    const float num = is_r ? (g - b) : (is_g ? (b - r) : (r - g));
+    // sextant offset 0 / 2 / 4 plus the hue shift, the three sums made once per sample
+    const float add = is_r ? shift : (is_g ? shift2 : shift4);
+    float hh = __builtin_fmaf(num, rd, add);
     hh = hh < 0.0f ? hh + 6.0f : hh;
     hh = hh >= 6.0f ? hh - 6.0f : hh;
     s = s * satf;
     s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
-    const int hi = (int)hh;
-    const float hf = hh - (float)hi;
+    // sector and fraction: hh - (float)(int)hh, with the truncation kept in floating point
+    const float hi = __builtin_truncf(hh);
+    const float hf = hh - hi;
     const float vsat = cmax * s;
     const float vsatf = vsat * hf;
     const float pp = cmax - vsat;
     const float qq = cmax - vsatf;
     const float tt = pp + vsatf;
     // sector table (hi >= 5 is the last sector):  r: V q p p t V   g: t V V q p p   b: p p t V V q
-    const bool h0 = hi == 0, h1 = hi == 1, h2 = hi == 2, h3 = hi == 3, h4 = hi == 4;
+    const bool h0 = hi == 0.0f, h1 = hi == 1.0f, h2 = hi == 2.0f, h3 = hi == 3.0f, h4 = hi == 4.0f;
     const float ro = h1 ? qq : ((h2 || h3) ? pp : (h4 ? tt : cmax));
     const float go = h0 ? tt : ((h1 || h2) ? cmax : (h3 ? qq : pp));
     const float bo = (h0 || h1) ? pp : (h2 ? tt : ((h3 || h4) ? cmax : qq));
@@ -83,7 +84,7 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
 #pragma unroll
         for (int k = 0; k < PX; k++) {
             if constexpr (KIND == COLOR_TWIST) {
-                twist_px(v[0][k], v[1][k], v[2][k], rcp, p0, p1, p2, p3);
+                twist_px(v[0][k], v[1][k], v[2][k], rcp, p0, p1, p2, p2 + 2.0f, p2 + 4.0f, p3);
             } else {
 #pragma unroll
                 for (int c = 0; c < 3; c++) v[c][k] = __builtin_fmaf(v[c][k] - p2, p0, p1);
