@@ -200,7 +200,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--config", type=int, default=1)
-    ap.add_argument("--all", action="store_true", help="also measure the other configurations (written to gpurun_out/bench_all.json)")
+    ap.add_argument("--all", action="store_true", help="also measure the other configurations (one JSON object per configuration, written to bench_all.json in the output folder)")
     ap.add_argument("--no-cpu", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
