@@ -5,7 +5,7 @@ A step is one pass of the hot path over one batch: the launch that replaces vxPr
 the fused node (what rocAL's own process timer brackets). Inputs and the per-batch parameter
 table are resident in HBM when the timed region starts. Prints ONE JSON line on stdout.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..4] [--all] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..6] [--all] [--no-cpu]
 """
 import argparse
 import json
@@ -26,6 +26,9 @@ WORKLOADS = {
     2: "C2 ColorTwist 224x224 u8->u8 NHWC batch 256 (configs[2])",
     3: "C3 WarpAffine 512x512 u8->u8 NHWC batch 128 (configs[3])",
     4: "C4 triangular 1920x1080->640x360 +normalize fp16 NCHW batch 32 (configs[4])",
+    # the rows next to the path (measured with --all or --config; not the benchmark's configurations)
+    5: "N1 ToTensor 224x224 u8 NHWC -> fp16 NCHW, reversed channels, batch 256",
+    6: "N2 C1 (RandomResizedCrop+CropMirrorNormalize ->224x224 fp16 NCHW batch 256) reading a ragged, tightly packed source",
 }
 
 
@@ -96,6 +99,39 @@ def build_case(cfg, ctx, n=None):
             from oracle import orc
             return orc.resize(c["img"][:k], c["roi"][:k], dw[:k], dh[:k], 360, 640, interp=orc.TRIANGULAR, mirror=c["mirror"][:k],
                               scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16)
+    elif cfg == 5:
+        n = n or 256
+        c = wl.config2(n)
+        mul = (1 / wl.STD).astype(np.float32)
+        add = (-(wl.MEAN / wl.STD)).astype(np.float32)
+        op = ops.ToTensor(ctx, ops.desc(n, 224, 224, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16))
+        op.update(mul, add, reverse_channels=True)
+
+        def cpu(k):
+            from oracle import orc
+            return orc.to_tensor(c["img"][:k], mul, add, reverse_channels=True, layout=orc.NCHW, dtype=orc.FP16)
+    elif cfg == 6:
+        n = n or 256
+        c = wl.config1(n)
+        scale, bias = scale_bias(n)
+        dw = np.full(n, 224, np.uint32)
+        # the same images, one after the other without padding
+        offsets, pos = [], 0
+        for i in range(n):
+            offsets.append(pos)
+            pos += int(c["H"][i]) * int(c["W"][i]) * 3
+        packed = np.concatenate([c["img"][i, :c["H"][i], :c["W"][i]].reshape(-1) for i in range(n)])
+        op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+        op.set_ragged_source(np.array(offsets, np.uint64), c["W"], c["H"], packed.size)
+        op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
+
+        padded, roi6, mirror6 = c["img"], c["roi"], c["mirror"]
+
+        def cpu(k):
+            from oracle import orc
+            return orc.resize(padded[:k], roi6[:k], dw[:k], dw[:k], 224, 224, interp=orc.LINEAR, mirror=mirror6[:k],
+                              scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16, flags=orc.F_QUANTIZE_U8)
+        c = dict(img=packed)
     else:
         raise SystemExit("unknown config %r" % cfg)
     src = torch.from_numpy(c["img"]).cuda()
@@ -218,7 +254,7 @@ def main():
     res["roofline"]["frac_of_copy_ceiling"] = round(res["roofline"]["achieved"] / ceiling, 4)
     if args.all:
         allres = {args.config: res}
-        for cfg in range(5):
+        for cfg in sorted(WORKLOADS):
             if cfg != args.config:
                 allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu)
                 allres[cfg]["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)

@@ -15,7 +15,7 @@ def _bits(a):
     return a.view(np.uint8)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6])
 def test_full_size_configuration_is_bit_identical_to_the_oracle(ctx, cfg):
     op, src, dst, n, cpu = bench.build_case(cfg, ctx)
     dst.zero_()
