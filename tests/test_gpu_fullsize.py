@@ -209,3 +209,48 @@ def test_warp_on_an_exact_size_source_and_tiny_windows(ctx, interp):
     got = out.cpu().numpy()
     for i in range(n):
         assert np.array_equal(got[i, :dh[i], :dw[i]], exp[i, :dh[i], :dw[i]]), "sample %d: %d values differ" % (i, int((got[i, :dh[i], :dw[i]] != exp[i, :dh[i], :dw[i]]).sum()))
+
+
+def test_launches_can_be_captured_in_a_graph_and_replayed(ctx):
+    """update() uploads the parameter table outside the capture; the launches of a resize -> colour twist -> flip
+    chain are recorded in a HIP graph and replayed several times, with eager work and synchronisation between
+    the replays and a new input each time; every replay must equal the eager result."""
+    import torch
+    s = torch.cuda.Stream()
+    c2 = ops.Context(0, stream=s.cuda_stream)
+    rng = np.random.default_rng(3)
+    n, H, W = 4, 90, 120
+    roi = np.array([[0, 0, 120, 90], [5, 5, 100, 80], [0, 0, 64, 64], [10, 0, 96, 90]], np.uint32)
+    dw, dh = np.full(n, 64, np.uint32), np.full(n, 48, np.uint32)
+    mid_roi = np.array([[0, 0, 64, 48]] * n, np.uint32)
+    one = lambda v: np.full(n, v, np.float32)
+    sd, md = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 48, 64, ops.NHWC, ops.UINT8)
+    resize, twist, flip = ops.Resize(c2, sd, md, ops.LINEAR), ops.ColorTwist(c2, md, md), ops.Flip(c2, md, md)
+    resize.update(roi, dw, dh)
+    twist.update(mid_roi, one(1.1), one(4.0), one(25.0), one(1.3))
+    flip.update(mid_roi, np.ones(n, np.uint32), np.zeros(n, np.uint32))
+    with torch.cuda.stream(s):
+        src = torch.zeros((n, H, W, 3), dtype=torch.uint8, device="cuda")
+        a, b, out = resize.alloc_output(), twist.alloc_output(), flip.alloc_output()
+        resize.launch(src, a); twist.launch(a, b); flip.launch(b, out)  # warm-up before the capture
+        s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        resize.launch(src, a)
+        twist.launch(a, b)
+        flip.launch(b, out)
+    for rep in range(4):
+        img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+        with torch.cuda.stream(s):
+            src.copy_(torch.from_numpy(img))
+            out.zero_()
+            g.replay()
+            s.synchronize()
+            got = out.cpu().numpy()
+            # the same chain eagerly, into other buffers
+            a2, b2, o2 = resize.alloc_output(), twist.alloc_output(), flip.alloc_output()
+            resize.launch(src, a2); twist.launch(a2, b2); flip.launch(b2, o2)
+            s.synchronize()
+        exp_mid = orc.color_twist(orc.resize(img, roi, dw, dh, 48, 64, interp=orc.LINEAR), mid_roi, one(1.1), one(4.0), one(25.0), one(1.3))
+        assert np.array_equal(got, o2.cpu().numpy()), "replay %d differs from the eager chain" % rep
+        assert np.array_equal(got, exp_mid[:, :, ::-1]), "replay %d differs from the oracle" % rep
