@@ -145,7 +145,7 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
                         colour(v);
                         PackedGroup<T> packed;
                         pack_group_dir<T, LAYOUT, false>(v, packed);
-                        store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                        store_packed<T, LAYOUT, sizeof(T) == 1>(dimg, a.dst_h, a.dst_w, r, gx, packed);  // u8: streaming stores
                     }
                 }
             }

@@ -239,7 +239,7 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
                 }
                 PackedGroup<T> packed;
                 pack_group<T, LAYOUT>(v, hf, packed);
-                store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, x0, packed);
+                store_packed<T, LAYOUT, sizeof(T) == 2>(dimg, a.dst_h, a.dst_w, r, x0, packed);  // fp16: streaming stores
             }
         }
         if (xt + tile_w < dw) wave_sync();  // the next tile overwrites the LDS slice
