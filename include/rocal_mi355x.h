@@ -156,6 +156,31 @@ RMX_API int rmx_create_saturation(rmx_ctx *ctx, const rmx_tensor_desc *src, cons
                                   int roi_type, rmx_op **out);
 RMX_API int rmx_update_saturation(rmx_op *op, const uint32_t *src_roi, const float *sat);
 
+/* ---- Streaming neighbours of the colour family (u8 NHWC in, one pass). Their arithmetic lives in RPP, which the
+ *      reference tree does not hold; the laws are the ones stated here.
+ *      Gamma: replaces vxExtRppGammaCorrection (rocAL/source/augmentations/color_augmentations/node_gamma.cpp:42):
+ *        out = lut[x], lut[v] = round-to-nearest-even, saturated powf(v/255, gamma)*255, one table per sample.
+ *      Exposure: replaces vxExtRppExposure (node_exposure.cpp:42): out = x * 2^factor.
+ *      ColorTemperature: replaces vxExtRppColorTemperature (node_color_temperature.cpp:42): red + adjustment,
+ *        green unchanged, blue - adjustment, saturating.
+ *      Blend: replaces vxExtRppBlend (node_blend.cpp:45): out = fmaf(a - b, ratio, b) = a*ratio + b*(1-ratio)
+ *        (rocal_api_augmentation.h:371), a and b two source batches of one shape read through the first one's ROI;
+ *        launched with rmx_op_launch2. ---- */
+RMX_API int rmx_create_gamma(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                             int roi_type, rmx_op **out);
+RMX_API int rmx_update_gamma(rmx_op *op, const uint32_t *src_roi, const float *gamma /*[N]*/);
+RMX_API int rmx_create_exposure(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                int roi_type, rmx_op **out);
+RMX_API int rmx_update_exposure(rmx_op *op, const uint32_t *src_roi, const float *factor /*[N]*/);
+RMX_API int rmx_create_color_temperature(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                                         int roi_type, rmx_op **out);
+RMX_API int rmx_update_color_temperature(rmx_op *op, const uint32_t *src_roi, const int32_t *adjustment /*[N]*/);
+RMX_API int rmx_create_blend(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst,
+                             int roi_type, rmx_op **out);
+RMX_API int rmx_update_blend(rmx_op *op, const uint32_t *src_roi, const float *ratio /*[N]*/);
+/* process step of a two-input node (Blend): as rmx_op_launch, with the second source batch. */
+RMX_API int rmx_op_launch2(rmx_op *op, const void *src1, const void *src2, void *dst);
+
 /* ---- WarpAffine: replaces vxExtRppWarpAffine (node_warp_affine.cpp:61-62). affine is [N][6] in
  *      rocAL's fill order x0,y0,x1,y1,o0,o1 (:43-48), read as M=[[x0,x1,o0],[y0,y1,o1]] mapping
  *      destination to source about the ROI / output centres. Out-of-ROI samples give 0. ---- */

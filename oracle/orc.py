@@ -67,6 +67,7 @@ def lib():
         _lib.orc_fixed_crop.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_int, C.c_float,
                                         C.c_float, C.c_uint32, C.c_uint32, C.c_void_p]
         _lib.orc_rotate_matrix.argtypes = [C.c_float, C.c_void_p]
+        _lib.orc_gamma_lut.argtypes = [C.c_float, C.c_void_p, C.c_uint]
     return _lib
 
 
@@ -131,11 +132,11 @@ def resize(img, roi_xywh, dst_w, dst_h, out_hmax, out_wmax, interp=LINEAR, mirro
     return out
 
 
-def _color_common(fn, img, roi_xywh, params, flags):
+def _color_common(fn, img, roi_xywh, params, flags, layout=NHWC, dtype=UINT8):
     roi_xywh = _u32(roi_xywh)
     params = [_f32(p) for p in params]
     n, h, w, c = img.shape
-    out, d = _alloc_dst(n, c, h, w, NHWC, UINT8)
+    out, d = _alloc_dst(n, c, h, w, layout, dtype)
     s = _src(img)
     fn(C.byref(s), _p(roi_xywh), *[_p(p) for p in params], C.byref(d), C.c_uint(flags))
     return out
@@ -147,6 +148,40 @@ def brightness(img, roi_xywh, alpha, beta, flags=0):
 
 def contrast(img, roi_xywh, factor, center, flags=0):
     return _color_common(lib().orc_contrast, img, roi_xywh, [factor, center], flags)
+
+
+def gamma_lut(gamma, flags=0):
+    lut = np.empty(256, np.uint8)
+    lib().orc_gamma_lut(C.c_float(gamma), _p(lut), C.c_uint(flags))
+    return lut
+
+
+def gamma(img, roi_xywh, gamma, flags=0, layout=NHWC, dtype=UINT8):
+    return _color_common(lib().orc_gamma, img, roi_xywh, [gamma], flags, layout, dtype)
+
+
+def exposure(img, roi_xywh, factor, flags=0, layout=NHWC, dtype=UINT8):
+    return _color_common(lib().orc_exposure, img, roi_xywh, [factor], flags, layout, dtype)
+
+
+def color_temperature(img, roi_xywh, adjustment, flags=0, layout=NHWC, dtype=UINT8):
+    roi_xywh = _u32(roi_xywh)
+    adj = np.ascontiguousarray(adjustment, np.int32)
+    n, h, w, c = img.shape
+    out, d = _alloc_dst(n, c, h, w, layout, dtype)
+    s = _src(img)
+    lib().orc_color_temperature(C.byref(s), _p(roi_xywh), _p(adj), C.byref(d), C.c_uint(flags))
+    return out
+
+
+def blend(img1, img2, roi_xywh, ratio, flags=0, layout=NHWC, dtype=UINT8):
+    assert img1.shape == img2.shape
+    roi_xywh, ratio = _u32(roi_xywh), _f32(ratio)
+    n, h, w, c = img1.shape
+    out, d = _alloc_dst(n, c, h, w, layout, dtype)
+    s1, s2 = _src(img1), _src(img2)
+    lib().orc_blend(C.byref(s1), C.byref(s2), _p(roi_xywh), _p(ratio), C.byref(d), C.c_uint(flags))
+    return out
 
 
 def color_twist(img, roi_xywh, alpha, beta, hue, sat, flags=0):

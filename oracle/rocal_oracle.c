@@ -414,6 +414,80 @@ void orc_contrast(const orc_src *src, const uint32_t *roi, const float *factor, 
     }
 }
 
+/* ---- streaming neighbours of the colour family. Their arithmetic lives only in RPP, which is absent from the
+ * reference tree: each law below is DEFINED here from the parameter meanings the tree gives (PARITY UNPINNED). */
+
+/* Gamma (vxExtRppGammaCorrection, node_gamma.cpp:42; gamma range 0.3..7, node_gamma.h:41): a 256-entry table per
+ * sample, lut[i] = u8 store of powf(i/255, gamma)*255; every channel of every pixel goes through it. A float
+ * destination receives the table value converted. */
+void orc_gamma_lut(float gamma, uint8_t *lut, unsigned flags) {
+    for (int i = 0; i < 256; i++) lut[i] = (uint8_t)round_u8(powf((float)i / 255.0f, gamma) * 255.0f, flags);
+}
+
+void orc_gamma(const orc_src *src, const uint32_t *roi, const float *gamma, const orc_dst *dst, unsigned flags) {
+    const int C = src->c;
+#pragma omp parallel for schedule(dynamic)
+    for (int n = 0; n < src->n; n++) {
+        int x0 = (int)roi[n * 4], y0 = (int)roi[n * 4 + 1], w = (int)roi[n * 4 + 2], h = (int)roi[n * 4 + 3];
+        uint8_t lut[256];
+        orc_gamma_lut(gamma[n], lut, flags);
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const uint8_t *p = src_px(src, n, y0 + y, x0 + x);
+                for (int c = 0; c < C; c++) store(dst, dst_index(dst, n, c, y, x), (float)lut[p[c]], flags);
+            }
+    }
+}
+
+/* Exposure (vxExtRppExposure, node_exposure.cpp:42; factor range 0.15..0.95, node_exposure.h:42):
+ * out = x * 2^factor, one fp32 product, u8 store. */
+void orc_exposure(const orc_src *src, const uint32_t *roi, const float *factor, const orc_dst *dst, unsigned flags) {
+    const int C = src->c;
+#pragma omp parallel for schedule(dynamic)
+    for (int n = 0; n < src->n; n++) {
+        int x0 = (int)roi[n * 4], y0 = (int)roi[n * 4 + 1], w = (int)roi[n * 4 + 2], h = (int)roi[n * 4 + 3];
+        const float m = exp2f(factor[n]);
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const uint8_t *p = src_px(src, n, y0 + y, x0 + x);
+                for (int c = 0; c < C; c++) store(dst, dst_index(dst, n, c, y, x), (float)p[c] * m, flags);
+            }
+    }
+}
+
+/* ColorTemperature (vxExtRppColorTemperature, node_color_temperature.cpp:42; integer adjustment -99..99,
+ * node_color_temperature.h:42-43): red + adj, green unchanged, blue - adj, saturating. */
+void orc_color_temperature(const orc_src *src, const uint32_t *roi, const int32_t *adj, const orc_dst *dst, unsigned flags) {
+#pragma omp parallel for schedule(dynamic)
+    for (int n = 0; n < src->n; n++) {
+        int x0 = (int)roi[n * 4], y0 = (int)roi[n * 4 + 1], w = (int)roi[n * 4 + 2], h = (int)roi[n * 4 + 3];
+        const float d[3] = {(float)adj[n], 0.0f, -(float)adj[n]};
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const uint8_t *p = src_px(src, n, y0 + y, x0 + x);
+                for (int c = 0; c < 3; c++) store(dst, dst_index(dst, n, c, y, x), (float)p[c] + d[c], flags);
+            }
+    }
+}
+
+/* Blend (vxExtRppBlend, node_blend.cpp:45; "output = input1*ratio + input2*(1-ratio)",
+ * rocal_api_augmentation.h:371): evaluated as fmaf(a - b, ratio, b); a - b is exact for bytes, so the documented
+ * value is rounded once. Both inputs share the first input's ROI (node_blend.cpp:45 passes only inputs[0]'s). */
+void orc_blend(const orc_src *src1, const orc_src *src2, const uint32_t *roi, const float *ratio, const orc_dst *dst, unsigned flags) {
+    const int C = src1->c;
+#pragma omp parallel for schedule(dynamic)
+    for (int n = 0; n < src1->n; n++) {
+        int x0 = (int)roi[n * 4], y0 = (int)roi[n * 4 + 1], w = (int)roi[n * 4 + 2], h = (int)roi[n * 4 + 3];
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const uint8_t *p = src_px(src1, n, y0 + y, x0 + x);
+                const uint8_t *q = src_px(src2, n, y0 + y, x0 + x);
+                for (int c = 0; c < C; c++)
+                    store(dst, dst_index(dst, n, c, y, x), fmaf((float)p[c] - (float)q[c], ratio[n], (float)q[c]), flags);
+            }
+    }
+}
+
 /* hue in degrees -> shift in sextants, reduced to [0,6] */
 static float hue_shift_sextants(float hue_deg, unsigned flags) {
     if (flags & ORC_F_HUE_INT_TRUNC) hue_deg = (float)((int)hue_deg % 360);

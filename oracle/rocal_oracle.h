@@ -30,6 +30,9 @@
  *   orc_to_tensor              pinned: rocal_hip_kernels.cpp:131-217 (oracle/_ref), closed form.
  *   orc_brightness/contrast    parity unpinned beyond the closed form alpha*x+beta (API doc
  *                              rocAL/include/api/rocal_api_augmentation.h:231-232).
+ *   orc_gamma/exposure/color_temperature/blend
+ *                              PARITY UNPINNED against RPP; closed forms tested (gamma 1 and 2, 2^k
+ *                              exposure, saturating +-adj, ratio 0 / 1 / 0.5).
  *   orc_color_twist/hue/sat    PARITY UNPINNED: HSV details live only in RPP. Invariants tested
  *                              (identity, grey fixed points, 360-periodicity, colorsys cross-check).
  *   orc_warp_affine            PARITY UNPINNED for matrix element order / centre convention;
@@ -109,6 +112,14 @@ void orc_brightness(const orc_src *src, const uint32_t *roi_xywh, const float *a
 /* out = fmaf(x - center, factor, center) -> u8 */
 void orc_contrast(const orc_src *src, const uint32_t *roi_xywh, const float *factor, const float *center,
                   const orc_dst *dst, unsigned flags);
+/* Gamma / Exposure / ColorTemperature / Blend: laws DEFINED in rocal_oracle.c (parity unpinned against RPP). */
+void orc_gamma_lut(float gamma, uint8_t *lut /*[256]*/, unsigned flags);
+void orc_gamma(const orc_src *src, const uint32_t *roi_xywh, const float *gamma, const orc_dst *dst, unsigned flags);
+void orc_exposure(const orc_src *src, const uint32_t *roi_xywh, const float *factor, const orc_dst *dst, unsigned flags);
+void orc_color_temperature(const orc_src *src, const uint32_t *roi_xywh, const int32_t *adjustment, const orc_dst *dst,
+                           unsigned flags);
+void orc_blend(const orc_src *src1, const orc_src *src2, const uint32_t *roi_xywh, const float *ratio, const orc_dst *dst,
+               unsigned flags);
 /* HSV colour twist; hue in degrees. */
 void orc_color_twist(const orc_src *src, const uint32_t *roi_xywh, const float *alpha, const float *beta,
                      const float *hue, const float *sat, const orc_dst *dst, unsigned flags);

@@ -57,6 +57,15 @@ _SIGS = {
     "rmx_update_hue": [_vp, _vp, _vp],
     "rmx_create_saturation": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
     "rmx_update_saturation": [_vp, _vp, _vp],
+    "rmx_create_gamma": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
+    "rmx_update_gamma": [_vp, _vp, _vp],
+    "rmx_create_exposure": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
+    "rmx_update_exposure": [_vp, _vp, _vp],
+    "rmx_create_color_temperature": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
+    "rmx_update_color_temperature": [_vp, _vp, _vp],
+    "rmx_create_blend": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
+    "rmx_update_blend": [_vp, _vp, _vp],
+    "rmx_op_launch2": [_vp, _vp, _vp, _vp],
     "rmx_create_warp_affine": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.POINTER(_vp)],
     "rmx_update_warp_affine": [_vp, _vp, _vp, _vp, _vp],
     "rmx_create_rotate": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.POINTER(_vp)],

@@ -37,7 +37,7 @@ int fail(int code, const char *fmt, ...) {
 
 enum OpKind {
     OP_CMN = 1, OP_CROP, OP_FLIP, OP_RESIZE, OP_COLOR_TWIST, OP_BRIGHTNESS, OP_CONTRAST, OP_HUE,
-    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE, OP_TO_TENSOR
+    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE, OP_TO_TENSOR, OP_GAMMA, OP_EXPOSURE, OP_COLOR_TEMPERATURE, OP_BLEND
 };
 
 constexpr int TABLE_RING = 4;  // updates in flight before the host has to wait on an old upload
@@ -72,7 +72,8 @@ struct rmx_op {
     bool norm = false, quant = false;
     int n = 0;
 
-    RmxSample *h_table[TABLE_RING] = {};  // pinned; n rows, then n source layout entries
+    RmxSample *h_table[TABLE_RING] = {};  // pinned; n rows, then n source layout entries, then n side-table entries
+    size_t extra_per_sample = 0;          // bytes of side table per sample (Gamma: its 256-entry table)
     std::vector<RmxSrcLayout> layout;     // ragged source (empty: one padded tensor); copied behind the rows on every update
     uint64_t ragged_bytes = 0;            // extent of the ragged source buffer
     bool slot_ragged[TABLE_RING] = {};    // what the table slot was committed with
@@ -104,7 +105,7 @@ int check_desc(const rmx_tensor_desc *d, const char *what) {
     return RMX_OK;
 }
 
-int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out, size_t extra_per_sample = 0) {
     if (!ctx) return fail(RMX_ERR_INVALID, "context is NULL");
     if (!out) return fail(RMX_ERR_INVALID, "output handle pointer is NULL");
     *out = nullptr;
@@ -124,7 +125,8 @@ int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor
     op->dst = *dst;
     op->roi_type = roi_type;
     op->n = (int)src->n;
-    size_t bytes = (sizeof(RmxSample) + sizeof(RmxSrcLayout)) * (size_t)op->n;
+    op->extra_per_sample = extra_per_sample;
+    size_t bytes = (sizeof(RmxSample) + sizeof(RmxSrcLayout) + extra_per_sample) * (size_t)op->n;
     for (int i = 0; i < TABLE_RING; i++) {
         hipError_t e = hipHostMalloc((void **)&op->h_table[i], bytes, hipHostMallocDefault);
         if (e == hipSuccess) e = hipMalloc((void **)&op->d_table[i], bytes);
@@ -154,6 +156,8 @@ int commit_slot(rmx_op *op, int slot) {
         memcpy(reinterpret_cast<char *>(op->h_table[slot]) + bytes, op->layout.data(), sizeof(RmxSrcLayout) * (size_t)op->n);
         bytes += sizeof(RmxSrcLayout) * (size_t)op->n;
     }
+    if (op->extra_per_sample)  // the side table lies behind the layout entries whether or not those are in use
+        bytes = (sizeof(RmxSample) + sizeof(RmxSrcLayout) + op->extra_per_sample) * (size_t)op->n;
     op->slot_ragged[slot] = !op->layout.empty();
     op->slot_src_bytes[slot] = op->ragged_bytes;
     HIP_TRY(hipMemcpyAsync(op->d_table[slot], op->h_table[slot], bytes, hipMemcpyHostToDevice, op->ctx->stream));
@@ -184,6 +188,11 @@ int read_roi(const rmx_op *op, const uint32_t *roi, int i, int32_t *x, int32_t *
     if (d > sh - b) d = sh - b;
     *x = (int32_t)a; *y = (int32_t)b; *w = (int32_t)c; *h = (int32_t)d;
     return RMX_OK;
+}
+
+// side table of a slot: behind the n rows and the n layout entries
+inline uint8_t *slot_extra(rmx_op *op, RmxSample *rows) {
+    return reinterpret_cast<uint8_t *>(rows) + (sizeof(RmxSample) + sizeof(RmxSrcLayout)) * (size_t)op->n;
 }
 
 size_t dtype_size(int dtype) { return dtype == RMX_FP32 ? 4 : dtype == RMX_FP16 ? 2 : 1; }
@@ -289,12 +298,13 @@ const char *rmx_op_plan(const rmx_op *op) {
 }
 const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : op->kernel_name) : ""; }
 
-int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
-    if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
+static int launch_impl(rmx_op *op, const void *src, const void *src2, void *dst) {
     if (!src || !dst) return fail(RMX_ERR_INVALID, "source/destination buffer is NULL");
     if (op->cur < 0 || !op->fn) return fail(RMX_ERR_INVALID, "op launched before its first update");
     RmxKArgs a{};
     a.src = (const uint8_t *)src;
+    a.src2 = (const uint8_t *)src2;
+    a.extra = op->extra_per_sample ? slot_extra(op, op->d_table[op->cur]) : nullptr;
     a.dst = dst;
     a.table = op->d_table[op->cur];
     a.src_bytes = op->slot_ragged[op->cur] ? op->slot_src_bytes[op->cur] : (uint64_t)op->src.n * op->src.h * op->src.w * op->src.c;
@@ -308,7 +318,7 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     a.lds_bytes = op->lds_per_wave;
     a.aux0 = op->aux0;
     a.aux1 = op->aux1;
-    if (((uintptr_t)src) & 3u) return fail(RMX_ERR_INVALID, "the source batch must start at a 4-byte aligned address");
+    if ((((uintptr_t)src) | ((uintptr_t)src2)) & 3u) return fail(RMX_ERR_INVALID, "the source batch must start at a 4-byte aligned address");
     if ((op->kind == OP_WARP_AFFINE || op->kind == OP_ROTATE) && (((uintptr_t)dst) & 15u)) a.aux1 &= ~1;  // packed stores need an aligned base
     // the fast specialisation wants 16-byte aligned batch bases (rows of both sides are then aligned too)
     const bool fast = op->fn_fast && (((uintptr_t)dst) & 15u) == 0 && (!op->fast_needs_src16 || (((uintptr_t)src) & 15u) == 0);
@@ -333,10 +343,24 @@ int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
     return RMX_OK;
 }
 
+int rmx_op_launch(rmx_op *op, const void *src, void *dst) {
+    if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
+    if (op->kind == OP_BLEND) return fail(RMX_ERR_INVALID, "a Blend node takes two sources: use rmx_op_launch2");
+    return launch_impl(op, src, nullptr, dst);
+}
+
+int rmx_op_launch2(rmx_op *op, const void *src1, const void *src2, void *dst) {
+    if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
+    if (op->kind != OP_BLEND) return fail(RMX_ERR_INVALID, "only a Blend node takes two sources");
+    if (!src2) return fail(RMX_ERR_INVALID, "second source buffer is NULL");
+    return launch_impl(op, src1, src2, dst);
+}
+
 /* ------------------------------------------------------------------ ragged sources */
 
 int rmx_op_set_ragged_source(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights, uint64_t buffer_bytes) {
     if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
+    if (op->kind == OP_BLEND) return fail(RMX_ERR_UNSUPPORTED, "a Blend node reads two padded tensors of one shape; ragged sources are not supported");
     if (!offsets && !widths && !heights) {  // back to one padded tensor
         op->layout.clear();
         op->ragged_bytes = 0;
@@ -896,6 +920,106 @@ int rmx_update_saturation(rmx_op *op, const uint32_t *src_roi, const float *sat)
     if (!op || op->kind != OP_SATURATION) return fail(RMX_ERR_INVALID, "op is not a Saturation node");
     if (!sat) return fail(RMX_ERR_INVALID, "sat array is required");
     return update_color(op, src_roi, nullptr, nullptr, nullptr, sat, 1, 0, 0, 1, true);
+}
+
+/* ------------------------------------------------------------------ streaming neighbours of K3 / K1 */
+
+int rmx_create_exposure(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_color(ctx, OP_EXPOSURE, src, dst, roi_type, out);
+}
+int rmx_update_exposure(rmx_op *op, const uint32_t *src_roi, const float *factor) {
+    if (!op || op->kind != OP_EXPOSURE) return fail(RMX_ERR_INVALID, "op is not an Exposure node");
+    if (!factor) return fail(RMX_ERR_INVALID, "exposure factor array is required");
+    // out = x * 2^factor: the multiplier is made once per sample on the host, the kernel multiplies
+    std::vector<float> m((size_t)op->n);
+    for (int i = 0; i < op->n; i++) m[i] = exp2f(factor[i]);
+    return update_color(op, src_roi, m.data(), nullptr, nullptr, nullptr, 1, 0, 0, 0, false);
+}
+
+int rmx_create_color_temperature(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_k1(ctx, OP_COLOR_TEMPERATURE, src, dst, roi_type, true, out);
+}
+int rmx_update_color_temperature(rmx_op *op, const uint32_t *src_roi, const int32_t *adjustment) {
+    if (!op || op->kind != OP_COLOR_TEMPERATURE) return fail(RMX_ERR_INVALID, "op is not a ColorTemperature node");
+    if (!adjustment) return fail(RMX_ERR_INVALID, "adjustment array is required");
+    // red + adj, green, blue - adj: a per-channel offset with unit scale, which is what the K1 kernel computes
+    std::vector<float> bias((size_t)op->n * 3);
+    for (int i = 0; i < op->n; i++) {
+        bias[(size_t)i * 3 + 0] = (float)adjustment[i];
+        bias[(size_t)i * 3 + 1] = 0.0f;
+        bias[(size_t)i * 3 + 2] = -(float)adjustment[i];
+    }
+    return update_k1(op, src_roi, nullptr, bias.data(), nullptr, nullptr);
+}
+
+static int create_point(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    int rc = make_op(ctx, kind, src, dst, roi_type, out, kind == OP_GAMMA ? 256 : 0);
+    if (rc) return rc;
+    (*out)->fn = rmx::select_point_kernel(kind == OP_BLEND ? 1 : 0, dst->dtype, dst->layout, false, &(*out)->kernel_name);
+    return RMX_OK;
+}
+
+// rows and launch plan of a one-pass op that writes the source window to the destination's origin
+static int update_point(rmx_op *op, const uint32_t *roi, const float *p0, const float *gamma) {
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    uint64_t bytes = 0;
+    int max_rows = 1;
+    const int sources = op->kind == OP_BLEND ? 2 : 1;
+    uint8_t *lut = slot_extra(op, t);
+    for (int i = 0; i < op->n; i++) {
+        RmxSample &s = t[i];
+        int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+        if (rc) return rc;
+        s.dst_w = std::min<int32_t>(s.src_w, (int32_t)op->dst.w);
+        s.dst_h = std::min<int32_t>(s.src_h, (int32_t)op->dst.h);
+        s.flags = 0;
+        s.color[0] = p0 ? p0[i] : 0.0f;
+        s.color[1] = s.color[2] = s.color[3] = 0.0f;
+        if (gamma) {
+            // lut[v] = u8 store (round to nearest even, saturate) of powf(v/255, gamma)*255
+            for (int v = 0; v < 256; v++) {
+                float r = rintf(powf((float)v / 255.0f, gamma[i]) * 255.0f);
+                r = !(r > 0.0f) ? 0.0f : (r > 255.0f ? 255.0f : r);  // a NaN becomes 0
+                lut[(size_t)i * 256 + v] = (uint8_t)r;
+            }
+        }
+        bytes += (uint64_t)s.dst_w * s.dst_h * 3 * (sources + dtype_size(op->dst.dtype));
+        max_rows = std::max(max_rows, (int)s.dst_h);
+    }
+    op->algo_bytes = bytes;
+    plan_streaming(op, max_rows, op->ctx->k3_rows);
+    bool aligned = op->dst.w % 8 == 0;
+    for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
+    op->fn_fast = nullptr;
+    if (aligned) {
+        op->fn_fast = rmx::select_point_kernel(op->kind == OP_BLEND ? 1 : 0, op->dst.dtype, op->dst.layout, true, &op->fast_name);
+        op->fast_strips = op->strips;
+        op->fast_lds = 0;
+        op->fast_rows = op->aux0;
+        op->fast_wpb = op->waves_per_block;
+        op->fast_needs_src16 = false;
+    }
+    return commit_slot(op, slot);
+}
+
+int rmx_create_gamma(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_point(ctx, OP_GAMMA, src, dst, roi_type, out);
+}
+int rmx_update_gamma(rmx_op *op, const uint32_t *src_roi, const float *gamma) {
+    if (!op || op->kind != OP_GAMMA) return fail(RMX_ERR_INVALID, "op is not a Gamma node");
+    if (!gamma) return fail(RMX_ERR_INVALID, "gamma array is required");
+    return update_point(op, src_roi, nullptr, gamma);
+}
+
+int rmx_create_blend(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    return create_point(ctx, OP_BLEND, src, dst, roi_type, out);
+}
+int rmx_update_blend(rmx_op *op, const uint32_t *src_roi, const float *ratio) {
+    if (!op || op->kind != OP_BLEND) return fail(RMX_ERR_INVALID, "op is not a Blend node");
+    if (!ratio) return fail(RMX_ERR_INVALID, "ratio array is required");
+    return update_point(op, src_roi, ratio, nullptr);
 }
 
 /* ------------------------------------------------------------------ K4 family */

@@ -52,6 +52,8 @@ struct RmxKArgs {
     int32_t wpb;             // wavefronts per workgroup of this launch
     uint32_t nblocks;        // workgroups of this launch
     const RmxSrcLayout *layout;  // per-sample source placement, or null: sample s starts at s*src_h*src_w*3
+    const uint8_t *src2;         // second source batch of the same shape (Blend), else null
+    const uint8_t *extra;        // per-sample side table behind the layout entries (Gamma: 256 bytes per sample), else null
 };
 
 #define RMX_WAVE 64

@@ -13,6 +13,7 @@ KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool qua
 KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name);
+KernelFn select_point_kernel(int kind, int dtype, int layout, bool fast, const char **name);
 KernelFn select_warp_kernel(int interp, int dtype, int layout, const char **name);
 void launch_copy(hipStream_t stream, const void *src, void *dst, size_t nbytes, int num_cus);
 }  // namespace rmx

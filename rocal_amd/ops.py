@@ -243,6 +243,44 @@ class Saturation(Op):
         self._update("rmx_update_saturation", (src_roi, _U), (sat, _F))
 
 
+class Gamma(Op):
+    _create = "rmx_create_gamma"
+
+    def update(self, src_roi, gamma):
+        self._update("rmx_update_gamma", (src_roi, _U), (gamma, _F))
+
+
+class Exposure(Op):
+    _create = "rmx_create_exposure"
+
+    def update(self, src_roi, factor):
+        self._update("rmx_update_exposure", (src_roi, _U), (factor, _F))
+
+
+class ColorTemperature(Op):
+    _create = "rmx_create_color_temperature"
+
+    def update(self, src_roi, adjustment):
+        self._update("rmx_update_color_temperature", (src_roi, _U), (adjustment, np.int32))
+
+
+class Blend(Op):
+    """Two source batches of one shape; launch(src1, src2, dst)."""
+    _create = "rmx_create_blend"
+
+    def update(self, src_roi, ratio):
+        self._update("rmx_update_blend", (src_roi, _U), (ratio, _F))
+
+    def launch(self, src1, src2, dst):
+        assert src1.is_cuda and src2.is_cuda and dst.is_cuda and src1.is_contiguous() and src2.is_contiguous() and dst.is_contiguous()
+        sd, dd = self.src_desc, self.dst_desc
+        need = sd.n * sd.h * sd.w * sd.c
+        assert src1.numel() * src1.element_size() >= need and src2.numel() * src2.element_size() >= need, "source buffer smaller than its descriptor"
+        esz = {FP32: 4, FP16: 2, UINT8: 1}[dd.dtype]
+        assert dst.numel() * dst.element_size() >= dd.n * dd.h * dd.w * dd.c * esz, "destination buffer smaller than its descriptor"
+        check(_lib.lib().rmx_op_launch2(self._h, C.c_void_p(src1.data_ptr()), C.c_void_p(src2.data_ptr()), C.c_void_p(dst.data_ptr())))
+
+
 class WarpAffine(Op):
     _create = "rmx_create_warp_affine"
     _n_pre = 1

@@ -239,6 +239,49 @@ def test_brightness_contrast_closed_forms():
     assert np.abs(out.astype(np.int32) - exp.astype(np.int32)).max() == 0
 
 
+def test_gamma_table_closed_forms():
+    # gamma 1 is the identity; gamma 2 is v*v/255 and gamma 0.5 is sqrt(255*v), each rounded once; the table is
+    # monotone and fixes both ends for every gamma of the node's range (node_gamma.h:41)
+    v = np.arange(256, dtype=np.float64)
+    assert (orc.gamma_lut(1.0) == np.arange(256)).all()
+    # v*v/255 and sqrt(255*v) are never within 1e-3 of a rounding boundary for integer v, so fp32 powf cannot flip them
+    assert (orc.gamma_lut(2.0).astype(int) == np.rint(v * v / 255.0)).all()
+    assert (orc.gamma_lut(0.5).astype(int) == np.rint(np.sqrt(255.0 * v))).all()
+    for g in (0.3, 0.8, 2.2, 7.0):
+        lut = orc.gamma_lut(g).astype(int)
+        assert lut[0] == 0 and lut[255] == 255 and (np.diff(lut) >= 0).all()
+        exact = 255.0 * (v / 255.0) ** g
+        assert np.abs(lut - exact).max() <= 0.5 + 1e-3
+    img = _img(2, 7, 13)
+    out = orc.gamma(img, _full(2, 7, 13), np.array([2.0, 0.5], np.float32))
+    assert (out[0] == orc.gamma_lut(2.0)[img[0]]).all() and (out[1] == orc.gamma_lut(0.5)[img[1]]).all()
+
+
+def test_exposure_color_temperature_blend_closed_forms():
+    img, img2 = _img(3, 9, 11), _img(3, 9, 11)
+    roi = _full(3, 9, 11)
+    # exposure: powers of two are exact, a fractional factor is one rounded product
+    out = orc.exposure(img, roi, np.array([1.0, 0.0, 0.5], np.float32))
+    assert (out[0] == np.minimum(img[0].astype(int) * 2, 255)).all() and (out[1] == img[1]).all()
+    m = np.float32(2.0) ** np.float32(0.5)
+    assert np.abs(out[2].astype(int) - np.clip(np.rint(img[2].astype(np.float32) * m), 0, 255).astype(int)).max() == 0
+    # colour temperature: integer shifts of red and blue in opposite directions, saturating; green untouched
+    out = orc.color_temperature(img, roi, np.array([40, -99, 0], np.int32))
+    i = img.astype(int)
+    assert (out[0, ..., 0] == np.minimum(i[0, ..., 0] + 40, 255)).all() and (out[0, ..., 2] == np.maximum(i[0, ..., 2] - 40, 0)).all()
+    assert (out[1, ..., 0] == np.maximum(i[1, ..., 0] - 99, 0)).all() and (out[1, ..., 2] == np.minimum(i[1, ..., 2] + 99, 255)).all()
+    assert (out[..., 1] == img[..., 1]).all() and (out[2] == img[2]).all()
+    # blend: ratio 1 and 0 return the inputs, 0.5 is the mean with ties to even, 0.25 is exact in fp32
+    out = orc.blend(img, img2, roi, np.array([1.0, 0.0, 0.5], np.float32))
+    assert (out[0] == img[0]).all() and (out[1] == img2[1]).all()
+    assert (out[2] == np.rint((i[2] + img2[2].astype(int)) / 2.0)).all()
+    out = orc.blend(img, img2, roi, np.array([0.25, 0.25, 0.25], np.float32))
+    assert (out == np.rint((i + 3 * img2.astype(int)) / 4.0)).all()
+    # a float destination keeps the unrounded value
+    outf = orc.blend(img, img2, roi, np.array([0.25, 0.25, 0.25], np.float32), layout=orc.NCHW, dtype=orc.FP32)
+    assert (outf == ((i + 3 * img2.astype(int)) / 4.0).transpose(0, 3, 1, 2)).all()
+
+
 def test_color_twist_invariants():
     img = _img(1, 32, 32)
     roi = _full(1, 32, 32)
