@@ -42,14 +42,15 @@ enum class Dims { KEEP, SET };
 // Common frame of every augmentation entry point.
 template <typename NodeT, typename InitFn>
 Tensor *add_op(RocalContext p_context, RocalTensor p_input, bool is_output, RocalTensorLayout output_layout, RocalTensorOutputType output_datatype,
-               Dims dims, unsigned width, unsigned height, const char *precondition_error, InitFn init) {
+               Dims dims, unsigned width, unsigned height, const char *precondition_error, InitFn init, RocalTensor p_input2 = nullptr,
+               bool two_inputs = false) {
     Tensor *output = nullptr;
     if (!p_context) {
         std::cerr << "Invalid rocal context passed" << std::endl;
         return output;
     }
     auto *context = static_cast<Context *>(p_context);
-    if (!p_input) {
+    if (!p_input || (two_inputs && !p_input2)) {
         context->capture_error("Invalid rocal tensor passed");
         std::cerr << "Invalid rocal tensor passed" << std::endl;
         return output;
@@ -66,7 +67,9 @@ Tensor *add_op(RocalContext p_context, RocalTensor p_input, bool is_output, Roca
         else
             output_info.set_tensor_layout(layout);
         output = context->master_graph->create_tensor(output_info, is_output);
-        auto node = context->master_graph->add_node<NodeT>({input}, {output});
+        std::vector<Tensor *> inputs{input};
+        if (two_inputs) inputs.push_back(static_cast<Tensor *>(p_input2));
+        auto node = context->master_graph->add_node<NodeT>(inputs, {output});
         init(*node);
         if constexpr (!std::is_void<typename MetaOf<NodeT>::type>::value) meta_add_node<typename MetaOf<NodeT>::type, NodeT>(context, node);
     } catch (const std::exception &e) {
@@ -512,6 +515,37 @@ RocalTensor rocalSaturation(RocalContext c, RocalTensor in, bool is_output, Roca
 }
 RocalTensor rocalSaturationFixed(RocalContext c, RocalTensor in, float sat, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
     return add_op<SaturationNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](SaturationNode &n) { n.init(sat); });
+}
+RocalTensor rocalGamma(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam gamma, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<GammaNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](GammaNode &n) { n.init(F(gamma)); });
+}
+RocalTensor rocalGammaFixed(RocalContext c, RocalTensor in, float gamma, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<GammaNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](GammaNode &n) { n.init(gamma); });
+}
+RocalTensor rocalExposure(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam exposure_factor, RocalTensorLayout layout,
+                          RocalTensorOutputType dtype) {
+    return add_op<ExposureNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](ExposureNode &n) { n.init(F(exposure_factor)); });
+}
+RocalTensor rocalExposureFixed(RocalContext c, RocalTensor in, float exposure_factor, bool is_output, RocalTensorLayout layout,
+                               RocalTensorOutputType dtype) {
+    return add_op<ExposureNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](ExposureNode &n) { n.init(exposure_factor); });
+}
+RocalTensor rocalColorTemp(RocalContext c, RocalTensor in, bool is_output, RocalIntParam adjustment, RocalTensorLayout layout,
+                           RocalTensorOutputType dtype) {
+    return add_op<ColorTemperatureNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr,
+                                        [&](ColorTemperatureNode &n) { n.init(I(adjustment)); });
+}
+RocalTensor rocalColorTempFixed(RocalContext c, RocalTensor in, int adjustment, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
+    return add_op<ColorTemperatureNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr,
+                                        [&](ColorTemperatureNode &n) { n.init(adjustment); });
+}
+RocalTensor rocalBlend(RocalContext c, RocalTensor in1, RocalTensor in2, bool is_output, RocalFloatParam ratio, RocalTensorLayout layout,
+                       RocalTensorOutputType dtype) {
+    return add_op<BlendNode>(c, in1, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](BlendNode &n) { n.init(F(ratio)); }, in2, true);
+}
+RocalTensor rocalBlendFixed(RocalContext c, RocalTensor in1, RocalTensor in2, float ratio, bool is_output, RocalTensorLayout layout,
+                            RocalTensorOutputType dtype) {
+    return add_op<BlendNode>(c, in1, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](BlendNode &n) { n.init(ratio); }, in2, true);
 }
 RocalTensor rocalColorTwist(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam alpha, RocalFloatParam beta, RocalFloatParam hue,
                             RocalFloatParam sat, RocalTensorLayout layout, RocalTensorOutputType dtype) {

@@ -230,6 +230,15 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         outs.push_back(rocalResizeCropMirrorFixed(ctx, src, 36, 28, true, 40, 50, rocalCreateIntParameter(1)));
         outs.push_back(rocalBrightnessFixed(ctx, src, 1.2f, 10.0f, true));
         outs.push_back(rocalContrastFixed(ctx, src, 1.3f, 70.0f, true));
+    } else if (scenario == "points") {
+        outs.push_back(rocalGammaFixed(ctx, src, 2.2f, true));
+        outs.push_back(rocalExposureFixed(ctx, src, 0.6f, true));
+        outs.push_back(rocalColorTempFixed(ctx, src, 40, true));
+        RocalTensor bright = rocalBrightnessFixed(ctx, src, 0.5f, 100.0f, true);
+        outs.push_back(bright);
+        outs.push_back(rocalBlendFixed(ctx, src, bright, 0.3f, true));
+        // a second input of another shape is refused when the graph is built, a missing one at once
+        if (rocalBlendFixed(ctx, src, nullptr, 0.3f, true) != nullptr) return 14;
     } else if (scenario == "to_tensor") {
         outs.push_back(rocalResize(ctx, src, 40, 32, true));
     } else if (scenario == "errors") {

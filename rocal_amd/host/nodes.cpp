@@ -561,6 +561,86 @@ void SaturationNode::update_node() {
     check(rmx_update_saturation(_node, roi.data(), _sat.values().data()), "rmx_update_saturation");
 }
 
+/* ======================================================================= gamma / exposure / colour temperature / blend */
+
+GammaNode::GammaNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)
+    : Node(inputs, outputs), _gamma(GAMMA_RANGE[0], GAMMA_RANGE[1]) {}
+void GammaNode::init(float gamma) { _gamma.set_param(gamma); }
+void GammaNode::init(FloatParam *gamma) { _gamma.set_param(core(gamma)); }
+
+void GammaNode::create_node() {
+    _gamma.create_array(_batch_size);
+    RMX_COLOR_CREATE(rmx_create_gamma)
+}
+
+void GammaNode::update_node() {
+    _gamma.update_array();
+    const auto roi = roi_as_array(_inputs[0]->info().roi());
+    check(rmx_update_gamma(_node, roi.data(), _gamma.values().data()), "rmx_update_gamma");
+}
+
+ExposureNode::ExposureNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)
+    : Node(inputs, outputs), _exposure_factor(EXPOSURE_FACTOR_RANGE[0], EXPOSURE_FACTOR_RANGE[1]) {}
+void ExposureNode::init(float exposure_factor) { _exposure_factor.set_param(exposure_factor); }
+void ExposureNode::init(FloatParam *exposure_factor) { _exposure_factor.set_param(core(exposure_factor)); }
+
+void ExposureNode::create_node() {
+    _exposure_factor.create_array(_batch_size);
+    RMX_COLOR_CREATE(rmx_create_exposure)
+}
+
+void ExposureNode::update_node() {
+    _exposure_factor.update_array();
+    const auto roi = roi_as_array(_inputs[0]->info().roi());
+    check(rmx_update_exposure(_node, roi.data(), _exposure_factor.values().data()), "rmx_update_exposure");
+}
+
+ColorTemperatureNode::ColorTemperatureNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)
+    : Node(inputs, outputs), _adj_value_param(ADJUSTMENT_RANGE[0], ADJUSTMENT_RANGE[1]) {}
+void ColorTemperatureNode::init(int adjustment) { _adj_value_param.set_param(adjustment); }
+void ColorTemperatureNode::init(IntParam *adjustment) { _adj_value_param.set_param(core(adjustment)); }
+
+void ColorTemperatureNode::create_node() {
+    _adj_value_param.create_array(_batch_size);
+    RMX_COLOR_CREATE(rmx_create_color_temperature)
+}
+
+void ColorTemperatureNode::update_node() {
+    _adj_value_param.update_array();
+    const auto roi = roi_as_array(_inputs[0]->info().roi());
+    static_assert(sizeof(int) == sizeof(int32_t), "the adjustment array is handed over as int32");
+    check(rmx_update_color_temperature(_node, roi.data(), reinterpret_cast<const int32_t *>(_adj_value_param.values().data())),
+          "rmx_update_color_temperature");
+}
+
+BlendNode::BlendNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)
+    : Node(inputs, outputs), _ratio(RATIO_RANGE[0], RATIO_RANGE[1]) {}
+void BlendNode::init(float ratio) { _ratio.set_param(ratio); }
+void BlendNode::init(FloatParam *ratio) { _ratio.set_param(core(ratio)); }
+
+void BlendNode::create_node() {
+    if (_node) return;
+    if (_inputs.size() < 2) THROW("Blend node needs two input images")
+    // the kernel addresses both batches with one sample stride and one row stride
+    const rmx_tensor_desc a = _inputs[0]->info().desc(), b = _inputs[1]->info().desc();
+    if (a.n != b.n || a.h != b.h || a.w != b.w || a.c != b.c || a.layout != b.layout || a.dtype != b.dtype)
+        THROW("Blend node needs two inputs of the same shape, layout and data type")
+    _ratio.create_array(_batch_size);
+    RMX_COLOR_CREATE(rmx_create_blend)
+}
+
+void BlendNode::update_node() {
+    _ratio.update_array();
+    const auto roi = roi_as_array(_inputs[0]->info().roi());
+    check(rmx_update_blend(_node, roi.data(), _ratio.values().data()), "rmx_update_blend");
+}
+
+void BlendNode::launch() {
+    Tensor *in1 = _inputs[0], *in2 = _inputs[1], *out = _outputs[0];
+    if (!in1->buffer() || !in2->buffer() || !out->buffer()) THROW("tensor without a device buffer at launch")
+    check(rmx_op_launch2(_node, in1->buffer(), in2->buffer(), out->buffer()), "rmx_op_launch2");
+}
+
 /* ======================================================================= warp affine / rotate */
 
 WarpAffineNode::WarpAffineNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)

@@ -279,6 +279,71 @@ class SaturationNode : public Node {
     static constexpr float SAT_RANGE[2] = {-0.5f, 0.5f};
 };
 
+// node_gamma.cpp:28-60 (range node_gamma.h:41)
+class GammaNode : public Node {
+   public:
+    GammaNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float gamma);
+    void init(FloatParam *gamma);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _gamma;
+    static constexpr float GAMMA_RANGE[2] = {0.3f, 7.00f};
+};
+
+// node_exposure.cpp:28-60 (range node_exposure.h:42)
+class ExposureNode : public Node {
+   public:
+    ExposureNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float exposure_factor);
+    void init(FloatParam *exposure_factor);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _exposure_factor;
+    static constexpr float EXPOSURE_FACTOR_RANGE[2] = {0.15f, 0.95f};
+};
+
+// node_color_temperature.cpp:28-60 (integer adjustment, range node_color_temperature.h:43)
+class ColorTemperatureNode : public Node {
+   public:
+    ColorTemperatureNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(int adjustment);
+    void init(IntParam *adjustment);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<int> _adj_value_param;
+    static constexpr int ADJUSTMENT_RANGE[2] = {-99, 99};
+};
+
+// node_blend.cpp:27-66: two inputs of one shape, the first one's ROI (range node_blend.h:42)
+class BlendNode : public Node {
+   public:
+    BlendNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(float ratio);
+    void init(FloatParam *ratio);
+    void launch() override;
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    ParameterVX<float> _ratio;
+    static constexpr float RATIO_RANGE[2] = {0.1f, 0.9f};
+};
+
 // node_warp_affine.cpp:37-105
 class WarpAffineNode : public Node {
    public:

@@ -158,6 +158,19 @@ def test_crop_variants_and_point_ops(tmp_path):
     _same(o[4][0], orc.contrast(img, _roi(), one(1.3), one(70.0)), "contrast")
 
 
+def test_gamma_exposure_colour_temperature_blend_nodes(tmp_path):
+    full = (np.uint8, (N, H, W, 3))
+    img, outs, _ = _run("points", tmp_path, 5, [full] * 5)
+    one = lambda v: np.full(N, v, np.float32)
+    for o in outs:  # fixed parameters: both batches give the same result
+        _same(o[0][0], orc.gamma(img, _roi(), one(2.2)), "gamma")
+        _same(o[1][0], orc.exposure(img, _roi(), one(0.6)), "exposure")
+        _same(o[2][0], orc.color_temperature(img, _roi(), np.full(N, 40, np.int32)), "colour temperature")
+        bright = orc.brightness(img, _roi(), one(0.5), one(100.0))
+        _same(o[3][0], bright, "brightness")
+        _same(o[4][0], orc.blend(img, bright, _roi(), one(0.3)), "blend of the source and a node's output")
+
+
 def test_to_tensor_of_the_u8_output(tmp_path):
     """rocalToTensor (rocal_api_data_transfer.cpp:30-52 -> MasterGraph::to_tensor): planar fp16 with reversed
     channels of the whole output, then an interleaved fp32 tensor of its top-left max_roi corner."""
