@@ -5,7 +5,7 @@ A step is one pass of the hot path over one batch: the launch that replaces vxPr
 the fused node (what rocAL's own process timer brackets). Inputs and the per-batch parameter
 table are resident in HBM when the timed region starts. Prints ONE JSON line on stdout.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..6] [--all] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..10] [--all] [--no-cpu]
 """
 import argparse
 import json
@@ -29,6 +29,10 @@ WORKLOADS = {
     # the rows next to the path (measured with --all or --config; not the benchmark's configurations)
     5: "N1 ToTensor 224x224 u8 NHWC -> fp16 NCHW, reversed channels, batch 256",
     6: "N2 C1 (RandomResizedCrop+CropMirrorNormalize ->224x224 fp16 NCHW batch 256) reading a ragged, tightly packed source",
+    7: "N4 Gamma 224x224 u8->u8 NHWC batch 256",
+    8: "N4 Blend of two batches 224x224 u8->u8 NHWC batch 256",
+    9: "N4 Exposure 224x224 u8->u8 NHWC batch 256",
+    10: "N4 ColorTemperature 224x224 u8->u8 NHWC batch 256",
 }
 
 
@@ -132,6 +136,42 @@ def build_case(cfg, ctx, n=None):
             return orc.resize(padded[:k], roi6[:k], dw[:k], dw[:k], 224, 224, interp=orc.LINEAR, mirror=mirror6[:k],
                               scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16, flags=orc.F_QUANTIZE_U8)
         c = dict(img=packed)
+    elif cfg in (7, 8, 9, 10):
+        n = n or 256
+        c = wl.config2(n)
+        sd = ops.desc(n, 224, 224, ops.NHWC, ops.UINT8)
+        rng = np.random.default_rng(4321 + cfg)
+        img, roi = c["img"], c["roi"]
+        if cfg == 7:
+            p = rng.uniform(0.3, 7.0, n).astype(np.float32)  # the node's default range
+            op = ops.Gamma(ctx, sd, sd)
+            op.update(roi, p)
+        elif cfg == 8:
+            p = rng.uniform(0.1, 0.9, n).astype(np.float32)
+            img2 = np.ascontiguousarray(img[::-1])
+            op = ops.Blend(ctx, sd, sd)
+            op.update(roi, p)
+        elif cfg == 9:
+            p = rng.uniform(0.15, 0.95, n).astype(np.float32)
+            op = ops.Exposure(ctx, sd, sd)
+            op.update(roi, p)
+        else:
+            p = rng.integers(-99, 100, n).astype(np.int32)
+            op = ops.ColorTemperature(ctx, sd, sd)
+            op.update(roi, p)
+
+        def cpu(k):
+            from oracle import orc
+            if cfg == 7:
+                return orc.gamma(img[:k], roi[:k], p[:k])
+            if cfg == 8:
+                return orc.blend(img[:k], img2[:k], roi[:k], p[:k])
+            if cfg == 9:
+                return orc.exposure(img[:k], roi[:k], p[:k])
+            return orc.color_temperature(img[:k], roi[:k], p[:k])
+        if cfg == 8:
+            dst = op.alloc_output()
+            return op, (torch.from_numpy(img).cuda(), torch.from_numpy(img2).cuda()), dst, n, cpu
     else:
         raise SystemExit("unknown config %r" % cfg)
     src = torch.from_numpy(c["img"]).cuda()
@@ -142,14 +182,15 @@ def build_case(cfg, ctx, n=None):
 def time_launches(op, src, dst, steps, warmup):
     """K launches between two HIP events recorded on the stream the kernel runs on."""
     import torch
+    srcs = src if isinstance(src, tuple) else (src,)
     for _ in range(warmup):
-        op.launch(src, dst)
+        op.launch(*srcs, dst)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for _ in range(steps):
-        op.launch(src, dst)
+        op.launch(*srcs, dst)
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
