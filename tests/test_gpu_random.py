@@ -304,3 +304,66 @@ def test_random_ops_on_a_ragged_source(ctx, seed):
     op.launch(torch.from_numpy(padded).cuda(), out2)
     ctx.sync()
     assert np.array_equal(_bits(out2.cpu().numpy()), _bits(exp))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_gamma_exposure_temperature_blend(ctx, seed):
+    """The streaming neighbours of the colour family on exact-size buffers; every third case reads a ragged source
+    (the one-input ops) or, for Blend, windows that end on the last byte of both batches."""
+    import torch
+    rng = np.random.default_rng(7000 + seed)
+    n = int(rng.integers(1, 5))
+    H, W = int(rng.integers(4, 100)), int(rng.integers(4, 160))
+    kind = seed % 4
+    ragged = seed % 3 == 0 and kind != 3
+    layout = [ops.NHWC, ops.NCHW][int(rng.integers(0, 2))]
+    dtype = [ops.UINT8, ops.UINT8, ops.FP16, ops.FP32][int(rng.integers(0, 4))]
+    if ragged:
+        img, src, offsets, ws, hs, nbytes = _ragged(rng, n, H, W)
+        roi = _roi_in(rng, ws, hs)
+    else:
+        img, src = _src(rng, n, H, W)
+        roi = _rand_roi(rng, n, H, W)
+        if seed % 2 and W >= 8:  # whole 8-pixel groups reach the aligned kernels
+            roi[:, 2] = np.maximum(8, roi[:, 2] // 8 * 8)
+            roi[:, 0] = np.minimum(roi[:, 0], W - roi[:, 2])
+    if kind == 3:
+        roi[0] = (W - roi[0, 2], H - roi[0, 3], roi[0, 2], roi[0, 3])  # ends on the last pixel of the first image
+        roi[-1] = (W - 1, H - 1, 1, 1)
+    oh, ow = H, (W + 7) // 8 * 8 if seed % 2 else W
+    sd, dd = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, oh, ow, layout, dtype)
+    f = lambda lo, hi: rng.uniform(lo, hi, n).astype(np.float32)
+    kw = dict(layout=layout, dtype=dtype)
+
+    def fit(exp):  # the oracle writes an H x W destination; the op's may be wider
+        full = np.zeros((n, 3, oh, ow) if layout == ops.NCHW else (n, oh, ow, 3), exp.dtype)
+        if layout == ops.NCHW:
+            full[:, :, :H, :W] = exp
+        else:
+            full[:, :H, :W] = exp
+        return full
+
+    srcs = [src]
+    if kind == 0:
+        p = f(0.3, 7.0)
+        op, exp = ops.Gamma(ctx, sd, dd), orc.gamma(img, roi, p, **kw)
+    elif kind == 1:
+        p = f(-2.0, 2.0)
+        op, exp = ops.Exposure(ctx, sd, dd), orc.exposure(img, roi, p, **kw)
+    elif kind == 2:
+        p = rng.integers(-99, 100, n).astype(np.int32)
+        op, exp = ops.ColorTemperature(ctx, sd, dd), orc.color_temperature(img, roi, p, **kw)
+    else:
+        p = f(0.0, 1.0)
+        img2, src2 = _src(rng, n, H, W)
+        srcs.append(src2)
+        op, exp = ops.Blend(ctx, sd, dd), orc.blend(img, img2, roi, p, **kw)
+    if ragged:
+        op.set_ragged_source(offsets, ws, hs, nbytes)
+    op.update(roi, p)
+    out = op.alloc_output()
+    op.launch(*srcs, out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    exp = fit(exp)
+    assert np.array_equal(_bits(got), _bits(exp)), "seed %d kind %d (%s, %s): %d values differ" % (seed, kind, op.kernel_name, op.plan, int((got != exp).sum()))
