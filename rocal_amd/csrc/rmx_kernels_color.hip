@@ -12,9 +12,34 @@ namespace rmx {
 
 enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
 
-// Branch-free: every choice is a select. Lanes of a wavefront hold pixels of different hue sectors, so
+
+// HSV -> RGB per hue sector: each output channel is one of V, q = V - V*S*f, p = V - V*S, t = p + V*S*f. All four have the form
+// fma(sg, V*S*f, fma(nb, V*S, V)) with sg in {0,-1,+1} and nb in {0,-1}: a multiplication by 0 or +-1 is exact, so the two FMAs
+// round exactly where the subtraction and the addition of the plain formulas round. The six coefficients of a sector come from
+// a small LDS table indexed by the sector, which replaces the compare/select network (14 compares and selects per pixel).
+//   sector:  0 1 2 3 4 5      r: V q p p t V      g: t V V q p p      b: p p t V V q
+struct SectorRow {
+    float sg[3], nb0;  // sg of r,g,b ; nb of r
+    float nb1, nb2, pad0, pad1;  // nb of g,b
+};
+RMX_DEV void sector_row(int hi, SectorRow &row) {
+    // codes: 0 = V, 1 = q, 2 = p, 3 = t
+    const int rc[6] = {0, 1, 2, 2, 3, 0}, gc[6] = {3, 0, 0, 1, 2, 2}, bc[6] = {2, 2, 3, 0, 0, 1};
+    const int h = hi > 5 ? 5 : hi;
+    const int code[3] = {rc[h], gc[h], bc[h]};
+    float sg[3], nb[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        sg[c] = code[c] == 1 ? -1.0f : (code[c] == 3 ? 1.0f : 0.0f);
+        nb[c] = code[c] >= 2 ? -1.0f : 0.0f;
+    }
+    row.sg[0] = sg[0]; row.sg[1] = sg[1]; row.sg[2] = sg[2]; row.nb0 = nb[0];
+    row.nb1 = nb[1]; row.nb2 = nb[2]; row.pad0 = 0.0f; row.pad1 = 0.0f;
+}
+
+// Branch-free: lanes of a wavefront hold pixels of different hue sectors, so
 // branches would run every case one after the other under changing execution masks.
-RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, float alpha, float beta, float shift, float shift2, float shift4, float satf) {
+RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const SectorRow *sect, float alpha, float beta, float shift, float shift2, float shift4, float satf) {
     const float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
     const float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
     const float delta = cmax - cmin;
@@ -30,19 +55,14 @@ RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, float alph
     hh = hh >= 6.0f ? hh - 6.0f : hh;
     s = s * satf;
     s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
-    // sector and fraction: hh - (float)(int)hh, with the truncation kept in floating point
-    const float hi = __builtin_truncf(hh);
-    const float hf = hh - hi;
+    // sector and fraction; hh lies in [0, 6), where hh - floor(hh) is exact and equals hh - trunc(hh)
+    const SectorRow row = sect[(int)hh];
+    const float hf = __builtin_amdgcn_fractf(hh);
     const float vsat = cmax * s;
     const float vsatf = vsat * hf;
-    const float pp = cmax - vsat;
-    const float qq = cmax - vsatf;
-    const float tt = pp + vsatf;
-    // sector table (hi >= 5 is the last sector):  r: V q p p t V   g: t V V q p p   b: p p t V V q
-    const bool h0 = hi == 0.0f, h1 = hi == 1.0f, h2 = hi == 2.0f, h3 = hi == 3.0f, h4 = hi == 4.0f;
-    const float ro = h1 ? qq : ((h2 || h3) ? pp : (h4 ? tt : cmax));
-    const float go = h0 ? tt : ((h1 || h2) ? cmax : (h3 ? qq : pp));
-    const float bo = (h0 || h1) ? pp : (h2 ? tt : ((h3 || h4) ? cmax : qq));
+    const float ro = __builtin_fmaf(row.sg[0], vsatf, __builtin_fmaf(row.nb0, vsat, cmax));
+    const float go = __builtin_fmaf(row.sg[1], vsatf, __builtin_fmaf(row.nb1, vsat, cmax));
+    const float bo = __builtin_fmaf(row.sg[2], vsatf, __builtin_fmaf(row.nb2, vsat, cmax));
     r = __builtin_fmaf(ro, alpha, beta);
     g = __builtin_fmaf(go, alpha, beta);
     b = __builtin_fmaf(bo, alpha, beta);
@@ -51,9 +71,11 @@ RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, float alph
 template <typename T, int LAYOUT, int KIND, bool FAST>
 __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     __shared__ float rcp[256];
+    __shared__ __attribute__((aligned(16))) SectorRow sect[8];
     if constexpr (KIND == COLOR_TWIST) {
         int t = threadIdx.x;
         if (t < 256) rcp[t] = (t == 0) ? 0.0f : 1.0f / (float)t;
+        if (t < 8) sector_row(t, sect[t]);
         __syncthreads();
     }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
@@ -84,7 +106,7 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
 #pragma unroll
         for (int k = 0; k < PX; k++) {
             if constexpr (KIND == COLOR_TWIST) {
-                twist_px(v[0][k], v[1][k], v[2][k], rcp, p0, p1, p2, p2 + 2.0f, p2 + 4.0f, p3);
+                twist_px(v[0][k], v[1][k], v[2][k], rcp, sect, p0, p1, p2, p2 + 2.0f, p2 + 4.0f, p3);
             } else {
 #pragma unroll
                 for (int c = 0; c < 3; c++) v[c][k] = __builtin_fmaf(v[c][k] - p2, p0, p1);
@@ -103,7 +125,7 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
         if constexpr (FAST) {
             // whole groups and aligned destination rows: the loads of up to NI row steps go out together,
             // the stores follow (one memory round trip per strip, see the CropMirrorNormalize kernel)
-            constexpr int NI = (KIND == COLOR_TWIST) ? 2 : 4;
+            constexpr int NI = (KIND == COLOR_TWIST) ? 1 : 4;  // twist: one group per step keeps 65 registers (7 wavefronts per SIMD); two need 111
             for (int rb = r0 + lr; rb < r1 && lr < G; rb += NI * G) {
                 const uint32_t *q[NI];
                 uint32_t ph[NI];
