@@ -59,6 +59,12 @@ def cases():
     rocal = np.tile(np.array([x0, y0, x1, y1, o0, o1], np.float32), (n, 1))  # rocAL's fill order
     out["warp_rocal_params"] = rocal
     out["warp_affine"] = orc.warp_affine(img, full, np.stack([orc.affine_from_rocal(a) for a in rocal]), sw, sh, H, W)
+    # gamma 0.5, exposure 1, colour temperature 70, blend of the image with its 45-degree rotation at 0.5
+    # (unit_tests.cpp:759,804,796,767-768)
+    out["gamma"] = orc.gamma(img, full, one(0.5))
+    out["exposure"] = orc.exposure(img, full, one(1.0))
+    out["color_temperature"] = orc.color_temperature(img, full, np.full(n, 70, np.int32))
+    out["blend_with_rotate45"] = orc.blend(img, out["rotate45"], full, one(0.5))
     return out
 
 

@@ -1,6 +1,6 @@
 """The oracle reproduces the committed vectors (tests/golden/augment_golden.npz) bit for bit.
 The vectors are oracle outputs (see tests/golden/make_golden.py for why no reference-made
-vectors exist); this guards the oracle against drift between rounds and toolchains."""
+vectors exist); this guards the oracle against drift between revisions and toolchains."""
 import os
 import sys
 

@@ -162,6 +162,15 @@ def test_hip_path_reproduces_golden_vectors(ctx):
     size = (np.full(n, W, np.uint32), np.full(n, H, np.uint32))
     same(run(ops.Rotate(ctx, sd, sd, ops.LINEAR), full, one(45.0), *size), g["rotate45"], "rotate")
     same(run(ops.WarpAffine(ctx, sd, sd, ops.LINEAR), full, g["warp_rocal_params"], *size), g["warp_affine"], "warp affine")
+    same(run(ops.Gamma(ctx, sd, sd), full, one(0.5)), g["gamma"], "gamma")
+    same(run(ops.Exposure(ctx, sd, sd), full, one(1.0)), g["exposure"], "exposure")
+    same(run(ops.ColorTemperature(ctx, sd, sd), full, np.full(n, 70, np.int32)), g["color_temperature"], "colour temperature")
+    blend = ops.Blend(ctx, sd, sd)
+    blend.update(full, one(0.5))
+    out = blend.alloc_output()
+    blend.launch(gi, torch.from_numpy(g["rotate45"]).cuda(), out)
+    ctx.sync()
+    same(out.cpu().numpy(), g["blend_with_rotate45"], "blend")
 
 
 @pytest.mark.parametrize("nchw,fp16,reverse", [(1, 0, 0), (1, 1, 1), (0, 0, 0), (0, 0, 1), (1, 1, 0)])
