@@ -25,7 +25,7 @@ struct SectorRow {
 RMX_DEV void sector_row(int hi, SectorRow &row) {
     // codes: 0 = V, 1 = q, 2 = p, 3 = t
     const int rc[6] = {0, 1, 2, 2, 3, 0}, gc[6] = {3, 0, 0, 1, 2, 2}, bc[6] = {2, 2, 3, 0, 0, 1};
-    const int h = hi > 5 ? 5 : hi;
+    const int h = hi == 6 ? 0 : (hi > 5 ? 5 : hi);  // row 6 repeats row 0 (see the hue reduction), row 7 is never read
     const int code[3] = {rc[h], gc[h], bc[h]};
     float sg[3], nb[3];
 #pragma unroll
@@ -51,11 +51,12 @@ RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const Sect
     // sextant offset 0 / 2 / 4 plus the hue shift, the three sums made once per sample
     const float add = is_r ? shift : (is_g ? shift2 : shift4);
     float hh = __builtin_fmaf(num, rd, add);
-    hh = hh < 0.0f ? hh + 6.0f : hh;
-    hh = hh >= 6.0f ? hh - 6.0f : hh;
+    // back into [0, 6]: one addition of +6, -6 or 0. A value just below zero can round to exactly 6.0 here; row 6 of the sector
+    // table repeats row 0 and fract(6.0) is 0, which is the pixel a second reduction to 0.0 would give.
+    hh = hh + (hh < 0.0f ? 6.0f : (hh >= 6.0f ? -6.0f : 0.0f));
     s = s * satf;
     s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
-    // sector and fraction; hh lies in [0, 6), where hh - floor(hh) is exact and equals hh - trunc(hh)
+    // sector and fraction; hh lies in [0, 6], where hh - floor(hh) is exact and equals hh - trunc(hh)
     const SectorRow row = sect[(int)hh];
     const float hf = __builtin_amdgcn_fractf(hh);
     const float vsat = cmax * s;
@@ -102,11 +103,15 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     const uint8_t *buf_end = a.src + a.src_bytes;
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
 
+    // sextant offset 0 / 2 / 4 plus the hue shift, summed once per wavefront and kept in vector registers, so that the choice
+    // between them is two selects per pixel (from scalar registers the compiler selects a constant and adds the shift again)
+    float sh0 = p2, sh2 = p2 + 2.0f, sh4 = p2 + 4.0f;
+    if constexpr (KIND == COLOR_TWIST) asm volatile("" : "+v"(sh0), "+v"(sh2), "+v"(sh4));
     auto colour = [&](float (&v)[3][PX]) {
 #pragma unroll
         for (int k = 0; k < PX; k++) {
             if constexpr (KIND == COLOR_TWIST) {
-                twist_px(v[0][k], v[1][k], v[2][k], rcp, sect, p0, p1, p2, p2 + 2.0f, p2 + 4.0f, p3);
+                twist_px(v[0][k], v[1][k], v[2][k], rcp, sect, p0, p1, sh0, sh2, sh4, p3);
             } else {
 #pragma unroll
                 for (int c = 0; c < 3; c++) v[c][k] = __builtin_fmaf(v[c][k] - p2, p0, p1);
