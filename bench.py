@@ -5,7 +5,7 @@ A step is one pass of the hot path over one batch: the launch that replaces vxPr
 the fused node (what rocAL's own process timer brackets). Inputs and the per-batch parameter
 table are resident in HBM when the timed region starts. Prints ONE JSON line on stdout.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..10] [--all] [--no-cpu]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..11] [--all] [--no-cpu]
 """
 import argparse
 import json
@@ -33,6 +33,7 @@ WORKLOADS = {
     8: "N4 Blend of two batches 224x224 u8->u8 NHWC batch 256",
     9: "N4 Exposure 224x224 u8->u8 NHWC batch 256",
     10: "N4 ColorTemperature 224x224 u8->u8 NHWC batch 256",
+    11: "C1 with a ColorTwist node fused between RandomResizedCrop and CropMirrorNormalize (one launch), ->224x224 fp16 NCHW batch 256",
 }
 
 
@@ -136,6 +137,23 @@ def build_case(cfg, ctx, n=None):
             return orc.resize(padded[:k], roi6[:k], dw[:k], dw[:k], 224, 224, interp=orc.LINEAR, mirror=mirror6[:k],
                               scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16, flags=orc.F_QUANTIZE_U8)
         c = dict(img=packed)
+    elif cfg == 11:
+        n = n or 256
+        c = wl.config1(n)
+        tw = wl.config2(n)
+        scale, bias = scale_bias(n)
+        dw = np.full(n, 224, np.uint32)
+        colour = (tw["alpha"], tw["beta"], tw["hue"], tw["sat"])
+        op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR,
+                        flags=ops.F_QUANTIZE_U8 | ops.F_COLOR_TWIST)
+        op.update_color_cmn(c["roi"], dw, dw, scale, bias, colour, c["mirror"])
+
+        def cpu(k):  # the three reference nodes one after the other
+            from oracle import orc
+            mid = orc.resize(c["img"][:k], c["roi"][:k], dw[:k], dw[:k], 224, 224, interp=orc.LINEAR)
+            whole = np.tile(np.array([0, 0, 224, 224], np.uint32), (k, 1))
+            mid = orc.color_twist(mid, whole, *[p[:k] for p in colour])
+            return orc.crop_mirror_normalize(mid, whole, scale[:3 * k], bias[:3 * k], c["mirror"][:k], 224, 224, orc.NCHW, orc.FP16)
     elif cfg in (7, 8, 9, 10):
         n = n or 256
         c = wl.config2(n)

@@ -49,8 +49,13 @@ enum { RMX_INTERP_NEAREST = 0, RMX_INTERP_LINEAR = 1, RMX_INTERP_TRIANGULAR = 5 
 
 /* flags for resize-family ops */
 enum {
-    RMX_F_QUANTIZE_U8 = 1u << 0 /* round the resampled value to u8 before normalising: reproduces the
-                                   two-node graph resize(u8) -> CropMirrorNormalize in one pass */
+    RMX_F_QUANTIZE_U8 = 1u << 0, /* round the resampled value to u8 before normalising: reproduces the
+                                    two-node graph resize(u8) -> CropMirrorNormalize in one pass */
+    /* one colour node between the resize and the CropMirrorNormalize stage of a fused chain (bilinear, with
+     * RMX_F_QUANTIZE_U8): reproduces the three-node graph resize(u8) -> colour(u8) -> CropMirrorNormalize in one pass,
+     * the colour node's rounded, saturated u8 output included. Parameters come with rmx_update_resize_color_cmn. */
+    RMX_F_COLOR_LINEAR = 1u << 1, /* Brightness / Contrast / Exposure: fma(x - c2, c0, c1) */
+    RMX_F_COLOR_TWIST = 1u << 2   /* ColorTwist / Hue / Saturation: c0 alpha, c1 beta, c2 hue in degrees, c3 saturation */
 };
 
 /* TensorInfo of one side of a node (rocAL/include/pipeline/tensor.h:65-309): padded maxima. */
@@ -135,6 +140,15 @@ RMX_API int rmx_update_resize(rmx_op *op, const uint32_t *src_roi /*[N][4]*/, co
 RMX_API int rmx_update_resize_cmn(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w,
                                   const uint32_t *dst_h, const uint32_t *crop_roi, const float *scale,
                                   const float *bias, const uint32_t *mirror);
+
+/* Fused chain resize -> colour node -> CropMirrorNormalize for an op created with RMX_F_COLOR_LINEAR or RMX_F_COLOR_TWIST
+ * (the graph rocalCropResize / rocalResize -> rocalBrightness | rocalContrast | rocalColorTwist | rocalHue | rocalSaturation
+ * -> rocalCropMirrorNormalize, rocal_api_augmentation.h:67,125,237,302,794,826,878,925). c0..c3 are [N] arrays of the colour
+ * node's parameters as the flag's comment lists them; a NULL array takes the neutral value (1, 0, 0, 1). The other
+ * arguments are those of rmx_update_resize_cmn. */
+RMX_API int rmx_update_resize_color_cmn(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                                        const uint32_t *crop_roi, const float *scale, const float *bias, const uint32_t *mirror,
+                                        const float *c0, const float *c1, const float *c2, const float *c3);
 
 /* ---- Colour family (u8 NHWC -> u8 NHWC): replaces vxExtRppColorTwist (node_color_twist.cpp:48-49),
  *      vxExtRppBrightness (node_brightness.cpp:44), vxExtRppContrast (node_contrast.cpp:44),

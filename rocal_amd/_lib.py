@@ -47,6 +47,7 @@ _SIGS = {
     "rmx_create_resize": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.c_uint32, C.POINTER(_vp)],
     "rmx_update_resize": [_vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "rmx_update_resize_cmn": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
+    "rmx_update_resize_color_cmn": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
     "rmx_create_color_twist": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
     "rmx_update_color_twist": [_vp, _vp, _vp, _vp, _vp, _vp],
     "rmx_create_brightness": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],

@@ -488,6 +488,13 @@ int rmx_create_resize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor
         if (out) *out = nullptr;
         return fail(RMX_ERR_UNSUPPORTED, "interpolation %d is outside the hot path (nearest=0, linear=1, triangular=5)", interpolation);
     }
+    const uint32_t chain = flags & (RMX_F_COLOR_LINEAR | RMX_F_COLOR_TWIST);
+    if (chain) {
+        if (out) *out = nullptr;
+        if (chain == (RMX_F_COLOR_LINEAR | RMX_F_COLOR_TWIST)) return fail(RMX_ERR_INVALID, "a fused chain holds one colour node: linear or twist, not both");
+        if (!(flags & RMX_F_QUANTIZE_U8)) return fail(RMX_ERR_INVALID, "a colour node in the chain reads the u8 output of the resize node: RMX_F_QUANTIZE_U8 is required");
+        if (interpolation != RMX_INTERP_LINEAR) return fail(RMX_ERR_UNSUPPORTED, "the fused colour chain is built for bilinear resize only");
+    }
     int rc = make_op(ctx, OP_RESIZE, src, dst, roi_type, out);
     if (rc) return rc;
     (*out)->interp = interpolation;
@@ -505,6 +512,7 @@ static inline float src_coord_h(int u, float ratio, float off, float lo) {
 
 static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     const bool quant = (op->flags & RMX_F_QUANTIZE_U8) != 0;
+    const int chain = (op->flags & RMX_F_COLOR_LINEAR) ? 1 : (op->flags & RMX_F_COLOR_TWIST) ? 2 : 0;
     // a quantised value that is not normalised is stored through an identity FMA
     const bool knorm = norm || (quant && op->dst.dtype != RMX_UINT8);
     op->norm = knorm;
@@ -620,7 +628,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     const char *nm = nullptr;
     op->fn = (op->interp == RMX_INTERP_NEAREST)
                  ? rmx::select_resize_nearest_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm)
-                 : rmx::select_resize_linear_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm);
+                 : rmx::select_resize_linear_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &nm);
     op->kernel_name = nm;
     // x-tile: up to 64 lanes x 8 px. Each wave keeps a ring of R staged source rows in LDS;
     // R and the row pitch are computed per sample with the kernel's own float formulas.
@@ -733,7 +741,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             }
         }
         if (ok) {
-            op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->fast_name);
+            op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &op->fast_name);
             op->fast_lds = (need_max + 15) / 16 * 16;
             op->fast_rows = rows;
             op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
@@ -745,10 +753,15 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     return RMX_OK;
 }
 
+static float hue_to_sextants(float hue_deg);
+
 static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
                                 const uint32_t *crop_roi, const float *scale, const float *bias,
-                                const float *mean, const float *stddev, const uint32_t *mirror) {
+                                const float *mean, const float *stddev, const uint32_t *mirror, const float *const *colour = nullptr) {
     if (!op || op->kind != OP_RESIZE) return fail(RMX_ERR_INVALID, "op is not a Resize node");
+    const uint32_t chain = op->flags & (RMX_F_COLOR_LINEAR | RMX_F_COLOR_TWIST);
+    if (chain && !colour) return fail(RMX_ERR_INVALID, "this Resize node was created with a colour node in its chain: use rmx_update_resize_color_cmn");
+    if (!chain && colour) return fail(RMX_ERR_INVALID, "this Resize node was created without a colour node in its chain");
     if (!dst_w || !dst_h) return fail(RMX_ERR_INVALID, "dst_w and dst_h arrays are required");
     if ((mean == nullptr) != (stddev == nullptr)) return fail(RMX_ERR_INVALID, "mean and stddev must be given together");
     if ((scale == nullptr) != (bias == nullptr)) return fail(RMX_ERR_INVALID, "scale and bias must be given together");
@@ -801,6 +814,17 @@ static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint3
                 s.bias[c] = 0.0f;
             }
         }
+        if (chain == RMX_F_COLOR_LINEAR) {  // fma(x - c2, c0, c1)
+            s.m[0] = colour[0] ? colour[0][i] : 1.0f;
+            s.m[1] = colour[1] ? colour[1][i] : 0.0f;
+            s.m[2] = colour[2] ? colour[2][i] : 0.0f;
+            s.m[3] = 0.0f;
+        } else if (chain == RMX_F_COLOR_TWIST) {  // alpha, beta, hue shift in sextants, saturation
+            s.m[0] = colour[0] ? colour[0][i] : 1.0f;
+            s.m[1] = colour[1] ? colour[1][i] : 0.0f;
+            s.m[2] = colour[2] ? hue_to_sextants(colour[2][i]) : 0.0f;
+            s.m[3] = colour[3] ? colour[3][i] : 1.0f;
+        }
         // bytes of the source window actually mapped by the written window
         double fx = s.rs_w > 0 ? (double)s.dst_w / s.rs_w : 0, fy = s.rs_h > 0 ? (double)s.dst_h / s.rs_h : 0;
         bytes += (uint64_t)std::llround((double)s.src_w * s.src_h * fx * fy) * 3 +
@@ -821,6 +845,14 @@ int rmx_update_resize_cmn(rmx_op *op, const uint32_t *src_roi, const uint32_t *d
                           const uint32_t *crop_roi, const float *scale, const float *bias, const uint32_t *mirror) {
     if (!scale || !bias) return fail(RMX_ERR_INVALID, "scale and bias arrays are required");
     return update_resize_common(op, src_roi, dst_w, dst_h, crop_roi, scale, bias, nullptr, nullptr, mirror);
+}
+
+int rmx_update_resize_color_cmn(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h, const uint32_t *crop_roi,
+                                const float *scale, const float *bias, const uint32_t *mirror, const float *c0, const float *c1, const float *c2,
+                                const float *c3) {
+    if (!scale || !bias) return fail(RMX_ERR_INVALID, "scale and bias arrays are required");
+    const float *colour[4] = {c0, c1, c2, c3};
+    return update_resize_common(op, src_roi, dst_w, dst_h, crop_roi, scale, bias, nullptr, nullptr, mirror, colour);
 }
 
 /* ------------------------------------------------------------------ K3 family */

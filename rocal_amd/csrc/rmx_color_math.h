@@ -1,0 +1,104 @@
+// Colour arithmetic shared by the colour kernel and by the resize kernels that run a colour node between the resize and the
+// CropMirrorNormalize stage of a fused chain: the HSV twist of one pixel, its two LDS tables, and the chain stage itself.
+#pragma once
+#include "rmx_device.h"
+
+namespace rmx {
+
+// HSV -> RGB per hue sector: each output channel is one of V, q = V - V*S*f, p = V - V*S, t = p + V*S*f. All four have the form
+// fma(sg, V*S*f, fma(nb, V*S, V)) with sg in {0,-1,+1} and nb in {0,-1}: a multiplication by 0 or +-1 is exact, so the two FMAs
+// round exactly where the subtraction and the addition of the plain formulas round. The six coefficients of a sector come from
+// a small LDS table indexed by the sector, which replaces the compare/select network (14 compares and selects per pixel).
+//   sector:  0 1 2 3 4 5      r: V q p p t V      g: t V V q p p      b: p p t V V q
+struct SectorRow {
+    float sg[3], nb0;  // sg of r,g,b ; nb of r
+    float nb1, nb2, pad0, pad1;  // nb of g,b
+};
+RMX_DEV void sector_row(int hi, SectorRow &row) {
+    // codes: 0 = V, 1 = q, 2 = p, 3 = t
+    const int rc[6] = {0, 1, 2, 2, 3, 0}, gc[6] = {3, 0, 0, 1, 2, 2}, bc[6] = {2, 2, 3, 0, 0, 1};
+    const int h = hi == 6 ? 0 : (hi > 5 ? 5 : hi);  // row 6 repeats row 0 (see the hue reduction), row 7 is never read
+    const int code[3] = {rc[h], gc[h], bc[h]};
+    float sg[3], nb[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        sg[c] = code[c] == 1 ? -1.0f : (code[c] == 3 ? 1.0f : 0.0f);
+        nb[c] = code[c] >= 2 ? -1.0f : 0.0f;
+    }
+    row.sg[0] = sg[0]; row.sg[1] = sg[1]; row.sg[2] = sg[2]; row.nb0 = nb[0];
+    row.nb1 = nb[1]; row.nb2 = nb[2]; row.pad0 = 0.0f; row.pad1 = 0.0f;
+}
+
+// Branch-free: lanes of a wavefront hold pixels of different hue sectors, so
+// branches would run every case one after the other under changing execution masks.
+RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const SectorRow *sect, float alpha, float beta, float shift, float shift2, float shift4, float satf) {
+    const float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
+    const float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
+    const float delta = cmax - cmin;
+    const float rd = rcp[(int)delta];      // 0 when delta == 0
+    float s = delta * rcp[(int)cmax];
+    // A grey pixel needs no case of its own: r == g == b makes it a "red is largest" pixel with g - b == 0.
+    const bool is_r = cmax == r, is_g = cmax == g;
+    const float num = is_r ? (g - b) : (is_g ? (b - r) : (r - g));
+    // sextant offset 0 / 2 / 4 plus the hue shift, the three sums made once per sample
+    const float add = is_r ? shift : (is_g ? shift2 : shift4);
+    float hh = __builtin_fmaf(num, rd, add);
+    // back into [0, 6]: one addition of +6, -6 or 0. A value just below zero can round to exactly 6.0 here; row 6 of the sector
+    // table repeats row 0 and fract(6.0) is 0, which is the pixel a second reduction to 0.0 would give.
+    hh = hh + (hh < 0.0f ? 6.0f : (hh >= 6.0f ? -6.0f : 0.0f));
+    s = s * satf;
+    s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
+    // sector and fraction; hh lies in [0, 6], where hh - floor(hh) is exact and equals hh - trunc(hh)
+    const SectorRow row = sect[(int)hh];
+    const float hf = __builtin_amdgcn_fractf(hh);
+    const float vsat = cmax * s;
+    const float vsatf = vsat * hf;
+    const float ro = __builtin_fmaf(row.sg[0], vsatf, __builtin_fmaf(row.nb0, vsat, cmax));
+    const float go = __builtin_fmaf(row.sg[1], vsatf, __builtin_fmaf(row.nb1, vsat, cmax));
+    const float bo = __builtin_fmaf(row.sg[2], vsatf, __builtin_fmaf(row.nb2, vsat, cmax));
+    r = __builtin_fmaf(ro, alpha, beta);
+    g = __builtin_fmaf(go, alpha, beta);
+    b = __builtin_fmaf(bo, alpha, beta);
+}
+
+// The two tables of the twist in LDS: correctly rounded reciprocals of 0..255 (entry 0 is 0) and the sector coefficients.
+struct __attribute__((aligned(16))) ColorTables {
+    float rcp[256];
+    SectorRow sect[8];
+};
+
+// Fills the tables from one wavefront. Every wavefront of a workgroup writes the same values, so none has to wait for another:
+// each reads only what it has written itself.
+RMX_DEV void color_tables_fill(ColorTables *t, int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int v = lane + RMX_WAVE * i;
+        t->rcp[v] = (v == 0) ? 0.0f : 1.0f / (float)v;
+    }
+    if (lane < 8) sector_row(lane, t->sect[lane]);
+    wave_sync();
+}
+
+// Colour node in the middle of a fused chain resize(u8) -> colour(u8) -> CropMirrorNormalize: the values come in as the rounded
+// u8 output of the resize node and leave as the rounded, saturated u8 output of the colour node.
+//   CHAIN_LINEAR: fma(x - c2, c0, c1)   (Brightness: c0 = alpha, c1 = beta, c2 = 0; Contrast: c0 = factor, c1 = c2 = centre)
+//   CHAIN_TWIST : twist_px with alpha = c0, beta = c1, hue shift in sextants = c2 (sh2, sh4 = c2 + 2, c2 + 4), saturation = c3
+enum { CHAIN_NONE = 0, CHAIN_LINEAR = 1, CHAIN_TWIST = 2 };
+
+template <int CHAIN>
+RMX_DEV void chain_colour(float &o0, float &o1, float &o2, const float (&cp)[4], float sh2, float sh4, const ColorTables *t) {
+    if constexpr (CHAIN == CHAIN_LINEAR) {
+        o0 = __builtin_fmaf(o0 - cp[2], cp[0], cp[1]);
+        o1 = __builtin_fmaf(o1 - cp[2], cp[0], cp[1]);
+        o2 = __builtin_fmaf(o2 - cp[2], cp[0], cp[1]);
+    } else if constexpr (CHAIN == CHAIN_TWIST) {
+        twist_px(o0, o1, o2, t->rcp, t->sect, cp[0], cp[1], cp[2], sh2, sh4, cp[3]);
+    }
+    if constexpr (CHAIN != CHAIN_NONE) {
+        o0 = round_u8(o0);
+        o1 = round_u8(o1);
+        o2 = round_u8(o2);
+    }
+}
+
+}  // namespace rmx

@@ -6,68 +6,13 @@
 // come from a 256-entry LDS table of correctly rounded reciprocals, so the result is
 // bit-identical to IEEE division by the same integers without paying for a division per pixel.
 #include "rmx_device.h"
+#include "rmx_color_math.h"
 #include "rmx_launch.h"
 
 namespace rmx {
 
 enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
 
-
-// HSV -> RGB per hue sector: each output channel is one of V, q = V - V*S*f, p = V - V*S, t = p + V*S*f. All four have the form
-// fma(sg, V*S*f, fma(nb, V*S, V)) with sg in {0,-1,+1} and nb in {0,-1}: a multiplication by 0 or +-1 is exact, so the two FMAs
-// round exactly where the subtraction and the addition of the plain formulas round. The six coefficients of a sector come from
-// a small LDS table indexed by the sector, which replaces the compare/select network (14 compares and selects per pixel).
-//   sector:  0 1 2 3 4 5      r: V q p p t V      g: t V V q p p      b: p p t V V q
-struct SectorRow {
-    float sg[3], nb0;  // sg of r,g,b ; nb of r
-    float nb1, nb2, pad0, pad1;  // nb of g,b
-};
-RMX_DEV void sector_row(int hi, SectorRow &row) {
-    // codes: 0 = V, 1 = q, 2 = p, 3 = t
-    const int rc[6] = {0, 1, 2, 2, 3, 0}, gc[6] = {3, 0, 0, 1, 2, 2}, bc[6] = {2, 2, 3, 0, 0, 1};
-    const int h = hi == 6 ? 0 : (hi > 5 ? 5 : hi);  // row 6 repeats row 0 (see the hue reduction), row 7 is never read
-    const int code[3] = {rc[h], gc[h], bc[h]};
-    float sg[3], nb[3];
-#pragma unroll
-    for (int c = 0; c < 3; c++) {
-        sg[c] = code[c] == 1 ? -1.0f : (code[c] == 3 ? 1.0f : 0.0f);
-        nb[c] = code[c] >= 2 ? -1.0f : 0.0f;
-    }
-    row.sg[0] = sg[0]; row.sg[1] = sg[1]; row.sg[2] = sg[2]; row.nb0 = nb[0];
-    row.nb1 = nb[1]; row.nb2 = nb[2]; row.pad0 = 0.0f; row.pad1 = 0.0f;
-}
-
-// Branch-free: lanes of a wavefront hold pixels of different hue sectors, so
-// branches would run every case one after the other under changing execution masks.
-RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const SectorRow *sect, float alpha, float beta, float shift, float shift2, float shift4, float satf) {
-    const float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
-    const float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
-    const float delta = cmax - cmin;
-    const float rd = rcp[(int)delta];      // 0 when delta == 0
-    float s = delta * rcp[(int)cmax];
-    // A grey pixel needs no case of its own: r == g == b makes it a "red is largest" pixel with g - b == 0.
-    const bool is_r = cmax == r, is_g = cmax == g;
-    const float num = is_r ? (g - b) : (is_g ? (b - r) : (r - g));
-    // sextant offset 0 / 2 / 4 plus the hue shift, the three sums made once per sample
-    const float add = is_r ? shift : (is_g ? shift2 : shift4);
-    float hh = __builtin_fmaf(num, rd, add);
-    // back into [0, 6]: one addition of +6, -6 or 0. A value just below zero can round to exactly 6.0 here; row 6 of the sector
-    // table repeats row 0 and fract(6.0) is 0, which is the pixel a second reduction to 0.0 would give.
-    hh = hh + (hh < 0.0f ? 6.0f : (hh >= 6.0f ? -6.0f : 0.0f));
-    s = s * satf;
-    s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
-    // sector and fraction; hh lies in [0, 6], where hh - floor(hh) is exact and equals hh - trunc(hh)
-    const SectorRow row = sect[(int)hh];
-    const float hf = __builtin_amdgcn_fractf(hh);
-    const float vsat = cmax * s;
-    const float vsatf = vsat * hf;
-    const float ro = __builtin_fmaf(row.sg[0], vsatf, __builtin_fmaf(row.nb0, vsat, cmax));
-    const float go = __builtin_fmaf(row.sg[1], vsatf, __builtin_fmaf(row.nb1, vsat, cmax));
-    const float bo = __builtin_fmaf(row.sg[2], vsatf, __builtin_fmaf(row.nb2, vsat, cmax));
-    r = __builtin_fmaf(ro, alpha, beta);
-    g = __builtin_fmaf(go, alpha, beta);
-    b = __builtin_fmaf(bo, alpha, beta);
-}
 
 template <typename T, int LAYOUT, int KIND, bool FAST>
 __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {

@@ -15,6 +15,7 @@
 // The loads of step k+1 are issued before the arithmetic of step k and committed to LDS after
 // it, so HBM latency overlaps the blend. HBM-bound by design: window bytes in, tensor bytes out.
 #include "rmx_device.h"
+#include "rmx_color_math.h"
 #include "rmx_launch.h"
 
 namespace rmx {
@@ -99,8 +100,11 @@ RMX_DEV void stage_commit(const StageCtx &S, uint32_t *lds, int lane, int new_lo
     }
 }
 
-template <typename T, int LAYOUT, bool NORM, bool QUANT, bool NEAREST>
+// CHAIN: a colour node between the (quantised) resize and the normalisation, see chain_colour().
+template <typename T, int LAYOUT, bool NORM, bool QUANT, bool NEAREST, int CHAIN = CHAIN_NONE>
 __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
+    static_assert(CHAIN == CHAIN_NONE || (QUANT && !NEAREST), "a colour node in the chain reads the u8 output of a bilinear resize node");
+    __shared__ __attribute__((aligned(16))) float chain_tables[CHAIN == CHAIN_TWIST ? sizeof(ColorTables) / 4 : 4];
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const int wib = threadIdx.x / RMX_WAVE;
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
@@ -134,6 +138,11 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
         sc[c] = P.scale[c];
         bi[c] = P.bias[c];
     }
+    // colour node of a fused chain: its four parameters travel in the (otherwise unused) affine fields of the row
+    const float cp[4] = {P.m[0], P.m[1], P.m[2], P.m[3]};
+    const float sh2 = cp[2] + 2.0f, sh4 = cp[2] + 4.0f;
+    const ColorTables *ctab = reinterpret_cast<const ColorTables *>(chain_tables);
+    if constexpr (CHAIN == CHAIN_TWIST) color_tables_fill(reinterpret_cast<ColorTables *>(chain_tables), lane);
 
     StageCtx S;
     {
@@ -258,16 +267,27 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
                         v[2][k] = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte2(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte2(br) * wy * wx[k])));
                     }
                 }
-#pragma unroll
-                for (int c = 0; c < 3; c++)
+                if constexpr (CHAIN != CHAIN_NONE) {
 #pragma unroll
                     for (int k = 0; k < PX; k++) {
-                        float t = v[c][k];
-                        // a convex blend of u8 values stays inside [0,255]: rounding alone saturates it
-                        if constexpr (QUANT) t = NEAREST ? t : __builtin_rintf(t);
-                        if constexpr (NORM) t = __builtin_fmaf(t, sc[c], bi[c]);
-                        v[c][k] = t;
+                        float o0 = __builtin_rintf(v[0][k]), o1 = __builtin_rintf(v[1][k]), o2 = __builtin_rintf(v[2][k]);
+                        chain_colour<CHAIN>(o0, o1, o2, cp, sh2, sh4, ctab);
+                        v[0][k] = __builtin_fmaf(o0, sc[0], bi[0]);
+                        v[1][k] = __builtin_fmaf(o1, sc[1], bi[1]);
+                        v[2][k] = __builtin_fmaf(o2, sc[2], bi[2]);
                     }
+                } else {
+#pragma unroll
+                    for (int c = 0; c < 3; c++)
+#pragma unroll
+                        for (int k = 0; k < PX; k++) {
+                            float t = v[c][k];
+                            // a convex blend of u8 values stays inside [0,255]: rounding alone saturates it
+                            if constexpr (QUANT) t = NEAREST ? t : __builtin_rintf(t);
+                            if constexpr (NORM) t = __builtin_fmaf(t, sc[c], bi[c]);
+                            v[c][k] = t;
+                        }
+                }
                 const int x0 = hf ? (dw - t0 - cnt) : t0;
                 store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, x0, cnt, v, hf);
             }
@@ -298,36 +318,40 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
 }
 
 template <typename T, int LAYOUT, bool NEAREST>
-static KernelFn pick3(bool norm, bool quant) {
+static KernelFn pick3(bool norm, bool quant, int chain) {
+    if constexpr (!NEAREST) {
+        if (norm && quant && chain == CHAIN_LINEAR) return (KernelFn)rmx_resize_kernel<T, LAYOUT, true, true, false, CHAIN_LINEAR>;
+        if (norm && quant && chain == CHAIN_TWIST) return (KernelFn)rmx_resize_kernel<T, LAYOUT, true, true, false, CHAIN_TWIST>;
+    }
     if (norm && quant) return (KernelFn)rmx_resize_kernel<T, LAYOUT, true, true, NEAREST>;
     if (norm) return (KernelFn)rmx_resize_kernel<T, LAYOUT, true, false, NEAREST>;
     return (KernelFn)rmx_resize_kernel<T, LAYOUT, false, false, NEAREST>;
 }
 
 template <bool NEAREST>
-static KernelFn pick(int dtype, int layout, bool norm, bool quant) {
+static KernelFn pick(int dtype, int layout, bool norm, bool quant, int chain) {
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return pick3<float, RMX_NCHW, NEAREST>(norm, quant);
-            case RMX_FP16: return pick3<__half, RMX_NCHW, NEAREST>(norm, quant);
-            default: return pick3<uint8_t, RMX_NCHW, NEAREST>(norm, quant);
+            case RMX_FP32: return pick3<float, RMX_NCHW, NEAREST>(norm, quant, chain);
+            case RMX_FP16: return pick3<__half, RMX_NCHW, NEAREST>(norm, quant, chain);
+            default: return pick3<uint8_t, RMX_NCHW, NEAREST>(norm, quant, chain);
         }
     }
     switch (dtype) {
-        case RMX_FP32: return pick3<float, RMX_NHWC, NEAREST>(norm, quant);
-        case RMX_FP16: return pick3<__half, RMX_NHWC, NEAREST>(norm, quant);
-        default: return pick3<uint8_t, RMX_NHWC, NEAREST>(norm, quant);
+        case RMX_FP32: return pick3<float, RMX_NHWC, NEAREST>(norm, quant, chain);
+        case RMX_FP16: return pick3<__half, RMX_NHWC, NEAREST>(norm, quant, chain);
+        default: return pick3<uint8_t, RMX_NHWC, NEAREST>(norm, quant, chain);
     }
 }
 
-KernelFn select_resize_linear_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
+KernelFn select_resize_linear_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name) {
     *name = "rmx_resize_kernel";
-    return pick<false>(dtype, layout, norm, quant);
+    return pick<false>(dtype, layout, norm, quant, chain);
 }
 
 KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
     *name = "rmx_resize_kernel";
-    return pick<true>(dtype, layout, norm, quant);
+    return pick<true>(dtype, layout, norm, quant, 0);
 }
 
 }  // namespace rmx

@@ -22,6 +22,7 @@
 // v_fma_mix_f32 (bit-exact through the fp16-subnormal trick, fewer instructions, but each costs more
 // issue time), and tighter register budgets for 20-24 wavefronts per CU.
 #include "rmx_device.h"
+#include "rmx_color_math.h"
 #include "rmx_launch.h"
 
 #include <type_traits>
@@ -39,8 +40,11 @@ RMX_DEV float src_coord_f(int u, float ratio, float off, float lo) {
 
 constexpr int SB = 12;  // staging slots per lane issued back to back: 12 x 64 items = a 12 KB window
 
-template <typename T, int LAYOUT, bool NORM, bool QUANT>
+// CHAIN: a colour node between the (quantised) resize and the normalisation, see chain_colour().
+template <typename T, int LAYOUT, bool NORM, bool QUANT, int CHAIN>
 __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
+    static_assert(CHAIN == CHAIN_NONE || QUANT, "a colour node in the chain reads the u8 output of the resize node");
+    __shared__ __attribute__((aligned(16))) float chain_tables[CHAIN == CHAIN_TWIST ? sizeof(ColorTables) / 4 : 4];
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const int wib = threadIdx.x / RMX_WAVE;
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
@@ -79,6 +83,11 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
         sc[c] = P.scale[c];
         bi[c] = P.bias[c];
     }
+    // colour node of a fused chain: its four parameters travel in the (otherwise unused) affine fields of the row
+    const float cp[4] = {P.m[0], P.m[1], P.m[2], P.m[3]};
+    const float sh2 = cp[2] + 2.0f, sh4 = cp[2] + 4.0f;
+    const ColorTables *ctab = reinterpret_cast<const ColorTables *>(chain_tables);
+    if constexpr (CHAIN == CHAIN_TWIST) color_tables_fill(reinterpret_cast<ColorTables *>(chain_tables), lane);
 
     // source addressing: dword-aligned base below the sample, 32-bit byte offsets from it
     uint32_t row_stride;
@@ -232,6 +241,7 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
                     if constexpr (QUANT) {
                         o0 = __builtin_rintf(o0); o1 = __builtin_rintf(o1); o2 = __builtin_rintf(o2);
                     }
+                    chain_colour<CHAIN>(o0, o1, o2, cp, sh2, sh4, ctab);
                     if constexpr (NORM) {
                         o0 = __builtin_fmaf(o0, sc[0], bi[0]); o1 = __builtin_fmaf(o1, sc[1], bi[1]); o2 = __builtin_fmaf(o2, sc[2], bi[2]);
                     }
@@ -247,25 +257,28 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
 }
 
 template <typename T, int LAYOUT>
-static KernelFn pick3(bool norm, bool quant) {
-    if (norm && quant) return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, true, true>;
-    if (norm) return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, true, false>;
-    return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, false, false>;
+static KernelFn pick3(bool norm, bool quant, int chain) {
+    if (norm && quant && chain == CHAIN_LINEAR) return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, true, true, CHAIN_LINEAR>;
+    if (norm && quant && chain == CHAIN_TWIST) return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, true, true, CHAIN_TWIST>;
+    if (norm && quant) return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, true, true, CHAIN_NONE>;
+    if (norm) return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, true, false, CHAIN_NONE>;
+    return (KernelFn)rmx_resize_fast_kernel<T, LAYOUT, false, false, CHAIN_NONE>;
 }
 
-KernelFn select_resize_fast_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
+// chain: 0 none, 1 linear colour node, 2 colour twist between resize and normalisation (only with norm and quant)
+KernelFn select_resize_fast_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name) {
     *name = "rmx_resize_fast_kernel";
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return pick3<float, RMX_NCHW>(norm, quant);
-            case RMX_FP16: return pick3<__half, RMX_NCHW>(norm, quant);
-            default: return pick3<uint8_t, RMX_NCHW>(norm, quant);
+            case RMX_FP32: return pick3<float, RMX_NCHW>(norm, quant, chain);
+            case RMX_FP16: return pick3<__half, RMX_NCHW>(norm, quant, chain);
+            default: return pick3<uint8_t, RMX_NCHW>(norm, quant, chain);
         }
     }
     switch (dtype) {
-        case RMX_FP32: return pick3<float, RMX_NHWC>(norm, quant);
-        case RMX_FP16: return pick3<__half, RMX_NHWC>(norm, quant);
-        default: return pick3<uint8_t, RMX_NHWC>(norm, quant);
+        case RMX_FP32: return pick3<float, RMX_NHWC>(norm, quant, chain);
+        case RMX_FP16: return pick3<__half, RMX_NHWC>(norm, quant, chain);
+        default: return pick3<uint8_t, RMX_NHWC>(norm, quant, chain);
     }
 }
 

@@ -15,6 +15,7 @@ FP32, FP16, UINT8 = 0, 1, 2
 ROI_LTRB, ROI_XYWH = 0, 1
 NEAREST, LINEAR, TRIANGULAR = 0, 1, 5
 F_QUANTIZE_U8 = 1
+F_COLOR_LINEAR, F_COLOR_TWIST = 2, 4
 
 
 def _torch():
@@ -206,6 +207,13 @@ class Resize(Op):
     def update_cmn(self, src_roi, dst_w, dst_h, scale, bias, mirror=None, crop_roi=None):
         self._update("rmx_update_resize_cmn", (src_roi, _U), (dst_w, _U), (dst_h, _U), (crop_roi, _U), (scale, _F),
                      (bias, _F), (mirror, _U))
+
+
+    def update_color_cmn(self, src_roi, dst_w, dst_h, scale, bias, colour, mirror=None, crop_roi=None):
+        """colour: up to four [N] arrays (None = neutral) of the chain's colour node, see RMX_F_COLOR_LINEAR / _TWIST."""
+        c = list(colour) + [None] * (4 - len(colour))
+        self._update("rmx_update_resize_color_cmn", (src_roi, _U), (dst_w, _U), (dst_h, _U), (crop_roi, _U), (scale, _F), (bias, _F),
+                     (mirror, _U), (c[0], _F), (c[1], _F), (c[2], _F), (c[3], _F))
 
 
 class ColorTwist(Op):

@@ -1,0 +1,128 @@
+"""GPU parity of the fused chain resize(u8) -> colour node(u8) -> CropMirrorNormalize (one launch) against the CPU oracle
+running the three reference nodes one after the other, bit for bit. Covers the aligned fast kernel and the general one,
+both colour stages (linear: Brightness / Contrast / Exposure; twist: ColorTwist / Hue / Saturation), ragged windows,
+mirrors, crops inside the resized image, and the RandomResizedCrop configuration at full size."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from rocal_amd import ops, workloads as wl
+from rocal_amd._lib import RmxError
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint8)
+
+
+def _scale_bias(n):
+    inv = (1 / wl.STD).astype(np.float32)
+    return np.tile(inv, n), np.tile(-(wl.MEAN * inv), n)
+
+
+def _colour_params(kind, rng, n):
+    """(flag, arrays for the library, oracle function of (mid image, roi))"""
+    f = lambda lo, hi: rng.uniform(lo, hi, n).astype(np.float32)
+    one, zero = np.ones(n, np.float32), np.zeros(n, np.float32)
+    if kind == "brightness":
+        a, b = f(0.3, 2.0), f(-40, 40)
+        return ops.F_COLOR_LINEAR, (a, b), lambda m, r: orc.brightness(m, r, a, b)
+    if kind == "contrast":
+        fa, ce = f(0.3, 2.5), f(0, 255)
+        return ops.F_COLOR_LINEAR, (fa, ce, ce), lambda m, r: orc.contrast(m, r, fa, ce)
+    if kind == "twist":
+        a, b, h, s = f(0.5, 1.8), f(-30, 30), f(-180, 180), f(0.0, 2.0)
+        return ops.F_COLOR_TWIST, (a, b, h, s), lambda m, r: orc.color_twist(m, r, a, b, h, s)
+    if kind == "hue":
+        h = f(-360, 360)
+        return ops.F_COLOR_TWIST, (None, None, h, None), lambda m, r: orc.color_twist(m, r, one, zero, h, one)
+    s = f(0.0, 3.0)
+    return ops.F_COLOR_TWIST, (None, None, None, s), lambda m, r: orc.color_twist(m, r, one, zero, zero, s)
+
+
+def _expected(img, roi, rw, rh, crop, scale, bias, mirror, oh, ow, layout, dtype, colour_fn):
+    n = img.shape[0]
+    mid = orc.resize(img, roi, rw, rh, int(rh.max()), int(rw.max()), interp=orc.LINEAR)
+    whole = np.stack([np.zeros(n), np.zeros(n), rw, rh], -1).astype(np.uint32)
+    mid = colour_fn(mid, whole)
+    return orc.crop_mirror_normalize(mid, crop, scale, bias, mirror, oh, ow, layout, dtype)
+
+
+@pytest.mark.parametrize("aligned", [True, False])
+@pytest.mark.parametrize("kind", ["brightness", "contrast", "twist", "hue", "saturation"])
+def test_resize_colour_cmn_chain(ctx, kind, aligned):
+    import torch
+    rng = np.random.default_rng(sum(map(ord, kind)) * 2 + int(aligned))
+    n, H, W = 5, 90, 120
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.5)
+    img[0] = rng.integers(0, 256, (H, W, 3), dtype=np.uint8)
+    roi = np.empty((n, 4), np.uint32)
+    for i in range(n):
+        w, h = int(rng.integers(8, W + 1)), int(rng.integers(8, H + 1))
+        roi[i] = (int(rng.integers(0, W - w + 1)), int(rng.integers(0, H - h + 1)), w, h)
+    rw = (rng.integers(3, 12, n) * 8).astype(np.uint32) if aligned else rng.integers(20, 90, n).astype(np.uint32)
+    rh = rng.integers(10, 70, n).astype(np.uint32)
+    crop = np.empty((n, 4), np.uint32)
+    for i in range(n):
+        cw = int(rng.integers(1, rw[i] // 8 + 1)) * 8 if aligned else int(rng.integers(1, rw[i] + 1))
+        ch = int(rng.integers(1, rh[i] + 1))
+        crop[i] = (int(rng.integers(0, rw[i] - cw + 1)), int(rng.integers(0, rh[i] - ch + 1)), cw, ch)
+    oh, ow = int(crop[:, 3].max()), int(crop[:, 2].max())
+    mirror = rng.integers(0, 2, n).astype(np.uint32)
+    scale, bias = _scale_bias(n)
+    flag, arrays, colour_fn = _colour_params(kind, rng, n)
+    for layout, dtype in ((ops.NCHW, ops.FP16), (ops.NHWC, ops.FP32)):
+        op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, oh, ow, layout, dtype), ops.LINEAR,
+                        flags=ops.F_QUANTIZE_U8 | flag)
+        op.update_color_cmn(roi, rw, rh, scale, bias, arrays, mirror, crop)
+        assert op.kernel_name == ("rmx_resize_fast_kernel" if aligned else "rmx_resize_kernel")
+        out = op.alloc_output()
+        op.launch(torch.from_numpy(img).cuda(), out)
+        ctx.sync()
+        got = out.cpu().numpy()
+        exp = _expected(img, roi, rw, rh, crop, scale, bias, mirror, oh, ow, layout, dtype, colour_fn)
+        assert np.array_equal(_bits(got), _bits(exp)), "%s aligned=%s (%s, %s): %d values differ" % (kind, aligned, op.kernel_name, op.plan, int((got != exp).sum()))
+
+
+def test_random_resized_crop_colour_twist_cmn_full_size(ctx):
+    """The RandomResizedCrop + CropMirrorNormalize configuration (256 ragged images -> 224 x 224 fp16 NCHW) with a
+    ColorTwist node between the two, every value compared."""
+    import torch
+    n = 256
+    c = wl.config1(n)
+    c2 = wl.config2(n)
+    scale, bias = _scale_bias(n)
+    dw = np.full(n, 224, np.uint32)
+    op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR,
+                    flags=ops.F_QUANTIZE_U8 | ops.F_COLOR_TWIST)
+    arrays = (c2["alpha"], c2["beta"], c2["hue"], c2["sat"])
+    op.update_color_cmn(c["roi"], dw, dw, scale, bias, arrays, c["mirror"])
+    assert op.kernel_name == "rmx_resize_fast_kernel"
+    out = op.alloc_output()
+    op.launch(torch.from_numpy(c["img"]).cuda(), out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    whole = np.tile(np.array([0, 0, 224, 224], np.uint32), (n, 1))
+    exp = _expected(c["img"], c["roi"], dw, dw, whole, scale, bias, c["mirror"], 224, 224, orc.NCHW, orc.FP16,
+                    lambda m, r: orc.color_twist(m, r, *arrays))
+    assert np.array_equal(_bits(got), _bits(exp)), "%d values differ" % int((got != exp).sum())
+
+
+def test_chain_protocol_errors(ctx):
+    n = 2
+    sd, dd = ops.desc(n, 32, 32, ops.NHWC, ops.UINT8), ops.desc(n, 16, 16, ops.NCHW, ops.FP16)
+    with pytest.raises(RmxError, match="QUANTIZE"):
+        ops.Resize(ctx, sd, dd, ops.LINEAR, flags=ops.F_COLOR_TWIST)
+    with pytest.raises(RmxError, match="not both"):
+        ops.Resize(ctx, sd, dd, ops.LINEAR, flags=ops.F_QUANTIZE_U8 | ops.F_COLOR_TWIST | ops.F_COLOR_LINEAR)
+    with pytest.raises(RmxError, match="bilinear"):
+        ops.Resize(ctx, sd, dd, ops.TRIANGULAR, flags=ops.F_QUANTIZE_U8 | ops.F_COLOR_LINEAR)
+    scale, bias = _scale_bias(n)
+    dw = np.full(n, 16, np.uint32)
+    chain = ops.Resize(ctx, sd, dd, ops.LINEAR, flags=ops.F_QUANTIZE_U8 | ops.F_COLOR_LINEAR)
+    with pytest.raises(RmxError, match="rmx_update_resize_color_cmn"):
+        chain.update_cmn(None, dw, dw, scale, bias)
+    plain = ops.Resize(ctx, sd, dd, ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+    with pytest.raises(RmxError, match="without a colour node"):
+        plain.update_color_cmn(None, dw, dw, scale, bias, (np.ones(n, np.float32),))
