@@ -164,7 +164,7 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
     RocalTensor src = rocalDeviceSource(ctx, W, H, false);
     std::vector<float> mean{123.675f, 116.28f, 103.53f}, stdv{58.395f, 57.12f, 57.375f};
     std::vector<RocalTensor> outs;
-    RocalTensor mid = nullptr;
+    RocalTensor mid = nullptr, mid2 = nullptr;
     // A fair coin for the mirror flags, created first so that it takes the first seed of the sequence.
     // (rocalCreateIntUniformRand(0, 1) truncates to 0 for every draw but one in 2^32, as in the reference.)
     const int coin_v[2] = {0, 1};
@@ -211,6 +211,14 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         mid = rocalCropResizeFixed(ctx, src, 64, 64, false, 0.5f, 1.2f, 0.3f, 0.7f);
         RocalIntParam mirror = coin;
         outs.push_back(rocalCropMirrorNormalize(ctx, mid, 56, 56, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP16));
+    } else if (scenario == "rrc_twist_cmn" || scenario == "rrc_contrast_cmn") {
+        // three nodes, two virtual tensors between them: one kernel
+        mid = rocalCropResizeFixed(ctx, src, 64, 64, false, 0.5f, 1.2f, 0.3f, 0.7f);
+        RocalTensor col = scenario == "rrc_twist_cmn" ? rocalColorTwistFixed(ctx, mid, 1.2f, 8.0f, 40.0f, 1.3f, false)
+                                                        : rocalContrastFixed(ctx, mid, 1.4f, 100.0f, false);
+        RocalIntParam mirror = coin;
+        outs.push_back(rocalCropMirrorNormalize(ctx, col, 56, 56, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP16));
+        mid2 = col;
     } else if (scenario == "chain") {
         RocalTensor a = rocalResize(ctx, src, 40, 32, false);
         RocalTensor b = rocalColorTwistFixed(ctx, a, 1.1f, 5.0f, 30.0f, 1.2f, true);
@@ -271,6 +279,7 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         return 7;
     }
     if (mid) std::cout << "intermediate_elided " << (rocalTensorBuffer(mid) == nullptr ? 1 : 0) << std::endl;
+    if (mid2) std::cout << "second_intermediate_elided " << (rocalTensorBuffer(mid2) == nullptr ? 1 : 0) << std::endl;
     for (int b = 0; b < 2; b++) {
         if (with_boxes && rocalSetBoundingBoxes(ctx, box_counts.data(), box_ltrb.data(), box_labels.data()) != ROCAL_OK) return 12;
         if (rocalDeviceSourceFeed(ctx, src, dev, rw.data(), rh.data()) != ROCAL_OK || rocalRun(ctx) != ROCAL_OK) {

@@ -197,10 +197,21 @@ bool ResizeFamilyNode::try_absorb(Node *next) {
     return true;
 }
 
+bool ResizeFamilyNode::try_absorb_chain(Node *colour, Node *next) {
+    const unsigned kind = colour->chain_colour_kind();
+    if (!kind || _interpolation_type != ROCAL_LINEAR_INTERPOLATION) return false;
+    // the colour node must hand a u8 NHWC image on, as the resize node does
+    const TensorInfo &mid = colour->output()[0]->info();
+    if (mid.data_type() != RocalTensorDataType::UINT8 || mid.layout() != RocalTensorlayout::NHWC) return false;
+    if (!try_absorb(next)) return false;
+    _absorbed_colour = colour;
+    return true;
+}
+
 void ResizeFamilyNode::create_resize_op(int interpolation) {
     const TensorInfo &out = (_absorbed ? _absorbed->output()[0] : _outputs[0])->info();
     rmx_tensor_desc s = _inputs[0]->info().desc(), d = out.desc();
-    const uint32_t flags = _absorbed ? RMX_F_QUANTIZE_U8 : 0;
+    const uint32_t flags = (_absorbed ? RMX_F_QUANTIZE_U8 : 0) | (_absorbed_colour ? _absorbed_colour->chain_colour_kind() : 0);
     check(rmx_create_resize(_graph->get(), &s, &d, interpolation, (int)RocalROIType::XYWH, flags, &_node), "rmx_create_resize");
 }
 
@@ -211,6 +222,14 @@ void ResizeFamilyNode::update_resize_op(const std::vector<uint32_t> &window, con
         _absorbed->refresh_for_fusion();
         const auto crop = _absorbed->get_crop_param()->xywh();
         const auto m = as_u32(_absorbed->mirror_values());
+        if (_absorbed_colour) {
+            const float *c[4];
+            _absorbed_colour->chain_colour_refresh(c);
+            check(rmx_update_resize_color_cmn(_node, window.data(), dst_w.data(), dst_h.data(), crop.data(), _absorbed->_scale.data(), _absorbed->_bias.data(),
+                                              m.data(), c[0], c[1], c[2], c[3]),
+                  "rmx_update_resize_color_cmn");
+            return;
+        }
         check(rmx_update_resize_cmn(_node, window.data(), dst_w.data(), dst_h.data(), crop.data(), _absorbed->_scale.data(), _absorbed->_bias.data(), m.data()),
               "rmx_update_resize_cmn");
         return;
@@ -471,7 +490,16 @@ void ColorTwistNode::create_node() {
     RMX_COLOR_CREATE(rmx_create_color_twist)
 }
 
+void ColorTwistNode::chain_colour_refresh(const float *arrays[4]) {
+    for (auto *p : {&_alpha, &_beta, &_hue, &_sat}) p->update_array();
+    arrays[0] = _alpha.values().data();
+    arrays[1] = _beta.values().data();
+    arrays[2] = _hue.values().data();
+    arrays[3] = _sat.values().data();
+}
+
 void ColorTwistNode::update_node() {
+    if (fused_away) return;  // renewed by the resize node that runs the chain
     for (auto *p : {&_alpha, &_beta, &_hue, &_sat}) p->update_array();
     const auto roi = roi_as_array(_inputs[0]->info().roi());
     check(rmx_update_color_twist(_node, roi.data(), _alpha.values().data(), _beta.values().data(), _hue.values().data(), _sat.values().data()),
@@ -497,7 +525,16 @@ void BrightnessNode::create_node() {
     RMX_COLOR_CREATE(rmx_create_brightness)
 }
 
+void BrightnessNode::chain_colour_refresh(const float *arrays[4]) {
+    _alpha.update_array();
+    _beta.update_array();
+    arrays[0] = _alpha.values().data();
+    arrays[1] = _beta.values().data();
+    arrays[2] = arrays[3] = nullptr;
+}
+
 void BrightnessNode::update_node() {
+    if (fused_away) return;
     _alpha.update_array();
     _beta.update_array();
     const auto roi = roi_as_array(_inputs[0]->info().roi());
@@ -523,7 +560,16 @@ void ContrastNode::create_node() {
     RMX_COLOR_CREATE(rmx_create_contrast)
 }
 
+void ContrastNode::chain_colour_refresh(const float *arrays[4]) {  // fma(x - centre, factor, centre)
+    _factor.update_array();
+    _center.update_array();
+    arrays[0] = _factor.values().data();
+    arrays[1] = arrays[2] = _center.values().data();
+    arrays[3] = nullptr;
+}
+
 void ContrastNode::update_node() {
+    if (fused_away) return;
     _factor.update_array();
     _center.update_array();
     const auto roi = roi_as_array(_inputs[0]->info().roi());
@@ -539,7 +585,14 @@ void HueNode::create_node() {
     RMX_COLOR_CREATE(rmx_create_hue)
 }
 
+void HueNode::chain_colour_refresh(const float *arrays[4]) {
+    _hue.update_array();
+    arrays[0] = arrays[1] = arrays[3] = nullptr;
+    arrays[2] = _hue.values().data();
+}
+
 void HueNode::update_node() {
+    if (fused_away) return;
     _hue.update_array();
     const auto roi = roi_as_array(_inputs[0]->info().roi());
     check(rmx_update_hue(_node, roi.data(), _hue.values().data()), "rmx_update_hue");
@@ -555,7 +608,14 @@ void SaturationNode::create_node() {
     RMX_COLOR_CREATE(rmx_create_saturation)
 }
 
+void SaturationNode::chain_colour_refresh(const float *arrays[4]) {
+    _sat.update_array();
+    arrays[0] = arrays[1] = arrays[2] = nullptr;
+    arrays[3] = _sat.values().data();
+}
+
 void SaturationNode::update_node() {
+    if (fused_away) return;
     _sat.update_array();
     const auto roi = roi_as_array(_inputs[0]->info().roi());
     check(rmx_update_saturation(_node, roi.data(), _sat.values().data()), "rmx_update_saturation");

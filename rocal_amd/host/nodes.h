@@ -106,6 +106,7 @@ class ResizeFamilyNode : public Node {
    public:
     using Node::Node;
     bool try_absorb(Node *next) override;
+    bool try_absorb_chain(Node *colour, Node *cmn) override;
     // the resize target (the padded output size), as the reference's metadata nodes read it
     unsigned get_dst_width() { return (unsigned)_outputs[0]->info().max_shape()[0]; }
     unsigned get_dst_height() { return (unsigned)_outputs[0]->info().max_shape()[1]; }
@@ -122,6 +123,7 @@ class ResizeFamilyNode : public Node {
                                     unsigned max_w, unsigned max_h);
     int _interpolation_type = ROCAL_LINEAR_INTERPOLATION;
     CropMirrorNormalizeNode *_absorbed = nullptr;
+    Node *_absorbed_colour = nullptr;  // the colour node between this node and _absorbed, when the three run as one kernel
 };
 
 // node_resize.cpp:31-138
@@ -204,6 +206,8 @@ class ColorTwistNode : public Node {
     ColorTwistNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float alpha, float beta, float hue, float sat);
     void init(FloatParam *alpha, FloatParam *beta, FloatParam *hue, FloatParam *sat);
+    unsigned chain_colour_kind() const override { return RMX_F_COLOR_TWIST; }
+    void chain_colour_refresh(const float *arrays[4]) override;
 
    protected:
     void create_node() override;
@@ -222,6 +226,8 @@ class BrightnessNode : public Node {
     BrightnessNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float alpha, float beta);
     void init(FloatParam *alpha, FloatParam *beta);
+    unsigned chain_colour_kind() const override { return RMX_F_COLOR_LINEAR; }
+    void chain_colour_refresh(const float *arrays[4]) override;
 
    protected:
     void create_node() override;
@@ -238,6 +244,8 @@ class ContrastNode : public Node {
     ContrastNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float contrast_factor, float contrast_center);
     void init(FloatParam *contrast_factor, FloatParam *contrast_center);
+    unsigned chain_colour_kind() const override { return RMX_F_COLOR_LINEAR; }
+    void chain_colour_refresh(const float *arrays[4]) override;
 
    protected:
     void create_node() override;
@@ -254,6 +262,8 @@ class HueNode : public Node {
     HueNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float hue);
     void init(FloatParam *hue);
+    unsigned chain_colour_kind() const override { return RMX_F_COLOR_TWIST; }
+    void chain_colour_refresh(const float *arrays[4]) override;
 
    protected:
     void create_node() override;
@@ -269,6 +279,8 @@ class SaturationNode : public Node {
     SaturationNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float sat);
     void init(FloatParam *sat);
+    unsigned chain_colour_kind() const override { return RMX_F_COLOR_TWIST; }
+    void chain_colour_refresh(const float *arrays[4]) override;
 
    protected:
     void create_node() override;

@@ -94,6 +94,24 @@ Graph::~Graph() { release(); }
 // Chain planning: a node may take over the work of the node that follows it (resize -> CropMirrorNormalize
 // through a virtual tensor nobody else reads). Everything else about verification happens in rmx_create_*.
 Graph::Status Graph::verify() {
+    auto readers = [&](Tensor *t) {
+        int n = 0;
+        for (Node *k : _order)
+            for (Tensor *in : k->input()) n += (in == t);
+        return n;
+    };
+    // resize -> colour node -> CropMirrorNormalize through two virtual tensors nobody else reads
+    for (size_t i = 0; i + 2 < _order.size(); i++) {
+        Node *a = _order[i], *b = _order[i + 1], *c = _order[i + 2];
+        if (a->fused_away || b->fused_away || c->fused_away) continue;
+        Tensor *mid1 = a->output()[0], *mid2 = b->output()[0];
+        if (b->input().size() != 1 || b->input()[0] != mid1 || c->input()[0] != mid2 || mid1->is_output || mid2->is_output) continue;
+        if (readers(mid1) != 1 || readers(mid2) != 1) continue;
+        if (a->try_absorb_chain(b, c)) {
+            b->fused_away = c->fused_away = true;
+            mid1->elided = mid2->elided = true;
+        }
+    }
     for (size_t i = 0; i + 1 < _order.size(); i++) {
         Node *a = _order[i], *b = _order[i + 1];
         if (a->fused_away || b->fused_away) continue;

@@ -116,6 +116,12 @@ class Node {
     bool fused_away = false;  // this node's work is done by the launch of the node that precedes it
     // A CropMirrorNormalize node directly behind a resize node: the pair runs as one kernel.
     virtual bool try_absorb(Node *) { return false; }
+    // A colour node and a CropMirrorNormalize node directly behind a bilinear resize node: the three run as one kernel.
+    virtual bool try_absorb_chain(Node *, Node *) { return false; }
+    // A colour node that can be the middle of such a chain says which stage it is (RMX_F_COLOR_LINEAR / RMX_F_COLOR_TWIST, 0 = none)
+    // and, per batch, renews its parameters and hands out their arrays (NULL = neutral value).
+    virtual unsigned chain_colour_kind() const { return 0; }
+    virtual void chain_colour_refresh(const float *arrays[4]) { arrays[0] = arrays[1] = arrays[2] = arrays[3] = nullptr; }
 
    protected:
     virtual void create_node() = 0;

@@ -99,6 +99,32 @@ def test_random_resized_crop_then_cmn_runs_as_one_kernel(tmp_path):
         assert np.array_equal(roi[:, 2:], crop[:, 2:])
 
 
+@pytest.mark.parametrize("scenario", ["rrc_twist_cmn", "rrc_contrast_cmn"])
+def test_random_resized_crop_colour_cmn_runs_as_one_kernel(tmp_path, scenario):
+    img, outs, log = _run(scenario, tmp_path, 1, [(np.float16, (N, 3, 56, 56))])
+    assert "intermediate_elided 1" in log and "second_intermediate_elided 1" in log  # neither u8 tensor is materialised
+    s = orc.FParam.simple
+    window = np.stack([orc.random_crop(s(0.5), s(1.2), s(0.3), s(0.7), w, h) for w, h in ROIS])
+    full = np.full(N, 64, np.uint32)
+    mid = orc.resize(img, window, full, full, 64, 64, interp=orc.LINEAR)
+    mid_w, mid_h = np.minimum(window[:, 2], 64), np.minimum(window[:, 3], 64)
+    one = lambda v: np.full(N, v, np.float32)
+    # the colour node works on the ROI the resize node publishes for its output
+    mid_roi = np.stack([np.zeros(N), np.zeros(N), mid_w, mid_h], -1).astype(np.uint32)
+    if scenario == "rrc_twist_cmn":
+        mid = orc.color_twist(mid, mid_roi, one(1.2), one(8.0), one(40.0), one(1.3))
+    else:
+        mid = orc.contrast(mid, mid_roi, one(1.4), one(100.0))
+    crop = np.stack([orc.fixed_crop(int(w), int(h), 56, 56, anchor=(0.5, 0.5)) for w, h in zip(mid_w, mid_h)])
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    mirrors = _coin_batches(2)
+    for b in range(2):
+        got, roi = outs[b][0]
+        exp = orc.crop_mirror_normalize(mid, crop, scale, bias, mirrors[b], 56, 56, orc.NCHW, orc.FP16)
+        _same(got, exp, "%s batch %d" % (scenario, b))
+        assert np.array_equal(roi[:, 2:], crop[:, 2:])
+
+
 def test_resize_colortwist_flip_chain_with_intermediate_tensors(tmp_path):
     img, outs, _ = _run("chain", tmp_path, 2, [(np.uint8, (N, 32, 40, 3))] * 2)
     dw, dh = np.full(N, 40, np.uint32), np.full(N, 32, np.uint32)
