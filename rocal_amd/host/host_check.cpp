@@ -211,11 +211,12 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         mid = rocalCropResizeFixed(ctx, src, 64, 64, false, 0.5f, 1.2f, 0.3f, 0.7f);
         RocalIntParam mirror = coin;
         outs.push_back(rocalCropMirrorNormalize(ctx, mid, 56, 56, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP16));
-    } else if (scenario == "rrc_twist_cmn" || scenario == "rrc_contrast_cmn") {
+    } else if (scenario == "rrc_twist_cmn" || scenario == "rrc_contrast_cmn" || scenario == "rrc_exposure_cmn") {
         // three nodes, two virtual tensors between them: one kernel
         mid = rocalCropResizeFixed(ctx, src, 64, 64, false, 0.5f, 1.2f, 0.3f, 0.7f);
-        RocalTensor col = scenario == "rrc_twist_cmn" ? rocalColorTwistFixed(ctx, mid, 1.2f, 8.0f, 40.0f, 1.3f, false)
-                                                        : rocalContrastFixed(ctx, mid, 1.4f, 100.0f, false);
+        RocalTensor col = scenario == "rrc_twist_cmn"      ? rocalColorTwistFixed(ctx, mid, 1.2f, 8.0f, 40.0f, 1.3f, false)
+                          : scenario == "rrc_contrast_cmn" ? rocalContrastFixed(ctx, mid, 1.4f, 100.0f, false)
+                                                           : rocalExposureFixed(ctx, mid, 0.4f, false);
         RocalIntParam mirror = coin;
         outs.push_back(rocalCropMirrorNormalize(ctx, col, 56, 56, 0.5f, 0.5f, mean, stdv, true, mirror, ROCAL_NCHW, ROCAL_FP16));
         mid2 = col;

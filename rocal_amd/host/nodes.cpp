@@ -649,7 +649,16 @@ void ExposureNode::create_node() {
     RMX_COLOR_CREATE(rmx_create_exposure)
 }
 
+void ExposureNode::chain_colour_refresh(const float *arrays[4]) {  // x * 2^factor = fma(x - 0, 2^factor, 0)
+    _exposure_factor.update_array();
+    _multiplier.resize(_batch_size);
+    for (size_t i = 0; i < _batch_size; i++) _multiplier[i] = exp2f(_exposure_factor.values()[i]);
+    arrays[0] = _multiplier.data();
+    arrays[1] = arrays[2] = arrays[3] = nullptr;
+}
+
 void ExposureNode::update_node() {
+    if (fused_away) return;
     _exposure_factor.update_array();
     const auto roi = roi_as_array(_inputs[0]->info().roi());
     check(rmx_update_exposure(_node, roi.data(), _exposure_factor.values().data()), "rmx_update_exposure");

@@ -313,6 +313,8 @@ class ExposureNode : public Node {
     ExposureNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
     void init(float exposure_factor);
     void init(FloatParam *exposure_factor);
+    unsigned chain_colour_kind() const override { return RMX_F_COLOR_LINEAR; }
+    void chain_colour_refresh(const float *arrays[4]) override;
 
    protected:
     void create_node() override;
@@ -320,6 +322,7 @@ class ExposureNode : public Node {
 
    private:
     ParameterVX<float> _exposure_factor;
+    std::vector<float> _multiplier;  // 2^factor per sample, for the fused chain
     static constexpr float EXPOSURE_FACTOR_RANGE[2] = {0.15f, 0.95f};
 };
 

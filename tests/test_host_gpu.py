@@ -99,7 +99,7 @@ def test_random_resized_crop_then_cmn_runs_as_one_kernel(tmp_path):
         assert np.array_equal(roi[:, 2:], crop[:, 2:])
 
 
-@pytest.mark.parametrize("scenario", ["rrc_twist_cmn", "rrc_contrast_cmn"])
+@pytest.mark.parametrize("scenario", ["rrc_twist_cmn", "rrc_contrast_cmn", "rrc_exposure_cmn"])
 def test_random_resized_crop_colour_cmn_runs_as_one_kernel(tmp_path, scenario):
     img, outs, log = _run(scenario, tmp_path, 1, [(np.float16, (N, 3, 56, 56))])
     assert "intermediate_elided 1" in log and "second_intermediate_elided 1" in log  # neither u8 tensor is materialised
@@ -113,8 +113,10 @@ def test_random_resized_crop_colour_cmn_runs_as_one_kernel(tmp_path, scenario):
     mid_roi = np.stack([np.zeros(N), np.zeros(N), mid_w, mid_h], -1).astype(np.uint32)
     if scenario == "rrc_twist_cmn":
         mid = orc.color_twist(mid, mid_roi, one(1.2), one(8.0), one(40.0), one(1.3))
-    else:
+    elif scenario == "rrc_contrast_cmn":
         mid = orc.contrast(mid, mid_roi, one(1.4), one(100.0))
+    else:
+        mid = orc.exposure(mid, mid_roi, one(0.4))
     crop = np.stack([orc.fixed_crop(int(w), int(h), 56, 56, anchor=(0.5, 0.5)) for w, h in zip(mid_w, mid_h)])
     scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
     mirrors = _coin_batches(2)
