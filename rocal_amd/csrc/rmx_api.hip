@@ -9,6 +9,7 @@
 #include <cstring>
 #include <new>
 #include <string>
+#include <limits>
 #include <vector>
 
 #include "rmx_common.h"
@@ -74,6 +75,8 @@ struct rmx_op {
 
     RmxSample *h_table[TABLE_RING] = {};  // pinned; n rows, then n source layout entries, then n side-table entries
     size_t extra_per_sample = 0;          // bytes of side table per sample (Gamma: its 256-entry table)
+    std::vector<float> lut_gamma;         // Gamma: the exponent each cached table was built for (NaN = none yet)
+    std::vector<uint8_t> lut_cache;       // Gamma: last table of every sample (256 powf per table are worth keeping)
     std::vector<RmxSrcLayout> layout;     // ragged source (empty: one padded tensor); copied behind the rows on every update
     uint64_t ragged_bytes = 0;            // extent of the ragged source buffer
     bool slot_ragged[TABLE_RING] = {};    // what the table slot was committed with
@@ -988,6 +991,10 @@ static int create_point(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, cons
     int rc = make_op(ctx, kind, src, dst, roi_type, out, kind == OP_GAMMA ? 256 : 0);
     if (rc) return rc;
     (*out)->fn = rmx::select_point_kernel(kind == OP_BLEND ? 1 : 0, dst->dtype, dst->layout, false, &(*out)->kernel_name);
+    if (kind == OP_GAMMA) {
+        (*out)->lut_gamma.assign((size_t)(*out)->n, std::numeric_limits<float>::quiet_NaN());
+        (*out)->lut_cache.assign((size_t)(*out)->n * 256, 0);
+    }
     return RMX_OK;
 }
 
@@ -1010,12 +1017,18 @@ static int update_point(rmx_op *op, const uint32_t *roi, const float *p0, const 
         s.color[0] = p0 ? p0[i] : 0.0f;
         s.color[1] = s.color[2] = s.color[3] = 0.0f;
         if (gamma) {
-            // lut[v] = u8 store (round to nearest even, saturate) of powf(v/255, gamma)*255
-            for (int v = 0; v < 256; v++) {
-                float r = rintf(powf((float)v / 255.0f, gamma[i]) * 255.0f);
-                r = !(r > 0.0f) ? 0.0f : (r > 255.0f ? 255.0f : r);  // a NaN becomes 0
-                lut[(size_t)i * 256 + v] = (uint8_t)r;
+            // lut[v] = u8 store (round to nearest even, saturate) of powf(v/255, gamma)*255; rebuilt only when the sample's
+            // exponent changed since the last update (a fixed gamma costs 256 powf per sample once, not per batch)
+            uint8_t *mine = op->lut_cache.data() + (size_t)i * 256;
+            if (!(op->lut_gamma[i] == gamma[i])) {
+                for (int v = 0; v < 256; v++) {
+                    float r = rintf(powf((float)v / 255.0f, gamma[i]) * 255.0f);
+                    r = !(r > 0.0f) ? 0.0f : (r > 255.0f ? 255.0f : r);  // a NaN becomes 0
+                    mine[v] = (uint8_t)r;
+                }
+                op->lut_gamma[i] = gamma[i];
             }
+            memcpy(lut + (size_t)i * 256, mine, 256);
         }
         bytes += (uint64_t)s.dst_w * s.dst_h * 3 * (sources + dtype_size(op->dst.dtype));
         max_rows = std::max(max_rows, (int)s.dst_h);
