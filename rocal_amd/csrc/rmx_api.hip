@@ -746,6 +746,9 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         if (ok) {
             op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &op->fast_name);
             op->fast_lds = (need_max + 15) / 16 * 16;
+            // interleaved fp32 output: room for the slab through which the lanes of a row exchange their runs before storing
+            // (64 lanes x the 24 dwords of one lane's run; the kernel takes it from the tail of the slice)
+            if (op->dst.dtype == RMX_FP32 && op->dst.layout == RMX_NHWC) op->fast_lds += 64 * 4 * 24;
             op->fast_rows = rows;
             op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
             // (default 1: a workgroup's LDS is released only when its last wavefront ends, one-wave groups keep the CU full)

@@ -17,6 +17,13 @@ namespace rmx {
 
 template <typename T, int LAYOUT, bool NORM, bool FAST>
 __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
+    // LDS slab through which the lanes of a row exchange their runs before storing (see store_packed_coalesced)
+    constexpr bool COALESCE = FAST && coalesce_pays<T, LAYOUT>();
+    uint32_t *slab = nullptr;
+    if constexpr (COALESCE) {
+        __shared__ __attribute__((aligned(16))) uint32_t slabs[4 * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>()];
+        slab = slabs + (threadIdx.x / RMX_WAVE) * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>();
+    }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + (threadIdx.x / RMX_WAVE);
@@ -120,7 +127,8 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
                         }
                         PackedGroup<T> packed;
                         pack_group<T, LAYOUT>(v, hf, packed);
-                        store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                        if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
+                        else store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
                     }
                 }
             }

@@ -25,6 +25,13 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
         __syncthreads();
     }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
+    // fp32 and interleaved fp16 outputs: the lanes of a row exchange their runs through LDS before storing (store_packed_coalesced)
+    constexpr bool COALESCE = FAST && coalesce_pays<T, LAYOUT>();
+    uint32_t *slab = nullptr;
+    if constexpr (COALESCE) {
+        __shared__ __attribute__((aligned(16))) uint32_t slabs[4 * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>()];
+        slab = slabs + (threadIdx.x / RMX_WAVE) * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>();
+    }
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
     uint32_t wave = blockIdx.x * (uint32_t)a.wpb + (threadIdx.x / RMX_WAVE);
     wave = __builtin_amdgcn_readfirstlane(wave);
@@ -117,7 +124,8 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
                         colour(v);
                         PackedGroup<T> packed;
                         pack_group_dir<T, LAYOUT, false>(v, packed);
-                        store_packed<T, LAYOUT, sizeof(T) == 1>(dimg, a.dst_h, a.dst_w, r, gx, packed);  // u8: streaming stores
+                        if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
+                        else store_packed<T, LAYOUT, sizeof(T) == 1>(dimg, a.dst_h, a.dst_w, r, gx, packed);  // u8: streaming stores
                     }
                 }
             }

@@ -22,6 +22,13 @@ template <typename T, int LAYOUT, int KIND, bool FAST>
 __global__ void __launch_bounds__(256) rmx_point_kernel(RmxKArgs a) {
     __shared__ uint32_t lut_words[4][64];  // one 256-byte table per wavefront of the workgroup
     const int lane = threadIdx.x & (RMX_WAVE - 1);
+    // fp32 and interleaved fp16 outputs: the lanes of a row exchange their runs through LDS before storing (store_packed_coalesced)
+    constexpr bool COALESCE = FAST && coalesce_pays<T, LAYOUT>();
+    uint32_t *slab = nullptr;
+    if constexpr (COALESCE) {
+        __shared__ __attribute__((aligned(16))) uint32_t slabs[4 * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>()];
+        slab = slabs + (threadIdx.x / RMX_WAVE) * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>();
+    }
     const int wib = threadIdx.x / RMX_WAVE;
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
     uint32_t wave = blockIdx.x * (uint32_t)a.wpb + (uint32_t)wib;
@@ -95,7 +102,8 @@ __global__ void __launch_bounds__(256) rmx_point_kernel(RmxKArgs a) {
                         finish(wa[i], wb[i], v);
                         PackedGroup<T> packed;
                         pack_group_dir<T, LAYOUT, false>(v, packed);
-                        store_packed<T, LAYOUT, sizeof(T) == 1>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                        if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
+                        else store_packed<T, LAYOUT, sizeof(T) == 1>(dimg, a.dst_h, a.dst_w, r, gx, packed);
                     }
                 }
             }
