@@ -142,12 +142,12 @@ def _color_common(fn, img, roi_xywh, params, flags, layout=NHWC, dtype=UINT8):
     return out
 
 
-def brightness(img, roi_xywh, alpha, beta, flags=0):
-    return _color_common(lib().orc_brightness, img, roi_xywh, [alpha, beta], flags)
+def brightness(img, roi_xywh, alpha, beta, flags=0, layout=NHWC, dtype=UINT8):
+    return _color_common(lib().orc_brightness, img, roi_xywh, [alpha, beta], flags, layout, dtype)
 
 
-def contrast(img, roi_xywh, factor, center, flags=0):
-    return _color_common(lib().orc_contrast, img, roi_xywh, [factor, center], flags)
+def contrast(img, roi_xywh, factor, center, flags=0, layout=NHWC, dtype=UINT8):
+    return _color_common(lib().orc_contrast, img, roi_xywh, [factor, center], flags, layout, dtype)
 
 
 def gamma_lut(gamma, flags=0):
@@ -184,8 +184,8 @@ def blend(img1, img2, roi_xywh, ratio, flags=0, layout=NHWC, dtype=UINT8):
     return out
 
 
-def color_twist(img, roi_xywh, alpha, beta, hue, sat, flags=0):
-    return _color_common(lib().orc_color_twist, img, roi_xywh, [alpha, beta, hue, sat], flags)
+def color_twist(img, roi_xywh, alpha, beta, hue, sat, flags=0, layout=NHWC, dtype=UINT8):
+    return _color_common(lib().orc_color_twist, img, roi_xywh, [alpha, beta, hue, sat], flags, layout, dtype)
 
 
 def warp_affine(img, roi_xywh, affine, dst_w, dst_h, out_hmax, out_wmax, interp=LINEAR, flags=0):

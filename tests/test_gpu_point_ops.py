@@ -11,7 +11,7 @@ from rocal_amd._lib import RmxError
 
 pytestmark = pytest.mark.gpu
 
-COMBOS = [(ops.NHWC, ops.UINT8), (ops.NCHW, ops.UINT8), (ops.NCHW, ops.FP16), (ops.NHWC, ops.FP32)]
+COMBOS = [(ops.NHWC, ops.UINT8), (ops.NCHW, ops.UINT8), (ops.NCHW, ops.FP16), (ops.NHWC, ops.FP32), (ops.NHWC, ops.FP16), (ops.NCHW, ops.FP32)]
 
 
 def _gpu(a):
@@ -70,6 +70,26 @@ def test_gamma_exposure_temperature_blend(ctx, layout, dtype, aligned):
     _same(got, orc.color_temperature(img, roi, adj, **kw), "colour temperature")
     got, _ = _run(ctx, ops.Blend, n, h, w, layout, dtype, lambda o: o.update(roi, ratio), [img, img2])
     _same(got, orc.blend(img, img2, roi, ratio, **kw), "blend")
+
+
+@pytest.mark.parametrize("aligned", [True, False])
+@pytest.mark.parametrize("layout,dtype", COMBOS[2:])
+def test_colour_family_float_outputs(ctx, layout, dtype, aligned):
+    """Brightness, Contrast and ColorTwist writing fp16 / fp32 tensors in both layouts (the coalescing stores of the aligned kernels)."""
+    n, h, w = 5, 29, 104 if aligned else 99
+    img, _, roi = _batch(21 + int(aligned), n, h, w, aligned)
+    rng = np.random.default_rng(5)
+    f = lambda lo, hi: rng.uniform(lo, hi, n).astype(np.float32)
+    kw = dict(layout=layout, dtype=dtype)
+    p = (f(0.3, 2.0), f(-40, 40))
+    got, _ = _run(ctx, ops.Brightness, n, h, w, layout, dtype, lambda o: o.update(roi, *p), [img])
+    _same(got, orc.brightness(img, roi, *p, **kw), "brightness")
+    p = (f(0.3, 2.5), f(0, 255))
+    got, _ = _run(ctx, ops.Contrast, n, h, w, layout, dtype, lambda o: o.update(roi, *p), [img])
+    _same(got, orc.contrast(img, roi, *p, **kw), "contrast")
+    p = (f(0.5, 1.8), f(-30, 30), f(-180, 180), f(0.0, 2.0))
+    got, _ = _run(ctx, ops.ColorTwist, n, h, w, layout, dtype, lambda o: o.update(roi, *p), [img])
+    _same(got, orc.color_twist(img, roi, *p, **kw), "colour twist")
 
 
 def test_full_size_u8_batches(ctx):
