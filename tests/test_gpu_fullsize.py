@@ -15,11 +15,11 @@ def _bits(a):
     return a.view(np.uint8)
 
 
-@pytest.mark.parametrize("cfg", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("cfg", sorted(bench.WORKLOADS))
 def test_full_size_configuration_is_bit_identical_to_the_oracle(ctx, cfg):
     op, src, dst, n, cpu = bench.build_case(cfg, ctx)
     dst.zero_()
-    op.launch(src, dst)
+    op.launch(*(src if isinstance(src, tuple) else (src,)), dst)
     ctx.sync()
     got = dst.cpu().numpy()
     exp = cpu(n)
@@ -254,3 +254,27 @@ def test_launches_can_be_captured_in_a_graph_and_replayed(ctx):
         exp_mid = orc.color_twist(orc.resize(img, roi, dw, dh, 48, 64, interp=orc.LINEAR), mid_roi, one(1.1), one(4.0), one(25.0), one(1.3))
         assert np.array_equal(got, o2.cpu().numpy()), "replay %d differs from the eager chain" % rep
         assert np.array_equal(got, exp_mid[:, :, ::-1]), "replay %d differs from the oracle" % rep
+
+
+@pytest.mark.parametrize("layout,dtype", [(ops.NHWC, ops.FP32), (ops.NCHW, ops.FP32), (ops.NHWC, ops.FP16)])
+def test_large_windows_in_narrow_tiles_every_float_format(ctx, layout, dtype):
+    """RandomResizedCrop + CropMirrorNormalize from windows of up to 640 x 640 pixels: the aligned kernel narrows its x-tiles
+    until a strip's window fits its LDS slice, so a row is written by several tiles; with mirrors, in every float format
+    (interleaved fp32 goes through the coalescing stores)."""
+    import torch
+    n = 16
+    c = wl.config1(n)
+    c["roi"][0] = (0, 0, c["W"][0], c["H"][0])  # a whole image
+    inv = (1 / wl.STD).astype(np.float32)
+    scale, bias = np.tile(inv, n), np.tile(-(wl.MEAN * inv), n)
+    dw = np.full(n, 224, np.uint32)
+    op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, layout, dtype), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+    op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
+    assert op.kernel_name == "rmx_resize_fast_kernel"
+    out = op.alloc_output()
+    op.launch(torch.from_numpy(c["img"]).cuda(), out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    exp = orc.resize(c["img"], c["roi"], dw, dw, 224, 224, interp=orc.LINEAR, mirror=c["mirror"], scale=scale, bias=bias,
+                     layout=layout, dtype=dtype, flags=orc.F_QUANTIZE_U8)
+    assert np.array_equal(got.view(np.uint8), exp.view(np.uint8)), "%d values differ (%s)" % (int((got != exp).sum()), op.plan)

@@ -153,3 +153,30 @@ def test_two_source_protocol_errors(ctx):
     with pytest.raises(RmxError, match="not a Gamma"):
         bright._update("rmx_update_gamma", (roi, np.uint32), (np.ones(n, np.float32), np.float32))
     ctx.sync()
+
+
+@pytest.mark.parametrize("layout,dtype", [(ops.NCHW, ops.FP32), (ops.NHWC, ops.FP32), (ops.NHWC, ops.FP16), (ops.NHWC, ops.UINT8)])
+def test_wide_rows_take_several_tiles(ctx, layout, dtype):
+    """Rows wider than one wavefront tile (512 columns): the second tile is narrower than the first and its lanes exchange
+    their runs in groups of another size. CropMirrorNormalize with mirrors, Brightness and Gamma on 1160 / 648 columns."""
+    n, h, w = 3, 9, 1160
+    rng = np.random.default_rng(77)
+    img = rng.integers(0, 256, (n, h, w, 3), dtype=np.uint8)
+    crop = np.array([[0, 0, 1160, 9], [8, 1, 648, 7], [3, 0, 1096, 9]], np.uint32)
+    mirror = np.array([1, 0, 1], np.uint32)
+    scale = rng.uniform(0.005, 0.03, n * 3).astype(np.float32)
+    bias = rng.uniform(-2.5, 0.5, n * 3).astype(np.float32)
+    if dtype == ops.UINT8:
+        scale[:], bias[:] = 1.0, 0.0
+    op = ops.CropMirrorNormalize(ctx, ops.desc(n, h, w, ops.NHWC, ops.UINT8), ops.desc(n, h, w, layout, dtype))
+    op.update(crop, scale, bias, mirror)
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    ctx.sync()
+    _same(out.cpu().numpy(), orc.crop_mirror_normalize(img, crop, scale, bias, mirror, h, w, layout, dtype), "cmn")
+    a, b = rng.uniform(0.3, 2.0, n).astype(np.float32), rng.uniform(-40, 40, n).astype(np.float32)
+    got, _ = _run(ctx, ops.Brightness, n, h, w, layout, dtype, lambda o: o.update(crop, a, b), [img])
+    _same(got, orc.brightness(img, crop, a, b, layout=layout, dtype=dtype), "brightness")
+    g = rng.uniform(0.3, 7.0, n).astype(np.float32)
+    got, _ = _run(ctx, ops.Gamma, n, h, w, layout, dtype, lambda o: o.update(crop, g), [img])
+    _same(got, orc.gamma(img, crop, g, layout=layout, dtype=dtype), "gamma")
