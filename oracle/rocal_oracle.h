@@ -33,10 +33,18 @@
  *   orc_gamma/exposure/color_temperature/blend
  *                              PARITY UNPINNED against RPP; closed forms tested (gamma 1 and 2, 2^k
  *                              exposure, saturating +-adj, ratio 0 / 1 / 0.5).
- *   orc_color_twist/hue/sat    PARITY UNPINNED: HSV details live only in RPP. Invariants tested
- *                              (identity, grey fixed points, 360-periodicity, colorsys cross-check).
- *   orc_warp_affine            PARITY UNPINNED for matrix element order / centre convention;
- *                              closed forms tested (identity, integer translation, 90-degree turns).
+ *   orc_resize (nearest)       law DEFINED here (floor of the half-pixel-centre coordinate + 0.5); the restatement is
+ *                              checked against hand-written indices (identity, 2x / 3x down, 2x / 3x replication, ROI and
+ *                              mirror); against RPP it is parity unpinned.
+ *   orc_color_twist/hue/sat    restatement checked on all 2^24 RGB triples against the same HSV round trip written
+ *                              with true divisions in numpy (5 parameter sets: at most one level apart, < 0.3 % of
+ *                              values differ), identity, grey fixed points, 360-periodicity, colorsys. Against RPP the
+ *                              HSV formulation is PARITY UNPINNED (it lives only in RPP).
+ *   orc_warp_affine            restatement checked by exact dyadic blends of fractional translations (weight order,
+ *                              neighbours, far-edge clamp), the out-of-ROI rule at floor == lo-1 / hi / hi+1, a float64
+ *                              brute force for rotation+scale+shift with an off-origin ROI and another destination
+ *                              size, and torch grid_sample in the interior. Matrix element order and centre
+ *                              convention are PARITY UNPINNED against RPP.
  *   orc_rotate                 direction/centre pinned by rocAL/source/meta_data/meta_node_rotate.cpp:53-77;
  *                              fp path from angle to matrix PARITY UNPINNED.
  *   parameter laws (orc_mt19937*, orc_seed_seq, orc_uniform_rand*, orc_custom_rand,
