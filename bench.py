@@ -5,6 +5,17 @@ A step is one pass of the hot path over one batch: the launch that replaces vxPr
 the fused node (what rocAL's own process timer brackets). Inputs and the per-batch parameter
 table are resident in HBM when the timed region starts. Prints ONE JSON line on stdout.
 
+Every step reads a source batch and writes a destination batch that no earlier step of the last
+gigabyte has touched: the timed loop rotates over K copies of the batch with K x (bytes per step)
+>= 1 GiB, four times the 256 MB last-level cache, as a pipeline that gets a fresh batch per step
+would. `value`, `ms_per_step` and `roofline.frac` are from that loop; `roofline.frac_warm` is the
+same kernel replayed on ONE source/destination pair (which fits the cache) and is reported for
+comparison only. Before anything is timed an untimed ramp of launches brings the GPU to its steady
+clocks (config.clock_ramp_ms). config.update_ms_per_batch is the host time of the per-batch update
+(parameter packing, launch planning, table upload) on fresh parameters, config.step_with_update_ms
+one update + launch + wait per batch, as rocAL's output thread runs them
+(rocAL/source/pipeline/master_graph.cpp:1010-1017).
+
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 0..11] [--all] [--no-cpu]
 """
 import argparse
@@ -38,8 +49,9 @@ WORKLOADS = {
 
 
 def build_case(cfg, ctx, n=None):
-    """Returns (op, src_tensor, dst_tensor, n_images, cpu_fn) for a configuration; cpu_fn(k) runs the
-    CPU checker on the first k images of the same batch."""
+    """Returns (op, src_tensor, dst_tensor, n_images, cpu_fn, update_fn) for a configuration; cpu_fn(k) runs the
+    CPU checker on the first k images of the same batch; update_fn(j) runs the op's per-batch update with the
+    j-th fresh parameter set (j = 0: the set the timed launches use), or is None."""
     import torch
     from rocal_amd import ops, workloads as wl
 
@@ -52,7 +64,9 @@ def build_case(cfg, ctx, n=None):
         c = wl.config0(n)
         scale, bias = scale_bias(n)
         op = ops.CropMirrorNormalize(ctx, ops.desc(n, 256, 256, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP32))
-        op.update(c["crop"], scale, bias, c["mirror"])
+        def update(j):
+            op.update(c["crop"], scale, bias, np.roll(c["mirror"], j))
+        update(0)
 
         def cpu(k):
             from oracle import orc
@@ -63,7 +77,14 @@ def build_case(cfg, ctx, n=None):
         scale, bias = scale_bias(n)
         dw = np.full(n, 224, np.uint32)
         op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
-        op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
+        def update(j):  # j > 0: a fresh set of RandomResizedCrop windows and mirror flags for the same images
+            if j == 0:
+                op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
+            else:
+                rng = np.random.default_rng(99000 + j)
+                roi = np.array([wl.rrc_window(rng, int(c["H"][i]), int(c["W"][i])) for i in range(n)], np.uint32)
+                op.update_cmn(roi, dw, dw, scale, bias, (rng.random(n) < 0.5).astype(np.uint32))
+        update(0)
 
         def cpu(k):
             from oracle import orc
@@ -74,7 +95,9 @@ def build_case(cfg, ctx, n=None):
         c = wl.config2(n)
         sd = ops.desc(n, 224, 224, ops.NHWC, ops.UINT8)
         op = ops.ColorTwist(ctx, sd, sd)
-        op.update(c["roi"], c["alpha"], c["beta"], c["hue"], c["sat"])
+        def update(j):
+            op.update(c["roi"], np.roll(c["alpha"], j), np.roll(c["beta"], j), np.roll(c["hue"], j), np.roll(c["sat"], j))
+        update(0)
 
         def cpu(k):
             from oracle import orc
@@ -85,7 +108,9 @@ def build_case(cfg, ctx, n=None):
         sd = ops.desc(n, 512, 512, ops.NHWC, ops.UINT8)
         dw = np.full(n, 512, np.uint32)
         op = ops.WarpAffine(ctx, sd, sd, ops.LINEAR)
-        op.update(c["roi"], c["affine"], dw, dw)
+        def update(j):
+            op.update(c["roi"], np.roll(c["affine"], j, axis=0), dw, dw)
+        update(0)
 
         def cpu(k):
             from oracle import orc
@@ -97,7 +122,9 @@ def build_case(cfg, ctx, n=None):
         dw = np.full(n, 640, np.uint32)
         dh = np.full(n, 360, np.uint32)
         op = ops.Resize(ctx, ops.desc(n, 1080, 1920, ops.NHWC, ops.UINT8), ops.desc(n, 360, 640, ops.NCHW, ops.FP16), ops.TRIANGULAR)
-        op.update(c["roi"], dw, dh, c["mirror"], np.tile(wl.MEAN, n), np.tile(wl.STD, n))
+        def update(j):
+            op.update(c["roi"], dw, dh, np.roll(c["mirror"], j), np.tile(wl.MEAN, n), np.tile(wl.STD, n))
+        update(0)
         scale, bias = scale_bias(n)
 
         def cpu(k):
@@ -189,30 +216,98 @@ def build_case(cfg, ctx, n=None):
             return orc.color_temperature(img[:k], roi[:k], p[:k])
         if cfg == 8:
             dst = op.alloc_output()
-            return op, (torch.from_numpy(img).cuda(), torch.from_numpy(img2).cuda()), dst, n, cpu
+            return op, (torch.from_numpy(img).cuda(), torch.from_numpy(img2).cuda()), dst, n, cpu, None
     else:
         raise SystemExit("unknown config %r" % cfg)
     src = torch.from_numpy(c["img"]).cuda()
     dst = op.alloc_output()
-    return op, src, dst, n, cpu
+    return op, src, dst, n, cpu, (update if cfg in (0, 1, 2, 3, 4) else None)
 
 
-def time_launches(op, src, dst, steps, warmup):
-    """K launches between two HIP events recorded on the stream the kernel runs on."""
+ROTATE_BYTES = 1 << 30   # the timed loop touches at least this much memory before it comes back to a buffer
+RAMP_MS = 120.0          # untimed launches before anything is timed: the GPU reaches its steady clocks in ~35 ms
+
+
+def _launcher(op, srcs, dst):
+    if len(srcs) == 1:
+        return op.prepared_launch(srcs[0], dst)
+    return lambda: op.launch(*srcs, dst)
+
+
+def clock_ramp(launchers, min_ms=RAMP_MS):
+    """Untimed launches (cycling through the buffer pairs) for at least min_ms of wall time; returns (launches, ms)."""
     import torch
-    srcs = src if isinstance(src, tuple) else (src,)
-    for _ in range(warmup):
-        op.launch(*srcs, dst)
+    t0 = time.perf_counter()
+    count = 0
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        for _ in range(200):
+            launchers[count % len(launchers)]()
+            count += 1
+        torch.cuda.synchronize()
+    return count, (time.perf_counter() - t0) * 1e3
+
+
+def time_loop(launchers, steps, warmup):
+    """`steps` launches, cycling through `launchers`, between two HIP events recorded on the stream the kernels run
+    on (the context borrows torch's current stream). Returns (ms per launch on the device, ms per step by the host clock)."""
+    import torch
+    k = len(launchers)
+    for i in range(warmup):
+        launchers[i % k]()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(steps):
-        op.launch(*srcs, dst)
+    for i in range(steps):
+        launchers[i % k]()
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return e0.elapsed_time(e1) / steps, wall * 1e3 / steps  # ms per launch (device), ms per step (host clock)
+    return e0.elapsed_time(e1) / steps, wall * 1e3 / steps
+
+
+def time_updates(op, update_fn, launchers, steps, sets=12):
+    """Host cost of the per-batch update on fresh parameters, and of whole steps that include it."""
+    import torch
+    calls = []
+    for j in range(1, sets + 1):
+        update_fn(j)
+        calls.append(op.prepared_update())
+    update_fn(0)
+    calls.append(op.prepared_update())  # the last one restores the parameters of the timed launches
+    torch.cuda.synchronize()
+    # (a) the update alone: packs, plans, starts the table upload; nothing waits for the GPU
+    t = []
+    for rep in range(5):
+        for c in calls:
+            t0 = time.perf_counter()
+            c()
+            t.append(time.perf_counter() - t0)
+        torch.cuda.synchronize()
+    update_ms = float(np.median(t)) * 1e3
+    # (b) update -> launch -> wait, one batch at a time, as rocAL's output thread runs them
+    k, m = len(launchers), len(calls)
+    nsteps = max(steps, 200)
+    for i in range(20):
+        calls[i % m]()
+        launchers[i % k]()
+        torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(nsteps):
+        calls[i % m]()
+        launchers[i % k]()
+        torch.cuda.synchronize()
+    serial_ms = (time.perf_counter() - t0) * 1e3 / nsteps
+    # (c) the same without waiting per batch: the 4-slot table ring lets the host run ahead of the GPU
+    t0 = time.perf_counter()
+    for i in range(nsteps):
+        calls[i % m]()
+        launchers[i % k]()
+    torch.cuda.synchronize()
+    piped_ms = (time.perf_counter() - t0) * 1e3 / nsteps
+    calls[-1]()
+    torch.cuda.synchronize()
+    return update_ms, serial_ms, piped_ms
 
 
 def copy_ceiling(ctx, nbytes=1 << 30, reps=20):
@@ -267,24 +362,47 @@ def measured_traffic(cfg, kernel):
     return rec["fetch_bytes"] + rec["write_bytes"]
 
 
-def run_config(cfg, ctx, steps, warmup, with_cpu):
+def run_config(cfg, ctx, steps, warmup, with_cpu, rotating_only=False):
     import torch
-    op, src, dst, n, cpu_fn = build_case(cfg, ctx)
-    ms_kernel, ms_step = time_launches(op, src, dst, steps, warmup)
+    op, src, dst, n, cpu_fn, update_fn = build_case(cfg, ctx)
+    srcs = src if isinstance(src, tuple) else (src,)
     algo = op.algorithmic_bytes
+    # K source/destination pairs at different addresses: K x (bytes a step touches) >= 1 GiB
+    copies = max(2, -(-ROTATE_BYTES // max(algo, 1)))
+    pairs = [(srcs, dst)] + [(tuple(t.clone() for t in srcs), torch.empty_like(dst)) for _ in range(copies - 1)]
+    launchers = [_launcher(op, sp, d) for sp, d in pairs]
+    ramp_launches, ramp_ms = clock_ramp(launchers)
+    ms_kernel, ms_step = time_loop(launchers, steps, warmup)          # rotating: the reported figure
+    ms_warm = ms_kernel
+    if not rotating_only:
+        ms_warm, _ = time_loop(launchers[:1], steps, warmup)          # one pair, cache-resident: for comparison
     achieved = algo / (ms_kernel * 1e-3) / 1e9
+    warm = algo / (ms_warm * 1e-3) / 1e9
     out = {
         "metric": "images/s", "value": round(n / (ms_kernel * 1e-3), 1), "unit": "images/s", "n_gpus": 1, "steps": steps,
         "warmup": warmup, "ms_per_step": round(ms_kernel, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": WORKLOADS[cfg], "batch": n, "kernel": op.kernel_name, "algorithmic_bytes_per_launch": algo, "plan": op.plan,
-                   "host_ms_per_step": round(ms_step, 6)},
+                   "host_ms_per_step": round(ms_step, 6), "rotating_buffer_pairs": copies,
+                   "clock_ramp_ms": round(ramp_ms, 1), "clock_ramp_launches": ramp_launches,
+                   "ms_per_step_warm": round(ms_warm, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(cfg, op.kernel_name)},
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": measured_traffic(cfg, op.kernel_name),
+                     "achieved_warm": round(warm, 1), "frac_warm": round(warm / HBM_PEAK_GBPS, 4)},
     }
+    if rotating_only:
+        for k in ("ms_per_step_warm",):
+            out["config"].pop(k)
+        for k in ("achieved_warm", "frac_warm"):
+            out["roofline"].pop(k)
+    if update_fn is not None and not rotating_only:
+        upd, serial, piped = time_updates(op, update_fn, launchers, steps)
+        out["config"]["update_ms_per_batch"] = round(upd, 6)
+        out["config"]["step_with_update_ms"] = round(serial, 6)
+        out["config"]["step_with_update_pipelined_ms"] = round(piped, 6)
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline(cpu_fn, n)
-    del op, src, dst
+    del op, src, dst, srcs, pairs, launchers
     torch.cuda.empty_cache()
     return out
 
@@ -293,14 +411,15 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     # After an idle spell (building the synthetic batch takes seconds of host time) the GPU needs about a thousand
-    # launches (~35 ms) to reach its steady clocks: the first 200 launches of configuration 1 average 44 us, the
-    # next 200 34 us, from the sixth chunk on 31.3 us. The default warm-up covers that; the timed region is long
-    # enough for the profiler's average over all launches to agree with it.
+    # launches (~35 ms) to reach its steady clocks; an untimed ramp of launches (clock_ramp) covers that whatever
+    # --warmup says. The default timed region is long enough for the profiler's average over all launches to agree.
     ap.add_argument("--steps", type=int, default=6000)
-    ap.add_argument("--warmup", type=int, default=1500)
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", type=int, default=1)
     ap.add_argument("--all", action="store_true", help="also measure the other configurations (one JSON object per configuration, written to bench_all.json in the output folder)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--rotating-only", action="store_true", help="only the ramp and the rotating timed loop: every launch of the process is of the "
+                    "reported kind, so a rocprofv3 kernel summary of this command averages the same thing")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build measures ONE GPU (the path shards trivially by sample; no multi-GPU figure is produced). "
@@ -311,7 +430,7 @@ def main():
     from rocal_amd import ops
     ctx = ops.Context(0)
     ceiling = copy_ceiling(ctx)
-    res = run_config(args.config, ctx, args.steps, args.warmup, not args.no_cpu)
+    res = run_config(args.config, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only)
     res["metric"] = "images/s + HBM GB/s (% peak), RandomResizedCrop+CMN 224^2 fp16, batch 256" if args.config == 1 else "images/s"
     res["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
     res["roofline"]["frac_of_copy_ceiling"] = round(res["roofline"]["achieved"] / ceiling, 4)
@@ -319,7 +438,7 @@ def main():
         allres = {args.config: res}
         for cfg in sorted(WORKLOADS):
             if cfg != args.config:
-                allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu)
+                allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only)
                 allres[cfg]["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
                 print("config %d: %s" % (cfg, json.dumps(allres[cfg])), file=sys.stderr)
         os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)

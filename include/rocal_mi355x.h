@@ -55,7 +55,12 @@ enum {
      * RMX_F_QUANTIZE_U8): reproduces the three-node graph resize(u8) -> colour(u8) -> CropMirrorNormalize in one pass,
      * the colour node's rounded, saturated u8 output included. Parameters come with rmx_update_resize_color_cmn. */
     RMX_F_COLOR_LINEAR = 1u << 1, /* Brightness / Contrast / Exposure: fma(x - c2, c0, c1) */
-    RMX_F_COLOR_TWIST = 1u << 2   /* ColorTwist / Hue / Saturation: c0 alpha, c1 beta, c2 hue in degrees, c3 saturation */
+    RMX_F_COLOR_TWIST = 1u << 2,  /* ColorTwist / Hue / Saturation: c0 alpha, c1 beta, c2 hue in degrees, c3 saturation */
+    /* Bilinear edge rule of the reference's device code (rocAL/rocAL_hip/rocal_hip_kernels.cpp:340-343,356-361): BOTH
+     * neighbours of a tap are clamped to [lo, hi-1], so the window's last column and row are never sampled; ratio, offsets
+     * and weights still come from the full window length. Without the flag the neighbours clamp to [lo, hi] (the textbook
+     * half-pixel-centre form, which torch.nn.functional.interpolate also computes). */
+    RMX_F_EDGE_REF = 1u << 3
 };
 
 /* TensorInfo of one side of a node (rocAL/include/pipeline/tensor.h:65-309): padded maxima. */

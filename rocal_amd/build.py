@@ -19,8 +19,14 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Wno-unknown-cuda-version"]
 
 
-def _compile(src):
+def _newest_header():
+    return max(os.path.getmtime(h) for h in glob.glob(os.path.join(CSRC, "*.h")) + [os.path.join(HERE, "..", "include", "rocal_mi355x.h")])
+
+
+def _compile(src, incremental=False):
     obj = os.path.join(OBJDIR, os.path.basename(src) + ".o")
+    if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _newest_header()):
+        return obj, ""
     cmd = [HIPCC] + FLAGS + os.environ.get("RMX_EXTRA_FLAGS", "").split() + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature name: that warning is expected
@@ -30,11 +36,16 @@ def _compile(src):
     return obj, err
 
 
-def build(verbose=False):
+def build(verbose=False, incremental=False):
+    """Compiles every source (incremental=True: only those older than their object or than a header)."""
     os.makedirs(OBJDIR, exist_ok=True)
     srcs = sorted(glob.glob(os.path.join(CSRC, "*.hip")))
+    # objects of sources that no longer exist must not be linked
+    for o in glob.glob(os.path.join(OBJDIR, "*.o")):
+        if os.path.join(CSRC, os.path.basename(o)[:-2]) not in srcs:
+            os.remove(o)
     with cf.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        results = list(ex.map(_compile, srcs))
+        results = list(ex.map(lambda s: _compile(s, incremental), srcs))
     objs = [o for o, _ in results]
     if verbose:
         for _, e in results:
@@ -46,4 +57,4 @@ def build(verbose=False):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, incremental="--incremental" in sys.argv))

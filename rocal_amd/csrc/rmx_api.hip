@@ -54,7 +54,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -93,8 +93,11 @@ struct rmx_op {
     int strips = 1, strip_rows = 1, tile_w = 512, lds_per_wave = 0, waves_per_block = 4;
     int aux0 = 0, aux1 = 0;
     int fast_lds = 0, fast_strips = 1, fast_rows = 8, fast_wpb = 1;  // plan of fn_fast
+    int fast_aux1 = 0;                                               // aux1 of fn_fast
     bool fast_needs_src16 = false;                                   // fn_fast also wants a 16-byte aligned source base
     uint64_t algo_bytes = 0;
+    rmx::KernelFn lds_fn[2] = {};  // kernels whose static LDS size has been asked of the runtime ([0] general, [1] fast)
+    int lds_static[2] = {};
 };
 
 namespace {
@@ -246,6 +249,8 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->fast_rows = tune_env("RMX_TUNE_FAST_ROWS", ctx->fast_rows, 1, 64);
         ctx->fast_lds = tune_env("RMX_TUNE_FAST_LDS", ctx->fast_lds, 2048, 48 * 1024);
         ctx->fast_wpb = tune_env("RMX_TUNE_FAST_WPB", ctx->fast_wpb, 1, 4);
+        ctx->dma = tune_env("RMX_TUNE_DMA", ctx->dma, 0, 1);  // 0: the bilinear fast path always stages through registers
+        ctx->dma_lds = tune_env("RMX_TUNE_DMA_LDS", ctx->dma_lds, 2048, 10 * 1024) & ~15;  // LDS window of a wavefront
         ctx->tri_wpb = tune_env("RMX_TUNE_TRI_WPB", ctx->tri_wpb, 1, 4);
         ctx->warp_passes = tune_env("RMX_TUNE_WARP_PASSES", ctx->warp_passes, 1, 8);
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
@@ -301,6 +306,22 @@ const char *rmx_op_plan(const rmx_op *op) {
 }
 const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : op->kernel_name) : ""; }
 
+// static LDS of a kernel (bytes), asked of the runtime once per op and kernel; -1 (with the error set) when the query fails
+static int static_lds_of(rmx_op *op, rmx::KernelFn fn) {
+    for (int i = 0; i < 2; i++)
+        if (op->lds_fn[i] == fn) return op->lds_static[i];
+    hipFuncAttributes attr;
+    hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(fn));
+    if (e != hipSuccess) {
+        fail(RMX_ERR_HIP, "hipFuncGetAttributes failed: %d (%s)", (int)e, hipGetErrorString(e));
+        return -1;
+    }
+    const int slot = (fn == op->fn_fast) ? 1 : 0;
+    op->lds_fn[slot] = fn;
+    op->lds_static[slot] = (int)attr.sharedSizeBytes;
+    return op->lds_static[slot];
+}
+
 static int launch_impl(rmx_op *op, const void *src, const void *src2, void *dst) {
     if (!src || !dst) return fail(RMX_ERR_INVALID, "source/destination buffer is NULL");
     if (op->cur < 0 || !op->fn) return fail(RMX_ERR_INVALID, "op launched before its first update");
@@ -330,15 +351,22 @@ static int launch_impl(rmx_op *op, const void *src, const void *src2, void *dst)
         a.strips = op->fast_strips;
         a.lds_bytes = op->fast_lds;
         a.aux0 = op->fast_rows;
+        a.aux1 = op->fast_aux1;
         wpb = op->fast_wpb;
     }
+    HIP_TRY(hipSetDevice(op->ctx->device));
+    rmx::KernelFn fn = fast ? op->fn_fast : op->fn;
+    // a workgroup's LDS = the wavefronts' dynamic slices + what the kernel declares statically (coalescing slabs, colour
+    // tables): fewer wavefronts per workgroup when the sum would not fit
+    const int static_lds = static_lds_of(op, fn);
+    if (static_lds < 0) return RMX_ERR_HIP;
+    while (wpb > 1 && (size_t)a.lds_bytes * wpb + (size_t)static_lds > (size_t)op->ctx->max_lds_per_block) wpb--;
+    const size_t lds = (size_t)a.lds_bytes * wpb;
+    if (lds + (size_t)static_lds > (size_t)op->ctx->max_lds_per_block)
+        return fail(RMX_ERR_INVALID, "plan needs %zu + %d bytes of LDS per workgroup (limit %d)", lds, static_lds, op->ctx->max_lds_per_block);
     const uint64_t waves = (uint64_t)op->n * (uint64_t)a.strips;
     const uint64_t blocks = (waves + wpb - 1) / wpb;
     if (blocks == 0 || blocks > 0x7fffffffull) return fail(RMX_ERR_INVALID, "grid of %llu workgroups is out of range", (unsigned long long)blocks);
-    const size_t lds = (size_t)a.lds_bytes * wpb;
-    if (lds > (size_t)op->ctx->max_lds_per_block) return fail(RMX_ERR_INVALID, "plan needs %zu bytes of LDS per workgroup (limit %d)", lds, op->ctx->max_lds_per_block);
-    HIP_TRY(hipSetDevice(op->ctx->device));
-    rmx::KernelFn fn = fast ? op->fn_fast : op->fn;
     a.wpb = wpb;
     a.nblocks = (uint32_t)blocks;
     hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
@@ -513,6 +541,18 @@ static inline float src_coord_h(int u, float ratio, float off, float lo) {
     return s;
 }
 
+// Upper bound of floor(c(u + d)) - floor(c(u)) for the kernels' coordinate law c(u) = u*ratio + off + lo evaluated in
+// fp32: the exact coordinates lie d*ratio apart, and each computed one carries three roundings of at most half an ulp
+// at a magnitude below `mag` (8 ulps of slack cover both ends). Used to size LDS windows without walking the rows.
+static inline int span_bound(int d, float ratio, float mag) {
+    if (d <= 0) return 1;
+    return (int)std::floor((double)d * (double)ratio + 8.0 * 5.9604645e-8 * (double)mag) + 1;
+}
+
+// Static LDS the resize kernels hold besides their dynamic slices (the colour tables of a fused twist stage); the
+// planners keep this much of a workgroup's LDS free.
+constexpr int kStaticLdsMax = 2048;
+
 static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     const bool quant = (op->flags & RMX_F_QUANTIZE_U8) != 0;
     const int chain = (op->flags & RMX_F_COLOR_LINEAR) ? 1 : (op->flags & RMX_F_COLOR_TWIST) ? 2 : 0;
@@ -570,7 +610,17 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 raw = raw + (float)ylo;
                 return (int)std::ceil(raw);
             };
-            for (int r = 0; r + 4 < s.dst_h && down; r++) {
+            if (s.dst_h <= 4) continue;
+            // Interior rows: the first taps of rows four apart lie at least floor(4*ry - rounding slack) source rows
+            // apart, which must reach past the ksz taps of the upper row. At the window's ends the clamp can fold two
+            // rows onto the same source row: that happens exactly when row 4 starts at or above the first source row,
+            // or the last-but-four row's taps reach the last one (first taps are monotone in the row index).
+            const double slack = 8.0 * 5.9604645e-8 * (double)(s.src_y + s.src_h + 2);
+            if ((int)std::floor(4.0 * (double)s.ry - slack) >= ksz) {
+                down = loc_of(4) > ylo && loc_of(s.dst_h - 5) + ksz - 1 < yhi;
+                continue;
+            }
+            for (int r = 0; r + 4 < s.dst_h && down; r++) {  // ratios just above 1: walk the rows
                 const int last = std::max(std::min(loc_of(r) + ksz - 1, yhi), ylo);
                 const int first = std::max(std::min(loc_of(r + 4), yhi), ylo);
                 down = first > last;
@@ -633,10 +683,12 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                  ? rmx::select_resize_nearest_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &nm)
                  : rmx::select_resize_linear_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &nm);
     op->kernel_name = nm;
-    // x-tile: up to 64 lanes x 8 px. Each wave keeps a ring of R staged source rows in LDS;
-    // R and the row pitch are computed per sample with the kernel's own float formulas.
+    // Both plans below size LDS from closed-form bounds (span_bound), a handful of operations per sample: the update
+    // runs once per batch on the thread that also launches, and must not cost more than the kernel it plans.
+    // General kernel: x-tile of up to 64 lanes x 8 px; each wave keeps a ring of R staged source rows in LDS.
     int tile_w = std::min(((max_dw + 7) / 8) * 8, 512);
     const int budget = 16 * 1024;
+    const int grows = op->ctx->gen_rows;
     int lds = 0;
     for (;;) {
         lds = 0;
@@ -646,91 +698,55 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 s.strip_rows = 1;
                 continue;
             }
-            const float offx = (s.rx - 1.0f) * 0.5f, offy = (s.ry - 1.0f) * 0.5f;
-            const int xlo = s.src_x, xhi = s.src_x + s.src_w - 1;
-            int ring = 1, pitch_max = 0, maxnew = 0;
-            for (int xt = 0; xt < s.dst_w; xt += tile_w) {
-                const int tw = std::min<int>(s.dst_w - xt, tile_w);
-                const int L = (tw + 7) / 8, G = 64 / L;
-                const int ixmin = (int)std::floor(src_coord_h(s.pc_x + xt, s.rx, offx, (float)xlo));
-                const int ixmax = (int)std::floor(src_coord_h(s.pc_x + xt + tw - 1, s.rx, offx, (float)xlo));
-                const int cs = std::max(std::min(ixmin, xhi), xlo), ce = std::max(std::min(ixmax + 1, xhi), xlo);
-                const int items = (ce - cs + 1 + 3) >> 2;
-                pitch_max = std::max(pitch_max, 4 + items * 4 + 4);
-                if (xt == 0 || tw != tile_w) {  // G only changes on the last, narrower tile
-                    for (int r = 0; r < s.dst_h; r++) {
-                        const int re = std::min(r + G - 1, s.dst_h - 1);
-                        const int a_k = (int)std::floor(src_coord_h(s.pc_y + r, s.ry, offy, (float)s.src_y));
-                        const int b_k = (int)std::floor(src_coord_h(s.pc_y + re, s.ry, offy, (float)s.src_y)) + 1;
-                        ring = std::max(ring, b_k - a_k + 1);
-                        if (r + G < s.dst_h) {  // rows that enter the window when the step after this one is staged
-                            const int rn = std::min(r + 2 * G - 1, s.dst_h - 1);
-                            const int a_n = (int)std::floor(src_coord_h(s.pc_y + r + G, s.ry, offy, (float)s.src_y));
-                            const int b_n = (int)std::floor(src_coord_h(s.pc_y + rn, s.ry, offy, (float)s.src_y)) + 1;
-                            maxnew = std::max(maxnew, b_n - std::max(b_k + 1, a_n) + 1);
-                        }
-                    }
-                }
-            }
+            // the last (narrowest) tile has the most rows per step: G = 64 / lanes per row
+            const int tw_last = s.dst_w - ((s.dst_w - 1) / tile_w) * tile_w;
+            const int G = 64 / ((tw_last + 7) / 8);
+            const float magx = (float)(s.src_x + s.src_w + 2), magy = (float)(s.src_y + s.src_h + 2);
+            const int ring = std::min<int>(s.src_h + 2, span_bound(std::min(std::min(G, grows), (int)s.dst_h) - 1, s.ry, magy) + 2);
+            const int nc = std::min<int>(s.src_w, span_bound(std::min<int>(tile_w, s.dst_w) - 1, s.rx, magx) + 2);
+            const int pitch = 4 + ((nc + 3) >> 2) * 4 + 4;
             s.strip_rows = ring;
-            s.flags = (s.flags & 0xffffu) | ((uint32_t)std::min(maxnew, 0xffff) << 16);
-            lds = std::max(lds, ring * pitch_max * 4);
+            lds = std::max(lds, ring * pitch * 4);
         }
         if (lds <= budget || tile_w <= 64) break;
         tile_w = std::max(64, (tile_w / 2 + 7) / 8 * 8);
     }
     op->lds_per_wave = (lds + 15) / 16 * 16;
-    if (op->lds_per_wave > op->ctx->max_lds_per_block)
+    if (op->lds_per_wave > op->ctx->max_lds_per_block - kStaticLdsMax)
         return fail(RMX_ERR_UNSUPPORTED, "resize plan needs %d bytes of LDS per wave", op->lds_per_wave);
-    op->waves_per_block = std::max(1, std::min(4, op->ctx->max_lds_per_block / std::max(1, op->lds_per_wave)));
+    op->waves_per_block = std::max(1, std::min(4, (op->ctx->max_lds_per_block - kStaticLdsMax) / std::max(1, op->lds_per_wave)));
     op->tile_w = tile_w;
     op->aux1 = tile_w;
     // strips: short ones. A wave's steps are serialised by memory latency, so many short-lived
     // waves (several residency rounds) overlap better than one long-lived wave per slot; the
     // price is one extra window of source rows per strip. 8 rows measured best on MI355X.
-    {
-        const int rows = op->ctx->gen_rows;
-        op->strip_rows = rows;
-        op->aux0 = rows;
-        op->strips = std::max(1, (max_dh + rows - 1) / rows);
-    }
+    op->strip_rows = grows;
+    op->aux0 = grows;
+    op->strips = std::max(1, (max_dh + grows - 1) / grows);
     // fast path: every written width a multiple of 8 and aligned destination rows. Its wavefronts stage
     // the whole source window of a strip of `rows` destination rows at once; the x-tile of a sample is
-    // narrowed until that window fits the LDS budget of one wavefront. The sizes are computed with the
-    // kernel's own float formulas.
+    // narrowed until that window fits the LDS budget of one wavefront.
     op->fn_fast = nullptr;
     if (op->interp == RMX_INTERP_LINEAR && op->dst.w % 8 == 0) {
         // (the kernel multiplies row indices and the row stride with 24-bit multiplies)
         bool ok = op->src.w * 3u < (1u << 23) && op->src.h < (1u << 23);
-        for (int i = 0; i < op->n && ok; i++) ok = (t[i].dst_w % 8 == 0);
         // 4 rows and a 10 KB slice measured best on MI355X (more, shorter-lived wavefronts per CU)
         const int rows = op->ctx->fast_rows, cap = op->ctx->fast_lds;
         int need_max = 64;
         for (int i = 0; i < op->n && ok; i++) {
             RmxSample &s = t[i];
             s.plan[0] = 8;
-            if (s.dst_w <= 0 || s.dst_h <= 0) continue;
-            const float offx = (s.rx - 1.0f) * 0.5f, offy = (s.ry - 1.0f) * 0.5f;
-            const int xlo = s.src_x, xhi = s.src_x + s.src_w - 1;
-            int nrows = 2;
-            for (int r0 = 0; r0 < s.dst_h; r0 += rows) {
-                const int r1 = std::min(r0 + rows, (int)s.dst_h);
-                const int a_v = (int)std::floor(src_coord_h(s.pc_y + r0, s.ry, offy, (float)s.src_y));
-                const int b_v = (int)std::floor(src_coord_h(s.pc_y + r1 - 1, s.ry, offy, (float)s.src_y)) + 1;
-                nrows = std::max(nrows, b_v - a_v + 1);
+            if (s.dst_w % 8 != 0) {
+                ok = false;
+                break;
             }
+            if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+            const float magx = (float)(s.src_x + s.src_w + 2), magy = (float)(s.src_y + s.src_h + 2);
+            const int nrows = std::max(2, span_bound(std::min<int>(rows, s.dst_h) - 1, s.ry, magy) + 2);
             int tw = std::min<int>(s.dst_w, 512);
             for (;;) {
-                int pitch = 0;
-                for (int xt = 0; xt < s.dst_w; xt += tw) {
-                    const int w = std::min<int>(s.dst_w - xt, tw);
-                    const int ixmin = (int)std::floor(src_coord_h(s.pc_x + xt, s.rx, offx, (float)xlo));
-                    const int ixmax = (int)std::floor(src_coord_h(s.pc_x + xt + w - 1, s.rx, offx, (float)xlo));
-                    const int cs = std::max(std::min(ixmin, xhi), xlo), ce = std::max(std::min(ixmax + 1, xhi), xlo);
-                    const int nc = ce - cs + 1;
-                    pitch = std::max(pitch, (8 + ((nc + 3) >> 2) * 4) * 4);  // bytes: one dword per pixel + replicas
-                }
-                const long need = (long)nrows * pitch;
+                const int nc = std::min<int>(s.src_w, span_bound(tw - 1, s.rx, magx) + 2);
+                const long need = (long)nrows * (8 + ((nc + 3) >> 2) * 4) * 4;  // bytes: one dword per pixel + replicas
                 if (need <= cap) {
                     s.plan[0] = tw;
                     need_max = std::max<int>(need_max, (int)need);
@@ -752,8 +768,58 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             op->fast_rows = rows;
             op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
             // (default 1: a workgroup's LDS is released only when its last wavefront ends, one-wave groups keep the CU full)
-            op->fast_wpb = std::max(1, std::min(op->ctx->fast_wpb, op->ctx->max_lds_per_block / std::max(1, op->fast_lds)));
+            op->fast_wpb = std::max(1, std::min(op->ctx->fast_wpb, (op->ctx->max_lds_per_block - kStaticLdsMax) / std::max(1, op->fast_lds)));
             op->fast_needs_src16 = false;  // its loads only need dword alignment
+            op->fast_aux1 = 0;
+            if (op->fast_lds > op->ctx->max_lds_per_block - kStaticLdsMax) op->fn_fast = nullptr;
+        }
+        // Streaming variant (source rows straight into LDS): needs every source row to start at
+        // the same byte phase (row stride a multiple of 4) and a destination format it is built for.
+        bool dma = ok && op->fn_fast && op->ctx->dma;
+        if (dma) {
+            if (op->layout.empty()) dma = (op->src.w * 3u) % 4u == 0;
+            else
+                for (int i = 0; i < op->n && dma; i++) dma = op->layout[i].row_stride % 4u == 0;
+        }
+        const char *dname = nullptr;
+        rmx::KernelFn dfn = dma ? rmx::select_resize_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &dname) : nullptr;
+        if (dfn) {
+            // 10 KB measured best on MI355X: smaller caps cut more rows into two tiles, and the kernel's registers allow 16
+            // wavefronts per CU, which 10 KB each still fit
+            const int bufcap = std::min(op->ctx->dma_lds, 10 * 1024);  // the kernel issues at most 10 loads of 1 KB per window
+            int need_max = 64;
+            std::vector<int32_t> tws((size_t)op->n, 8);
+            for (int i = 0; i < op->n && dma; i++) {
+                const RmxSample &s = t[i];
+                if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+                const float magx = (float)(s.src_x + s.src_w + 2), magy = (float)(s.src_y + s.src_h + 2);
+                const int nrows = std::max(2, span_bound(std::min<int>(rows, s.dst_h) - 1, s.ry, magy) + 2);
+                int tw = std::min<int>(s.dst_w, 512);
+                for (;;) {
+                    const int nc = std::min<int>(s.src_w, span_bound(tw - 1, s.rx, magx) + 2);
+                    const long need = (long)nrows * (1 + ((3 + 3 * (nc + 2) + 8 + 15) >> 4)) * 16;  // margin piece + data + replicas
+                    if (need <= bufcap) {
+                        tws[(size_t)i] = tw;
+                        need_max = std::max<int>(need_max, (int)need);
+                        break;
+                    }
+                    if (tw <= 8) {
+                        dma = false;
+                        break;
+                    }
+                    tw = std::max(8, (tw / 2) / 8 * 8);
+                }
+            }
+            if (dma && need_max <= op->ctx->max_lds_per_block - kStaticLdsMax) {
+                for (int i = 0; i < op->n; i++) t[i].plan[0] = tws[(size_t)i];
+                op->fn_fast = dfn;
+                op->fast_name = dname;
+                op->fast_lds = (need_max + 15) / 16 * 16;
+                op->fast_rows = rows;
+                op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
+                op->fast_wpb = std::max(1, std::min(op->ctx->fast_wpb, (op->ctx->max_lds_per_block - kStaticLdsMax) / std::max(1, op->fast_lds)));
+                op->fast_aux1 = 0;
+            }
         }
     }
     return RMX_OK;
@@ -775,6 +841,7 @@ static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint3
     int slot = next_slot(op, &t);
     if (slot < 0) return RMX_ERR_HIP;
     uint64_t bytes = 0;
+    const bool edge_ref = (op->flags & RMX_F_EDGE_REF) && op->interp == RMX_INTERP_LINEAR;
     for (int i = 0; i < op->n; i++) {
         RmxSample &s = t[i];
         int rc = read_roi(op, src_roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
@@ -797,7 +864,7 @@ static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint3
         s.dst_w = std::min<int32_t>(s.dst_w, (int32_t)op->dst.w);
         s.dst_h = std::min<int32_t>(s.dst_h, (int32_t)op->dst.h);
         if (s.src_w <= 0 || s.src_h <= 0 || s.rs_w <= 0 || s.rs_h <= 0) s.dst_w = s.dst_h = 0;
-        s.flags = (mirror && mirror[i]) ? RMX_S_HFLIP : 0u;
+        s.flags = ((mirror && mirror[i]) ? RMX_S_HFLIP : 0u) | (edge_ref ? RMX_S_EDGE_REF : 0u);
         if (s.dst_w > 0) {
             s.rx = (float)s.src_w / (float)s.rs_w;
             s.ry = (float)s.src_h / (float)s.rs_h;

@@ -36,7 +36,12 @@ struct RmxSrcLayout {
 };
 static_assert(sizeof(RmxSrcLayout) == 16, "source layout entry must stay 16 bytes");
 
-enum : uint32_t { RMX_S_HFLIP = 1u, RMX_S_VFLIP = 2u, RMX_S_CHREV = 4u /* output channel k reads source channel 2-k */ };
+enum : uint32_t {
+    RMX_S_HFLIP = 1u,
+    RMX_S_VFLIP = 2u,
+    RMX_S_CHREV = 4u,    // output channel k reads source channel 2-k
+    RMX_S_EDGE_REF = 8u  // bilinear: both neighbours clamp to the window's last-but-one column / row (RMX_F_EDGE_REF)
+};
 
 struct RmxKArgs {
     const uint8_t *src;      // batch base, u8 NHWC

@@ -1,0 +1,311 @@
+// K2 streaming path: bilinear resize + epilogue for batches in which every written width is a multiple of 8, the
+// destination base is 16-byte aligned and every source row starts at the same byte phase (row stride a multiple of 4:
+// padded batches whose width is a multiple of 4, which the training shapes are).
+//
+// One wavefront = a strip of destination rows of one sample, one x-tile at a time, as in the staged kernel
+// (rmx_kernels_resize_fast.hip), but the source window travels from global memory straight into LDS
+// (global_load_lds_dwordx4: 16 bytes per lane, no vector register, no unpacking, no LDS store instruction):
+//   1. LDS holds the raw packed-RGB rows. A row is a sequence of 16-byte pieces: piece 0 is a margin for the left
+//      edge replica, pieces 1.. are the row's bytes from the dword that holds the window's first pixel. (row, piece)
+//      pairs form one flat index space dealt to the 64 lanes; every load instruction fills 1 KB of LDS. The compiler
+//      does not order LDS reads behind such loads, so arrival is awaited with an explicit s_waitcnt vmcnt(0) between
+//      two wavefront fences; the x taps are computed while the loads are in flight;
+//   2. the blend reads a tap pair (two packed pixels, 6 bytes at any byte phase) as three aligned dwords and
+//      realigns them with two v_alignbyte; every value and every operation after that is the general kernel's,
+//      operation for operation (bit-identical results).
+// Against the staged kernel this trades about 25 staging instructions per 4 source pixels for 4 realignments per
+// destination pixel (the vector-instruction count stays within 3 %), frees the registers the staged loads occupy and
+// needs a quarter less LDS (3 bytes per pixel instead of 4). Measured on the RandomResizedCrop batch with every launch
+// reading and writing buffers that were not touched for a gigabyte: 33.9 us against 36.4 us; replayed on one
+// cache-resident pair both take 29.5 us. Tried and measured slower: two windows per wavefront with the next strip's loads
+// in flight during the blend (38-41 us: 12 KB of LDS per wavefront leaves 13 wavefronts per CU), all LDS reads of a pass
+// issued before its arithmetic (129 registers, 3 wavefronts per SIMD), register budgets of 96 and 80 (spills).
+#include "rmx_device.h"
+#include "rmx_color_math.h"
+#include "rmx_launch.h"
+
+#include <type_traits>
+
+namespace rmx {
+
+extern __shared__ uint32_t rmx_lds_dma[];
+
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+typedef __attribute__((address_space(3))) uint8_t lds_u8;    // explicit LDS pointers: every access below is a DS instruction,
+typedef __attribute__((address_space(3))) uint32_t lds_u32;  // never a FLAT one (which would also count as vector memory)
+
+RMX_DEV float src_coord_d(int u, float ratio, float off, float lo) {
+    float s = (float)u * ratio;
+    s = s + off;
+    s = s + lo;
+    return s;
+}
+
+constexpr int DMA_SLOTS = 10;  // load instructions per window at most: 10 x 64 pieces of 16 bytes = 10 KB
+
+// One window: a strip of destination rows x one x-tile. Every member is wave-uniform.
+struct DmaItem {
+    int r0, r1;      // destination rows [r0, r1)
+    int xt, tw;      // destination columns [xt, xt + tw)
+    int a_v, nrows;  // virtual source rows a_v .. a_v + nrows - 1 (clamped into the window when fetched)
+    int cs, nc;      // source columns cs .. cs + nc - 1
+    int ph;          // byte phase of pixel cs inside its dword
+    int ppr;         // 16-byte pieces per LDS row (margin + data + room for the right replicas)
+    int nd;          // data pieces per row
+    uint32_t col4;   // byte offset (from base4) of the dword that holds pixel cs, within a row
+    int ns;          // load instructions
+    bool rep_l, rep_r, safe;
+};
+
+// CHAIN: a colour node between the (quantised) resize and the normalisation, see chain_colour().
+template <typename T, int LAYOUT, bool NORM, bool QUANT, int CHAIN>
+__global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
+    static_assert(CHAIN == CHAIN_NONE || QUANT, "a colour node in the chain reads the u8 output of the resize node");
+    static_assert(!(sizeof(T) == 4 && LAYOUT == RMX_NHWC), "interleaved fp32 goes through the coalescing stores of the staged kernel");
+    __shared__ __attribute__((aligned(16))) float chain_tables[CHAIN == CHAIN_TWIST ? sizeof(ColorTables) / 4 : 4];
+    const int lane = threadIdx.x & (RMX_WAVE - 1);
+    const int wib = threadIdx.x / RMX_WAVE;
+    const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
+    uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
+    wave = __builtin_amdgcn_readfirstlane(wave);
+    if (wave >= nwaves) return;
+    const int s = (int)(wave / (uint32_t)a.strips);
+    const int grp = (int)(wave % (uint32_t)a.strips);
+    const RmxSample P = a.table[s];
+    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.plan[0]));
+
+    const int dw = P.dst_w, dh = P.dst_h;
+    const int srows = a.aux0;
+    const int r_begin = grp * srows;
+    if (r_begin >= dh || dw <= 0) return;
+    const int r_end = min(r_begin + srows, dh);
+    const bool hf = (P.flags & RMX_S_HFLIP) != 0;
+
+    const int xlo = P.src_x, ylo = P.src_y;
+    const int edge = (int)((P.flags / RMX_S_EDGE_REF) & 1u);
+    const int xhi = max(xlo + P.src_w - 1 - edge, xlo), yhi = max(ylo + P.src_h - 1 - edge, ylo);
+    const float rx = P.rx, ry = P.ry;
+    const float offx = (rx - 1.0f) * 0.5f, offy = (ry - 1.0f) * 0.5f;
+    const float fxlo = (float)xlo, fylo = (float)ylo;
+    const int pcx = P.pc_x, pcy = P.pc_y;
+
+    T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
+    uint32_t *lds = rmx_lds_dma + (size_t)wib * (a.lds_bytes >> 2);
+
+    float sc[3], bi[3];
+#pragma unroll
+    for (int c = 0; c < 3; c++) {
+        sc[c] = P.scale[c];
+        bi[c] = P.bias[c];
+    }
+    const float cp[4] = {P.m[0], P.m[1], P.m[2], P.m[3]};
+    const float sh2 = cp[2] + 2.0f, sh4 = cp[2] + 4.0f;
+    const ColorTables *ctab = reinterpret_cast<const ColorTables *>(chain_tables);
+    if constexpr (CHAIN == CHAIN_TWIST) color_tables_fill(reinterpret_cast<ColorTables *>(chain_tables), lane);
+
+    uint32_t row_stride;
+    const uint8_t *simg = sample_base(a, s, row_stride);
+    const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
+    const uint8_t *base4 = simg - skew;
+    const uint64_t left = (uint64_t)((a.src + a.src_bytes) - base4);
+    const uint32_t lim = left > 0xffffffffull ? 0xffffffffu : (uint32_t)left;
+
+    const int tile_w = max(P.plan[0], PX);
+    const int ntx = (dw + tile_w - 1) / tile_w;
+
+    auto make_item = [&](int tile) {
+        DmaItem g;
+        g.r0 = r_begin;
+        g.r1 = r_end;
+        g.xt = tile * tile_w;
+        g.tw = min(dw - g.xt, tile_w);
+        g.a_v = (int)floorf(src_coord_d(pcy + g.r0, ry, offy, fylo));
+        const int b_v = (int)floorf(src_coord_d(pcy + g.r1 - 1, ry, offy, fylo)) + 1;
+        g.nrows = b_v - g.a_v + 1;
+        const int ixmin = (int)floorf(src_coord_d(pcx + g.xt, rx, offx, fxlo));
+        const int ixmax = (int)floorf(src_coord_d(pcx + g.xt + g.tw - 1, rx, offx, fxlo));
+        g.cs = max(min(ixmin, xhi), xlo);
+        const int ce = max(min(ixmax + 1, xhi), xlo);
+        g.nc = ce - g.cs + 1;
+        g.rep_l = ixmin < xlo;
+        g.rep_r = ixmax + 1 > xhi;
+        const uint32_t colb = (uint32_t)g.cs * 3u + skew;
+        g.ph = (int)(colb & 3u);
+        g.col4 = colb & ~3u;
+        g.nd = (g.ph + 3 * g.nc + 15) >> 4;
+        g.ppr = 1 + ((g.ph + 3 * (g.nc + 2) + 8 + 15) >> 4);
+        const int tp = g.nrows * g.ppr;
+        g.ns = (tp + RMX_WAVE - 1) / RMX_WAVE;
+        // every 16-byte piece of every row lies inside the batch buffer (the last rows of the last sample may not)
+        const uint32_t last_row = (uint32_t)max(min(b_v, yhi), ylo) * row_stride + g.col4;
+        g.safe = (uint64_t)last_row + 16ull * (uint64_t)g.nd <= (uint64_t)lim;
+        return g;
+    };
+
+    // Starts the window's transfer into `buf`. A piece is 16 bytes at a dword-aligned address; the margin piece and the
+    // pieces behind the row's data repeat a neighbouring data piece (their content is never read before a replica is
+    // written over it).
+    auto issue = [&](DmaItem &g, uint32_t *buf) {
+        const int tp = g.nrows * g.ppr;
+        const float inv_ppr = 1.0f / (float)g.ppr;
+        if (g.safe) {
+#pragma unroll
+            for (int j = 0; j < DMA_SLOTS; j++) {
+                if (j < g.ns) {
+                    const int idx = j * RMX_WAVE + lane;
+                    if (idx < tp) {
+                        const int r = (int)(((float)idx + 0.5f) * inv_ppr);  // idx / ppr, exact: idx < 2^16
+                        const int c = idx - __mul24(r, g.ppr);
+                        const int ysrc = max(min(g.a_v + r, yhi), ylo);
+                        const int piece = max(min(c - 1, g.nd - 1), 0);
+                        const uint32_t off = (uint32_t)__mul24(ysrc, (int)row_stride) + g.col4 + 16u * (uint32_t)piece;
+                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(base4 + off), (lds_ptr_t)(buf + j * (RMX_WAVE * 4)), 16, 0, 0);
+                    }
+                }
+            }
+        } else {
+            // the window touches the last bytes of the batch buffer: bounds-checked byte loads, stored by the lanes
+            for (int idx = lane; idx < tp; idx += RMX_WAVE) {
+                const int r = idx / g.ppr;
+                const int c = idx - r * g.ppr;
+                const int ysrc = max(min(g.a_v + r, yhi), ylo);
+                const int piece = max(min(c - 1, g.nd - 1), 0);
+                const uint32_t off = (uint32_t)ysrc * row_stride + g.col4 + 16u * (uint32_t)piece;
+                uint32_t w[4];
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t v = 0;
+#pragma unroll
+                    for (int b = 0; b < 4; b++) {
+                        const uint32_t ob = off + 4u * i + b;
+                        v |= (ob < lim ? (uint32_t)base4[ob] : 0u) << (8 * b);
+                    }
+                    w[i] = v;
+                }
+                lds_u32 *dst4 = (lds_u32 *)(lds_ptr_t)(buf + 4 * idx);
+                dst4[0] = w[0]; dst4[1] = w[1]; dst4[2] = w[2]; dst4[3] = w[3];
+            }
+            g.ns = 0;
+        }
+    };
+
+    // x taps of a tile: byte offset of the left neighbour inside an LDS row (dword part and byte phase) and the weights
+    uint32_t bo4[PX], bsh[PX];
+    float wx[PX], omx[PX];
+    int L = 1, G = 1, lr = 0, gl = 0, t0 = 0;
+    bool lane_on = false;
+    auto taps = [&](const DmaItem &g) {
+        L = g.tw / PX;
+        G = RMX_WAVE / L;
+        lr = lane / L;
+        gl = lane - lr * L;
+        t0 = g.xt + gl * PX;
+        lane_on = lr < G;
+#pragma unroll
+        for (int k = 0; k < PX; k++) {
+            float sx = src_coord_d(pcx + t0 + k, rx, offx, fxlo);
+            float fx = floorf(sx);
+            wx[k] = sx - fx;
+            omx[k] = 1.0f - wx[k];
+            const uint32_t b = (uint32_t)(16 + g.ph + 3 * ((int)fx - g.cs));
+            bo4[k] = b & ~3u;
+            bsh[k] = b & 3u;
+        }
+    };
+
+    for (int tile = 0; tile < ntx; tile++) {
+        uint32_t *buf = lds;
+        DmaItem cur = make_item(tile);
+        wave_sync();  // the blend of the tile before has read the window for the last time
+        issue(cur, buf);
+        taps(cur);  // while the loads are in flight
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        wave_sync();
+        const int pitch_b = cur.ppr * 16;
+        lds_u8 *bufb = (lds_u8 *)(lds_ptr_t)buf;
+        // clamp-to-edge: the pixel before the window's first column repeats it, the two after its last column repeat that
+        if (cur.rep_l || cur.rep_r) {
+            for (int rr = lane; rr < cur.nrows; rr += RMX_WAVE) {
+                lds_u8 *row = bufb + rr * pitch_b + 16 + cur.ph;
+                if (cur.rep_l) {
+#pragma unroll
+                    for (int b = 0; b < 3; b++) row[b - 3] = row[b];
+                }
+                if (cur.rep_r) {
+                    lds_u8 *lastpx = row + 3 * (cur.nc - 1);
+#pragma unroll
+                    for (int b = 0; b < 3; b++) lastpx[3 + b] = lastpx[6 + b] = lastpx[b];
+                }
+            }
+            wave_sync();
+        }
+
+        // ---- blend, epilogue, store: G rows per pass
+        const int x0 = hf ? (dw - t0 - PX) : t0;
+        for (int rs = cur.r0; rs < cur.r1; rs += G) {
+            const int r = rs + lr;
+            if (lane_on && r < cur.r1) {
+                float sy = src_coord_d(pcy + r, ry, offy, fylo);
+                float fy = floorf(sy);
+                float wy = sy - fy;
+                const lds_u8 *row0 = bufb + ((int)fy - cur.a_v) * pitch_b;
+                const lds_u8 *row1 = row0 + pitch_b;
+                const float omy = 1.0f - wy;
+                float v[3][PX];
+#pragma unroll
+                for (int k = 0; k < PX; k++) {
+                    const lds_u32 *q0 = (const lds_u32 *)(row0 + bo4[k]);
+                    const lds_u32 *q1 = (const lds_u32 *)(row1 + bo4[k]);
+                    const uint32_t a0 = q0[0], a1 = q0[1], a2 = q0[2], b0 = q1[0], b1 = q1[1], b2 = q1[2];
+                    // tl = R G B of the left neighbour and R of the right one; tr = G B of the right one
+                    const uint32_t tl = __builtin_amdgcn_alignbyte(a1, a0, bsh[k]), tr = __builtin_amdgcn_alignbyte(a2, a1, bsh[k]);
+                    const uint32_t bl = __builtin_amdgcn_alignbyte(b1, b0, bsh[k]), br = __builtin_amdgcn_alignbyte(b2, b1, bsh[k]);
+                    float w00 = omy * omx[k], w01 = omy * wx[k], w10 = wy * omx[k];
+                    float o0 = __builtin_fmaf(ubyte0(tl), w00, __builtin_fmaf(ubyte3(tl), w01, __builtin_fmaf(ubyte0(bl), w10, ubyte3(bl) * wy * wx[k])));
+                    float o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte0(br) * wy * wx[k])));
+                    float o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte1(br) * wy * wx[k])));
+                    if constexpr (QUANT) {
+                        o0 = __builtin_rintf(o0); o1 = __builtin_rintf(o1); o2 = __builtin_rintf(o2);
+                    }
+                    chain_colour<CHAIN>(o0, o1, o2, cp, sh2, sh4, ctab);
+                    if constexpr (NORM) {
+                        o0 = __builtin_fmaf(o0, sc[0], bi[0]); o1 = __builtin_fmaf(o1, sc[1], bi[1]); o2 = __builtin_fmaf(o2, sc[2], bi[2]);
+                    }
+                    v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
+                }
+                PackedGroup<T> packed;
+                pack_group<T, LAYOUT>(v, hf, packed);
+                store_packed<T, LAYOUT, sizeof(T) == 2>(dimg, a.dst_h, a.dst_w, r, x0, packed);  // fp16: streaming stores
+            }
+        }
+    }
+}
+
+template <typename T, int LAYOUT>
+static KernelFn pick3(bool norm, bool quant, int chain) {
+    if (norm && quant && chain == CHAIN_LINEAR) return (KernelFn)rmx_resize_dma_kernel<T, LAYOUT, true, true, CHAIN_LINEAR>;
+    if (norm && quant && chain == CHAIN_TWIST) return (KernelFn)rmx_resize_dma_kernel<T, LAYOUT, true, true, CHAIN_TWIST>;
+    if (norm && quant) return (KernelFn)rmx_resize_dma_kernel<T, LAYOUT, true, true, CHAIN_NONE>;
+    if (norm) return (KernelFn)rmx_resize_dma_kernel<T, LAYOUT, true, false, CHAIN_NONE>;
+    return (KernelFn)rmx_resize_dma_kernel<T, LAYOUT, false, false, CHAIN_NONE>;
+}
+
+// Null for the one combination this kernel leaves to the staged fast kernel (interleaved fp32).
+KernelFn select_resize_dma_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name) {
+    *name = "rmx_resize_dma_kernel";
+    if (layout == RMX_NCHW) {
+        switch (dtype) {
+            case RMX_FP32: return pick3<float, RMX_NCHW>(norm, quant, chain);
+            case RMX_FP16: return pick3<__half, RMX_NCHW>(norm, quant, chain);
+            default: return pick3<uint8_t, RMX_NCHW>(norm, quant, chain);
+        }
+    }
+    switch (dtype) {
+        case RMX_FP32: return nullptr;
+        case RMX_FP16: return pick3<__half, RMX_NHWC>(norm, quant, chain);
+        default: return pick3<uint8_t, RMX_NHWC>(norm, quant, chain);
+    }
+}
+
+}  // namespace rmx

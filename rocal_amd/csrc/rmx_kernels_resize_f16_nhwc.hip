@@ -1,0 +1,6 @@
+// K2 general path, instantiations for one destination type and layout (see rmx_kernels_resize_impl.h).
+#include "rmx_kernels_resize_impl.h"
+
+namespace rmx {
+RMX_RESIZE_UNIT(__half, RMX_NHWC, resize_unit_f16_nhwc)
+}  // namespace rmx

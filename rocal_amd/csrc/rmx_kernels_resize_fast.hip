@@ -73,7 +73,9 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
     const bool hf = (P.flags & RMX_S_HFLIP) != 0;
 
     const int xlo = P.src_x, ylo = P.src_y;
-    const int xhi = xlo + P.src_w - 1, yhi = ylo + P.src_h - 1;
+    // last column / row a tap may read: the window's last one, or the one before it under the reference's device edge rule
+    const int edge = (int)((P.flags / RMX_S_EDGE_REF) & 1u);
+    const int xhi = max(xlo + P.src_w - 1 - edge, xlo), yhi = max(ylo + P.src_h - 1 - edge, ylo);
     const float rx = P.rx, ry = P.ry;
     const float offx = (rx - 1.0f) * 0.5f, offy = (ry - 1.0f) * 0.5f;
     const float fxlo = (float)xlo, fylo = (float)ylo;
@@ -219,7 +221,7 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
             for (int rr = lane; rr < nrows; rr += RMX_WAVE) {
                 uint32_t *row = lds + rr * pitch;
                 if (rep_l) row[3] = row[4];
-                if (rep_r) row[4 + nc] = row[4 + nc - 1];
+                if (rep_r) row[4 + nc] = row[4 + nc + 1] = row[4 + nc - 1];  // two: under the device edge rule a left tap can lie one beyond
             }
             wave_sync();
         }

@@ -248,6 +248,14 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         outs.push_back(rocalBlendFixed(ctx, src, bright, 0.3f, true));
         // a second input of another shape is refused when the graph is built, a missing one at once
         if (rocalBlendFixed(ctx, src, nullptr, 0.3f, true) != nullptr) return 14;
+    } else if (scenario == "second_reader") {
+        // the resized tensor feeds CropMirrorNormalize AND is the second input of a Blend node: it has two readers, so
+        // resize -> CropMirrorNormalize must not be fused (the tensor has to exist for the Blend)
+        mid = rocalResize(ctx, src, 40, 32, false);
+        outs.push_back(rocalCropMirrorNormalize(ctx, mid, 32, 40, 0.5f, 0.5f, mean, stdv, true, rocalCreateIntParameter(0), ROCAL_NCHW, ROCAL_FP32));
+        RocalTensor other = rocalResize(ctx, src, 40, 32, true, ROCAL_SCALING_MODE_STRETCH, {}, 0, 0, ROCAL_NEAREST_NEIGHBOR_INTERPOLATION);
+        outs.push_back(other);
+        outs.push_back(rocalBlendFixed(ctx, other, mid, 0.25f, true));
     } else if (scenario == "to_tensor") {
         outs.push_back(rocalResize(ctx, src, 40, 32, true));
     } else if (scenario == "errors") {

@@ -116,11 +116,8 @@ Graph::Status Graph::verify() {
         Node *a = _order[i], *b = _order[i + 1];
         if (a->fused_away || b->fused_away) continue;
         Tensor *mid = a->output()[0];
-        if (b->input()[0] != mid || mid->is_output) continue;
-        bool other_reader = false;
-        for (size_t k = 0; k < _order.size(); k++)
-            if (k != i + 1 && _order[k]->input()[0] == mid) other_reader = true;
-        if (other_reader) continue;
+        if (b->input().size() != 1 || b->input()[0] != mid || mid->is_output) continue;
+        if (readers(mid) != 1) continue;  // counts every input of every node: a two-input node may read it as its second
         if (a->try_absorb(b)) {
             b->fused_away = true;
             mid->elided = true;

@@ -16,6 +16,7 @@ ROI_LTRB, ROI_XYWH = 0, 1
 NEAREST, LINEAR, TRIANGULAR = 0, 1, 5
 F_QUANTIZE_U8 = 1
 F_COLOR_LINEAR, F_COLOR_TWIST = 2, 4
+F_EDGE_REF = 8  # bilinear neighbours clamp to the window's last-but-one column / row, as the reference's device code does
 
 
 def _torch():
@@ -99,7 +100,28 @@ class Op:
             arr, p = _arr(a, dt)
             keep.append(arr)
             ptrs.append(p)
-        check(getattr(_lib.lib(), name)(self._h, *ptrs))
+        fn = getattr(_lib.lib(), name)
+        self._last_update = (fn, keep, ptrs)
+        check(fn(self._h, *ptrs))
+
+    def prepared_update(self):
+        """A zero-argument callable that repeats the last update with the same (already converted) host arrays:
+        the C-ABI call alone, without numpy conversions - what a C++ caller pays per batch."""
+        fn, keep, ptrs = self._last_update
+        h = self._h
+
+        def call(_keep=keep):
+            check(fn(h, *ptrs))
+        return call
+
+    def prepared_launch(self, src, dst):
+        """A zero-argument callable that launches on these two batch buffers (checked once, here)."""
+        assert src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()
+        fn, h, ps, pd = _lib.lib().rmx_op_launch, self._h, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr())
+
+        def call(_keep=(src, dst)):
+            check(fn(h, ps, pd))
+        return call
 
     def launch(self, src, dst):
         """src/dst: torch CUDA tensors (the batch buffers). Asynchronous on the context's stream."""

@@ -76,7 +76,8 @@ def test_resize_colour_cmn_chain(ctx, kind, aligned):
         op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, oh, ow, layout, dtype), ops.LINEAR,
                         flags=ops.F_QUANTIZE_U8 | flag)
         op.update_color_cmn(roi, rw, rh, scale, bias, arrays, mirror, crop)
-        assert op.kernel_name == ("rmx_resize_fast_kernel" if aligned else "rmx_resize_kernel")
+        # aligned: the streaming kernel (planar fp16; the source rows are 360 bytes) or the staged one (interleaved fp32)
+        assert op.kernel_name == (("rmx_resize_dma_kernel" if dtype == ops.FP16 else "rmx_resize_fast_kernel") if aligned else "rmx_resize_kernel")
         out = op.alloc_output()
         op.launch(torch.from_numpy(img).cuda(), out)
         ctx.sync()
@@ -98,7 +99,7 @@ def test_random_resized_crop_colour_twist_cmn_full_size(ctx):
                     flags=ops.F_QUANTIZE_U8 | ops.F_COLOR_TWIST)
     arrays = (c2["alpha"], c2["beta"], c2["hue"], c2["sat"])
     op.update_color_cmn(c["roi"], dw, dw, scale, bias, arrays, c["mirror"])
-    assert op.kernel_name == "rmx_resize_fast_kernel"
+    assert op.kernel_name == "rmx_resize_dma_kernel"
     out = op.alloc_output()
     op.launch(torch.from_numpy(c["img"]).cuda(), out)
     ctx.sync()

@@ -1,0 +1,140 @@
+"""The two aligned bilinear kernels against each other and against the oracle, bit for bit: the streaming kernel (source rows
+straight into LDS) and the staged kernel (windows through registers). Covers what is specific to the streaming kernel: the
+byte phases of packed pixels inside LDS rows, both edge replicas, rows cut into several x-tiles, strips of one to eight rows,
+the window that ends on the last byte of the batch buffer, ragged sources and every destination format it serves."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from rocal_amd import ops, workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _run(c, desc_src, desc_dst, flags, update, img):
+    op = ops.Resize(c, desc_src, desc_dst, ops.LINEAR, flags=flags)
+    update(op)
+    out = op.alloc_output()
+    op.launch(img, out)
+    c.sync()
+    return out.cpu().numpy(), op.kernel_name, op.plan
+
+
+def _scale_bias(n):
+    return orc.cmn_scale_bias(wl.MEAN, wl.STD, n)
+
+
+@pytest.mark.parametrize("layout,dtype", [(ops.NCHW, ops.FP16), (ops.NCHW, ops.FP32), (ops.NCHW, ops.UINT8), (ops.NHWC, ops.FP16), (ops.NHWC, ops.UINT8)])
+def test_streaming_and_staged_kernels_agree_with_the_oracle(ctx, ctx_staged, ctx_dma_small, layout, dtype):
+    rng = np.random.default_rng(4400 + 7 * layout + dtype)
+    n, H, W = 10, 150, 200  # 600-byte rows: every row starts at the same byte phase
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.empty((n, 4), np.uint32)
+    for i in range(n):
+        w, h = int(rng.integers(1, W + 1)), int(rng.integers(1, H + 1))
+        roi[i] = (int(rng.integers(0, W - w + 1)), int(rng.integers(0, H - h + 1)), w, h)
+    roi[0] = (0, 0, W, H)            # both edge replicas of the whole image
+    roi[1] = (W - 9, H - 5, 9, 5)    # the window that ends on the last byte ... of sample 1
+    roi[n - 1] = (W - 40, H - 30, 40, 30)  # ... and of the batch buffer: the bounds-checked staging
+    roi[2] = (3, 5, 1, 1)            # a single pixel
+    # ratios of at most 3 in both directions: windows that fit the smallest LDS setting in tiles of at least 8 columns
+    dw = np.array([8 * int(rng.integers(-(-int(roi[i, 2]) // 24), 17)) for i in range(n)], np.uint32)
+    dh = np.array([int(rng.integers(-(-int(roi[i, 3]) // 3), 100)) for i in range(n)], np.uint32)
+    dw[0], dh[0] = 128, 97
+    mirror = rng.integers(0, 2, n).astype(np.uint32)
+    scale, bias = _scale_bias(n)
+    norm = dtype != ops.UINT8
+    flags = ops.F_QUANTIZE_U8 if norm else 0
+    oflags = orc.F_QUANTIZE_U8 if norm else 0
+    exp = orc.resize(img, roi, dw, dh, 100, 128, interp=orc.LINEAR, mirror=mirror, scale=scale if norm else None, bias=bias if norm else None,
+                     layout=layout, dtype=dtype, flags=oflags)
+    sd, dd = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 100, 128, layout, dtype)
+
+    def update(op):
+        if norm:
+            op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        else:
+            op.update(roi, dw, dh, mirror)
+    dimg = _gpu(img)
+    names = []
+    for c in (ctx, ctx_staged, ctx_dma_small):
+        got, name, plan = _run(c, sd, dd, flags, update, dimg)
+        names.append(name)
+        # written windows only: the rest of the padded destination keeps the fill value on both sides
+        for i in range(n):
+            g = got[i, :, :dh[i], :dw[i]] if layout == ops.NCHW else got[i, :dh[i], :dw[i]]
+            e = exp[i, :, :dh[i], :dw[i]] if layout == ops.NCHW else exp[i, :dh[i], :dw[i]]
+            assert np.array_equal(g.view(np.uint8), e.view(np.uint8)), "sample %d differs (%s, %s)" % (i, name, plan)
+    assert names == ["rmx_resize_dma_kernel", "rmx_resize_fast_kernel", "rmx_resize_dma_kernel"]
+
+
+@pytest.mark.parametrize("rows", [1, 3, 4, 8])
+def test_strip_heights(rows):
+    """Strips of one to eight rows, with destination heights that leave a short last strip."""
+    from conftest import _ctx_with_env
+    c = _ctx_with_env(RMX_TUNE_FAST_ROWS=rows)
+    rng = np.random.default_rng(99)
+    n, H, W = 6, 96, 128
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    roi = np.array([[0, 0, 128, 96], [7, 9, 100, 80], [0, 0, 64, 96], [20, 20, 31, 17], [1, 0, 127, 96], [0, 3, 128, 90]], np.uint32)
+    dw = np.array([64, 128, 8, 72, 128, 96], np.uint32)
+    dh = np.array([61, 1, 47, 4, 96, 5], np.uint32)
+    mirror = np.array([0, 1, 1, 0, 1, 0], np.uint32)
+    scale, bias = _scale_bias(n)
+    exp = orc.resize(img, roi, dw, dh, 96, 128, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                     flags=orc.F_QUANTIZE_U8)
+    got, name, plan = _run(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 96, 128, ops.NCHW, ops.FP16), ops.F_QUANTIZE_U8,
+                           lambda op: op.update_cmn(roi, dw, dh, scale, bias, mirror), _gpu(img))
+    assert name == "rmx_resize_dma_kernel" and ("strip_rows=%d " % rows) in plan, plan
+    for i in range(n):
+        assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp[i, :, :dh[i], :dw[i]].view(np.uint16)), "sample %d (%s)" % (i, plan)
+    c.close()
+
+
+def test_ragged_source_with_dword_row_strides(ctx):
+    """Tightly packed images whose widths are multiples of 4 (row strides multiples of 4 bytes, bases at any dword): the streaming
+    kernel; one odd width sends the batch to the staged kernel. Same results."""
+    rng = np.random.default_rng(5)
+    n = 6
+    widths = np.array([64, 100, 36, 128, 88, 12], np.uint32)
+    heights = np.array([50, 33, 80, 64, 21, 9], np.uint32)
+    for odd in (False, True):
+        w = widths.copy()
+        if odd:
+            w[2] = 37
+        imgs = [rng.integers(0, 256, (int(heights[i]), int(w[i]), 3), dtype=np.uint8) for i in range(n)]
+        offsets, pos, parts = [], 0, []
+        for im in imgs:
+            pad = (-pos) % 4  # images start at dword addresses
+            parts.append(np.zeros(pad, np.uint8))
+            pos += pad
+            offsets.append(pos)
+            parts.append(im.reshape(-1))
+            pos += im.size
+        packed = np.concatenate(parts)
+        padded = np.zeros((n, 80, 128, 3), np.uint8)
+        for i, im in enumerate(imgs):
+            padded[i, :im.shape[0], :im.shape[1]] = im
+        roi = np.array([[0, 0, w[i], heights[i]] for i in range(n)], np.uint32)
+        roi[1] = (10, 5, 80, 20)
+        dw = np.array([48, 64, 40, 128, 8, 24], np.uint32)
+        dh = np.array([40, 30, 90, 50, 30, 18], np.uint32)
+        mirror = np.array([1, 0, 0, 1, 1, 0], np.uint32)
+        scale, bias = _scale_bias(n)
+        exp = orc.resize(padded, roi, dw, dh, 90, 128, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                         flags=orc.F_QUANTIZE_U8)
+        op = ops.Resize(ctx, ops.desc(n, 80, 128, ops.NHWC, ops.UINT8), ops.desc(n, 90, 128, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+        op.set_ragged_source(np.array(offsets, np.uint64), w, heights, packed.size)
+        op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        assert op.kernel_name == ("rmx_resize_fast_kernel" if odd else "rmx_resize_dma_kernel")
+        out = op.alloc_output()
+        op.launch(_gpu(packed), out)
+        ctx.sync()
+        got = out.cpu().numpy()
+        for i in range(n):
+            assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp[i, :, :dh[i], :dw[i]].view(np.uint16)), "sample %d, odd=%s" % (i, odd)

@@ -17,7 +17,7 @@ def _bits(a):
 
 @pytest.mark.parametrize("cfg", sorted(bench.WORKLOADS))
 def test_full_size_configuration_is_bit_identical_to_the_oracle(ctx, cfg):
-    op, src, dst, n, cpu = bench.build_case(cfg, ctx)
+    op, src, dst, n, cpu, _ = bench.build_case(cfg, ctx)
     dst.zero_()
     op.launch(*(src if isinstance(src, tuple) else (src,)), dst)
     ctx.sync()
@@ -30,7 +30,7 @@ def test_full_size_configuration_is_bit_identical_to_the_oracle(ctx, cfg):
 def test_fast_and_general_resize_kernels_agree_at_full_size(ctx):
     """A destination that is not 16-byte aligned sends the same batch through the general kernel."""
     import torch
-    op, src, dst, n, _ = bench.build_case(1, ctx)
+    op, src, dst, n, _, _ = bench.build_case(1, ctx)
     assert "fast=1" in op.plan
     op.launch(src, dst)
     big = torch.zeros(dst.numel() + 8, dtype=dst.dtype, device="cuda")
@@ -270,7 +270,7 @@ def test_large_windows_in_narrow_tiles_every_float_format(ctx, layout, dtype):
     dw = np.full(n, 224, np.uint32)
     op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, layout, dtype), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
     op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
-    assert op.kernel_name == "rmx_resize_fast_kernel"
+    assert op.kernel_name == ("rmx_resize_fast_kernel" if (layout, dtype) == (ops.NHWC, ops.FP32) else "rmx_resize_dma_kernel")
     out = op.alloc_output()
     op.launch(torch.from_numpy(c["img"]).cuda(), out)
     ctx.sync()

@@ -179,6 +179,42 @@ def test_rrc_cmn_fused_config1_small(ctx):
     assert np.array_equal(two.view(np.uint16), exp.view(np.uint16))
 
 
+@pytest.mark.parametrize("aligned", [True, False])
+def test_bilinear_reference_device_edge_rule(ctx, aligned):
+    """RMX_F_EDGE_REF: both neighbours clamp to [lo, hi-1] (rocal_hip_kernels.cpp:340-343,356-361), against the oracle's
+    ORC_F_BILINEAR_EDGE_QUIRK. Up-scaled, identity-size and down-scaled samples, windows of one and two columns / rows,
+    mirror; widths that take the aligned fast kernel and widths that take the general one."""
+    rng = np.random.default_rng(1234)
+    n, H, W = 8, 60, 72
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.array([[0, 0, 72, 60], [3, 2, 40, 30], [0, 0, 24, 20], [10, 5, 1, 1], [7, 7, 2, 2], [0, 0, 72, 3], [5, 0, 3, 60], [1, 1, 64, 48]], np.uint32)
+    if aligned:
+        dw = np.array([72, 80, 96, 8, 16, 72, 24, 64], np.uint32)
+    else:
+        dw = np.array([72, 81, 95, 7, 13, 70, 21, 64], np.uint32)
+    dh = np.array([60, 64, 80, 9, 12, 7, 60, 48], np.uint32)
+    mirror = np.array([0, 1, 0, 1, 0, 1, 0, 1], np.uint32)
+    exp = orc.resize(img, roi, dw, dh, 80, 96, interp=orc.LINEAR, mirror=mirror, flags=orc.F_BILINEAR_EDGE_QUIRK)
+    plain = orc.resize(img, roi, dw, dh, 80, 96, interp=orc.LINEAR, mirror=mirror)
+    assert (exp != plain).any()  # the rule changes the last columns / rows of up-scaled and same-size samples
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 80, 96, ops.NHWC, ops.UINT8), ops.LINEAR, flags=ops.F_EDGE_REF)
+    op.update(roi, dw, dh, mirror)
+    assert ("fast=1" in op.plan) == aligned
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="device edge rule, aligned=%s" % aligned)
+    # the fused RandomResizedCrop + CropMirrorNormalize chain under the same rule, fp16 planar
+    scale, bias = _mean_std(n)
+    expf = orc.resize(img, roi, dw, dh, 80, 96, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                      flags=orc.F_BILINEAR_EDGE_QUIRK | orc.F_QUANTIZE_U8)
+    op2 = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 80, 96, ops.NCHW, ops.FP16), ops.LINEAR,
+                     flags=ops.F_EDGE_REF | ops.F_QUANTIZE_U8)
+    op2.update_cmn(roi, dw, dh, scale, bias, mirror)
+    out2 = op2.alloc_output()
+    op2.launch(_gpu(img), out2)
+    _check(_cpu(out2, ctx), expf, ops.FP16, exact=True, what="device edge rule, fused chain, aligned=%s" % aligned)
+
+
 def test_resize_then_center_crop_fused(ctx):
     """resize(256) -> CMN centre crop 224 as one launch (post-crop window inside the resized image)."""
     rng = np.random.default_rng(11)

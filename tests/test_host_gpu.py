@@ -199,6 +199,22 @@ def test_gamma_exposure_colour_temperature_blend_nodes(tmp_path):
         _same(o[4][0], orc.blend(img, bright, _roi(), one(0.3)), "blend of the source and a node's output")
 
 
+def test_tensor_read_as_a_second_input_is_not_fused_away(tmp_path):
+    """resize -> {CropMirrorNormalize, Blend(other, resized)}: the resized tensor has two readers, one of them through a
+    node's second input, so the pair resize -> CropMirrorNormalize stays two launches and the tensor exists."""
+    img, outs, stdout = _run("second_reader", tmp_path, 3, [(np.float32, (N, 3, 32, 40)), (np.uint8, (N, 32, 40, 3)), (np.uint8, (N, 32, 40, 3))])
+    assert "intermediate_elided 0" in stdout
+    dw, dh = np.full(N, 40, np.uint32), np.full(N, 32, np.uint32)
+    mid = orc.resize(img, _roi(), dw, dh, 32, 40, interp=orc.LINEAR)
+    other = orc.resize(img, _roi(), dw, dh, 32, 40, interp=orc.NEAREST)
+    whole = np.tile(np.array([0, 0, 40, 32], np.uint32), (N, 1))
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    for o in outs:
+        _same(o[0][0], orc.crop_mirror_normalize(mid, whole, scale, bias, np.zeros(N, np.uint32), 32, 40, orc.NCHW, orc.FP32), "CropMirrorNormalize of the resized tensor")
+        _same(o[1][0], other, "nearest resize")
+        _same(o[2][0], orc.blend(other, mid, whole, np.full(N, 0.25, np.float32)), "blend with the resized tensor as second input")
+
+
 def test_to_tensor_of_the_u8_output(tmp_path):
     """rocalToTensor (rocal_api_data_transfer.cpp:30-52 -> MasterGraph::to_tensor): planar fp16 with reversed
     channels of the whole output, then an interleaved fp32 tensor of its top-left max_roi corner."""
