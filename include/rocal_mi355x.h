@@ -155,6 +155,21 @@ RMX_API int rmx_update_resize_color_cmn(rmx_op *op, const uint32_t *src_roi, con
                                         const uint32_t *crop_roi, const float *scale, const float *bias, const uint32_t *mirror,
                                         const float *c0, const float *c1, const float *c2, const float *c3);
 
+/* ---- The fused chain resize -> CropMirrorNormalize in ONE call that allocates nothing. It has no counterpart in the
+ *      reference; it is for callers that cannot allocate: code under HIP stream capture, tight serving loops, harnesses that
+ *      forbid hipMalloc. Same arguments, kernels and results as rmx_create_resize + rmx_update_resize_cmn + rmx_op_launch
+ *      (padded source tensor, no colour node in the chain: flags may hold RMX_F_QUANTIZE_U8 and RMX_F_EDGE_REF). The
+ *      per-batch parameter table lives in a static device array of RMX_NOALLOC_MAX_SAMPLES rows (64 KiB on every GPU the
+ *      library runs on, held until the process ends) and is written by small kernels that carry the rows as arguments, so
+ *      the call makes no hipMalloc / hipFree / hipHostMalloc and no memory copy. A batch of more samples is refused.
+ *      All calls on one GPU share that array: calls that overlap (two streams, two threads) race; calls on one stream
+ *      are ordered by it. Asynchronous on the context's stream. ---- */
+#define RMX_NOALLOC_MAX_SAMPLES 512
+RMX_API int rmx_resize_cmn_noalloc(rmx_ctx *ctx, const rmx_tensor_desc *src_desc, const rmx_tensor_desc *dst_desc, int interpolation,
+                                   int roi_type, uint32_t flags, const void *src, void *dst, const uint32_t *src_roi /*[N][4]*/,
+                                   const uint32_t *dst_w /*[N]*/, const uint32_t *dst_h /*[N]*/, const uint32_t *crop_roi /*[N][4] or NULL*/,
+                                   const float *scale /*[N*C]*/, const float *bias /*[N*C]*/, const uint32_t *mirror /*[N] or NULL*/);
+
 /* ---- Colour family (u8 NHWC -> u8 NHWC): replaces vxExtRppColorTwist (node_color_twist.cpp:48-49),
  *      vxExtRppBrightness (node_brightness.cpp:44), vxExtRppContrast (node_contrast.cpp:44),
  *      vxExtRppHue (node_hue.cpp:42), vxExtRppSaturation (node_saturation.cpp:42). ---- */

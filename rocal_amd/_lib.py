@@ -74,6 +74,7 @@ _SIGS = {
     "rmx_create_to_tensor": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.POINTER(_vp)],
     "rmx_update_to_tensor": [_vp, _vp, _vp, C.c_int],
     "rmx_copy_bytes": [_vp, _vp, _vp, C.c_size_t],
+    "rmx_resize_cmn_noalloc": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
 }
 _RESTYPES = {"rmx_last_error": C.c_char_p, "rmx_version": C.c_char_p, "rmx_ctx_stream": _vp,
              "rmx_op_algorithmic_bytes": C.c_uint64, "rmx_op_kernel_name": C.c_char_p, "rmx_op_plan": C.c_char_p}

@@ -45,7 +45,26 @@ constexpr int TABLE_RING = 4;  // updates in flight before the host has to wait 
 
 }  // namespace
 
+// ---- parameter table of the entry point that allocates nothing (rmx_resize_cmn_noalloc) ----
+// Every GPU the library runs on holds its own copy of this array until the process ends. In host code the array's name is
+// only a stand-in: its device address is asked for once per device (rmx_ctx_create) and kept in the context.
+constexpr int RMX_NOALLOC_ROWS = RMX_NOALLOC_MAX_SAMPLES;
+static __device__ __align__(256) unsigned char scratch[(size_t)RMX_NOALLOC_ROWS * sizeof(RmxSample)];
+
+// The rows travel as kernel arguments (16 rows = 2 KB per launch): no staging buffer, no copy from host memory, nothing
+// that a stream capture could not record.
+struct RmxRowPack {
+    RmxSample rows[16];
+};
+__global__ void __launch_bounds__(512) rmx_table_fill_kernel(RmxRowPack pack, RmxSample *table, int first, int count) {
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(pack.rows);
+    uint32_t *dst = reinterpret_cast<uint32_t *>(table + first);
+    const int words = count * (int)(sizeof(RmxSample) / 4);
+    for (int i = threadIdx.x; i < words; i += blockDim.x) dst[i] = src[i];
+}
+
 struct rmx_ctx {
+    void *scratch_ptr = nullptr;  // device address of `scratch` on this context's device
     int device = 0;
     hipStream_t stream = nullptr;
     bool owns_stream = false;
@@ -238,6 +257,15 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         }
         ctx->owns_stream = true;
     }
+    {
+        // device address of the static parameter table of rmx_resize_cmn_noalloc, with this device current
+        hipError_t e = hipGetSymbolAddress(&ctx->scratch_ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ctx->scratch_ptr) {
+            if (ctx->owns_stream) (void)hipStreamDestroy(ctx->stream);
+            delete ctx;
+            return fail(RMX_ERR_HIP, "hipGetSymbolAddress(scratch) failed: %d (%s)", (int)e, hipGetErrorString(e));
+        }
+    }
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, device) == hipSuccess) {
         ctx->num_cus = prop.multiProcessorCount;
@@ -322,17 +350,29 @@ static int static_lds_of(rmx_op *op, rmx::KernelFn fn) {
     return op->lds_static[slot];
 }
 
+// Enqueues the op's kernel with the given device table (and, for ragged sources, its layout entries).
+static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *layout, const uint8_t *extra, uint64_t ragged_bytes,
+                        const void *src, const void *src2, void *dst);
+
 static int launch_impl(rmx_op *op, const void *src, const void *src2, void *dst) {
-    if (!src || !dst) return fail(RMX_ERR_INVALID, "source/destination buffer is NULL");
     if (op->cur < 0 || !op->fn) return fail(RMX_ERR_INVALID, "op launched before its first update");
+    const bool ragged = op->slot_ragged[op->cur];
+    return launch_table(op, op->d_table[op->cur], ragged ? reinterpret_cast<const RmxSrcLayout *>(op->d_table[op->cur] + op->n) : nullptr,
+                        op->extra_per_sample ? slot_extra(op, op->d_table[op->cur]) : nullptr, ragged ? op->slot_src_bytes[op->cur] : 0, src, src2, dst);
+}
+
+static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *layout, const uint8_t *extra, uint64_t ragged_bytes,
+                        const void *src, const void *src2, void *dst) {
+    if (!src || !dst) return fail(RMX_ERR_INVALID, "source/destination buffer is NULL");
+    if (!op->fn) return fail(RMX_ERR_INVALID, "op launched before its first update");
     RmxKArgs a{};
     a.src = (const uint8_t *)src;
     a.src2 = (const uint8_t *)src2;
-    a.extra = op->extra_per_sample ? slot_extra(op, op->d_table[op->cur]) : nullptr;
+    a.extra = extra;
     a.dst = dst;
-    a.table = op->d_table[op->cur];
-    a.src_bytes = op->slot_ragged[op->cur] ? op->slot_src_bytes[op->cur] : (uint64_t)op->src.n * op->src.h * op->src.w * op->src.c;
-    a.layout = op->slot_ragged[op->cur] ? reinterpret_cast<const RmxSrcLayout *>(op->d_table[op->cur] + op->n) : nullptr;
+    a.table = table;
+    a.src_bytes = layout ? ragged_bytes : (uint64_t)op->src.n * op->src.h * op->src.w * op->src.c;
+    a.layout = layout;
     a.n = op->n;
     a.src_h = (int)op->src.h;
     a.src_w = (int)op->src.w;
@@ -788,9 +828,9 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             // wavefronts per CU, which 10 KB each still fit
             const int bufcap = std::min(op->ctx->dma_lds, 10 * 1024);  // the kernel issues at most 10 loads of 1 KB per window
             int need_max = 64;
-            std::vector<int32_t> tws((size_t)op->n, 8);
             for (int i = 0; i < op->n && dma; i++) {
-                const RmxSample &s = t[i];
+                RmxSample &s = t[i];
+                s.plan[1] = 8;
                 if (s.dst_w <= 0 || s.dst_h <= 0) continue;
                 const float magx = (float)(s.src_x + s.src_w + 2), magy = (float)(s.src_y + s.src_h + 2);
                 const int nrows = std::max(2, span_bound(std::min<int>(rows, s.dst_h) - 1, s.ry, magy) + 2);
@@ -799,7 +839,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                     const int nc = std::min<int>(s.src_w, span_bound(tw - 1, s.rx, magx) + 2);
                     const long need = (long)nrows * (1 + ((3 + 3 * (nc + 2) + 8 + 15) >> 4)) * 16;  // margin piece + data + replicas
                     if (need <= bufcap) {
-                        tws[(size_t)i] = tw;
+                        s.plan[1] = tw;
                         need_max = std::max<int>(need_max, (int)need);
                         break;
                     }
@@ -811,7 +851,6 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 }
             }
             if (dma && need_max <= op->ctx->max_lds_per_block - kStaticLdsMax) {
-                for (int i = 0; i < op->n; i++) t[i].plan[0] = tws[(size_t)i];
                 op->fn_fast = dfn;
                 op->fast_name = dname;
                 op->fast_lds = (need_max + 15) / 16 * 16;
@@ -827,19 +866,16 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
 
 static float hue_to_sextants(float hue_deg);
 
-static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
-                                const uint32_t *crop_roi, const float *scale, const float *bias,
-                                const float *mean, const float *stddev, const uint32_t *mirror, const float *const *colour = nullptr) {
-    if (!op || op->kind != OP_RESIZE) return fail(RMX_ERR_INVALID, "op is not a Resize node");
+// Rows and launch plan of a resize-family batch into the host table `t` (n rows); touches no device state.
+static int fill_resize_rows(rmx_op *op, RmxSample *t, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                            const uint32_t *crop_roi, const float *scale, const float *bias,
+                            const float *mean, const float *stddev, const uint32_t *mirror, const float *const *colour) {
     const uint32_t chain = op->flags & (RMX_F_COLOR_LINEAR | RMX_F_COLOR_TWIST);
     if (chain && !colour) return fail(RMX_ERR_INVALID, "this Resize node was created with a colour node in its chain: use rmx_update_resize_color_cmn");
     if (!chain && colour) return fail(RMX_ERR_INVALID, "this Resize node was created without a colour node in its chain");
     if (!dst_w || !dst_h) return fail(RMX_ERR_INVALID, "dst_w and dst_h arrays are required");
     if ((mean == nullptr) != (stddev == nullptr)) return fail(RMX_ERR_INVALID, "mean and stddev must be given together");
     if ((scale == nullptr) != (bias == nullptr)) return fail(RMX_ERR_INVALID, "scale and bias must be given together");
-    RmxSample *t;
-    int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
     uint64_t bytes = 0;
     const bool edge_ref = (op->flags & RMX_F_EDGE_REF) && op->interp == RMX_INTERP_LINEAR;
     for (int i = 0; i < op->n; i++) {
@@ -904,7 +940,17 @@ static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint3
                  (uint64_t)s.dst_w * s.dst_h * 3 * dtype_size(op->dst.dtype);
     }
     op->algo_bytes = bytes;
-    int rc = plan_resize(op, t, scale != nullptr || mean != nullptr);
+    return plan_resize(op, t, scale != nullptr || mean != nullptr);
+}
+
+static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                                const uint32_t *crop_roi, const float *scale, const float *bias,
+                                const float *mean, const float *stddev, const uint32_t *mirror, const float *const *colour = nullptr) {
+    if (!op || op->kind != OP_RESIZE) return fail(RMX_ERR_INVALID, "op is not a Resize node");
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    int rc = fill_resize_rows(op, t, src_roi, dst_w, dst_h, crop_roi, scale, bias, mean, stddev, mirror, colour);
     if (rc) return rc;
     return commit_slot(op, slot);
 }
@@ -1223,6 +1269,51 @@ int rmx_update_rotate(rmx_op *op, const uint32_t *src_roi, const float *angle_de
     if (!op || op->kind != OP_ROTATE) return fail(RMX_ERR_INVALID, "op is not a Rotate node");
     if (!angle_deg) return fail(RMX_ERR_INVALID, "angle array is required");
     return update_warp(op, src_roi, nullptr, angle_deg, dst_w, dst_h);
+}
+
+/* ------------------------------------------------------------------ one entry point that allocates nothing */
+
+int rmx_resize_cmn_noalloc(rmx_ctx *ctx, const rmx_tensor_desc *src_desc, const rmx_tensor_desc *dst_desc, int interpolation, int roi_type,
+                           uint32_t flags, const void *src, void *dst, const uint32_t *src_roi, const uint32_t *dst_w, const uint32_t *dst_h,
+                           const uint32_t *crop_roi, const float *scale, const float *bias, const uint32_t *mirror) {
+    if (!ctx) return fail(RMX_ERR_INVALID, "context is NULL");
+    int rc;
+    if ((rc = check_desc(src_desc, "source"))) return rc;
+    if ((rc = check_desc(dst_desc, "destination"))) return rc;
+    if (src_desc->dtype != RMX_UINT8 || src_desc->layout != RMX_NHWC) return fail(RMX_ERR_UNSUPPORTED, "source must be uint8 NHWC (decoded RGB batch)");
+    if (src_desc->n != dst_desc->n) return fail(RMX_ERR_INVALID, "batch size mismatch: source %u, destination %u", src_desc->n, dst_desc->n);
+    if (src_desc->n > (uint32_t)RMX_NOALLOC_ROWS)
+        return fail(RMX_ERR_INVALID, "batch of %u samples exceeds the %d rows of the static parameter table (RMX_NOALLOC_MAX_SAMPLES)", src_desc->n, RMX_NOALLOC_ROWS);
+    if (roi_type != RMX_ROI_LTRB && roi_type != RMX_ROI_XYWH) return fail(RMX_ERR_INVALID, "roi_type %d invalid", roi_type);
+    if (interpolation != RMX_INTERP_LINEAR && interpolation != RMX_INTERP_NEAREST && interpolation != RMX_INTERP_TRIANGULAR)
+        return fail(RMX_ERR_UNSUPPORTED, "interpolation %d is outside the hot path (nearest=0, linear=1, triangular=5)", interpolation);
+    if (flags & ~(uint32_t)(RMX_F_QUANTIZE_U8 | RMX_F_EDGE_REF)) return fail(RMX_ERR_UNSUPPORTED, "only RMX_F_QUANTIZE_U8 and RMX_F_EDGE_REF are supported here");
+    if (!scale || !bias) return fail(RMX_ERR_INVALID, "scale and bias arrays are required");
+    if (!ctx->scratch_ptr) return fail(RMX_ERR_INVALID, "the context holds no address of the static parameter table");
+    HIP_TRY(hipSetDevice(ctx->device));
+    // an op that lives on this call's stack: same packing, same planner, same kernels as rmx_create_resize + rmx_update_resize_cmn
+    rmx_op op;
+    op.ctx = ctx;
+    op.kind = OP_RESIZE;
+    op.src = *src_desc;
+    op.dst = *dst_desc;
+    op.roi_type = roi_type;
+    op.n = (int)src_desc->n;
+    op.interp = interpolation;
+    op.flags = flags;
+    RmxSample rows[RMX_NOALLOC_ROWS];  // host side of the table, on this call's stack (64 KiB)
+    memset(rows, 0, sizeof(RmxSample) * (size_t)op.n);
+    rc = fill_resize_rows(&op, rows, src_roi, dst_w, dst_h, crop_roi, scale, bias, nullptr, nullptr, mirror, nullptr);
+    if (rc) return rc;
+    RmxSample *table = static_cast<RmxSample *>(ctx->scratch_ptr);  // the address asked of the runtime, never the array's name
+    for (int first = 0; first < op.n; first += 16) {
+        RmxRowPack pack;
+        const int count = std::min(16, op.n - first);
+        memcpy(pack.rows, rows + first, sizeof(RmxSample) * (size_t)count);
+        hipLaunchKernelGGL(rmx_table_fill_kernel, dim3(1), dim3(512), 0, ctx->stream, pack, table, first, count);
+        HIP_TRY(hipGetLastError());
+    }
+    return launch_table(&op, table, nullptr, nullptr, 0, src, nullptr, dst);
 }
 
 /* ------------------------------------------------------------------ measurement helper */

@@ -21,7 +21,7 @@ struct __attribute__((aligned(16))) RmxSample {
     float scale[3], bias[3];             // normalisation: out = v*scale + bias
     union {
         float color[4];                  // colour twist: alpha, beta, hue shift in sextants [0,6], saturation
-        int32_t plan[4];                 // resize fast path: [0] = x-tile width for this sample
+        int32_t plan[4];                 // bilinear fast paths: x-tile width for this sample, [0] staged kernel, [1] streaming kernel
     };
     float m[6];                          // warp: destination -> source affine about the centres
 };

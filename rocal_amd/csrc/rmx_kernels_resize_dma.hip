@@ -73,7 +73,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     const int s = (int)(wave / (uint32_t)a.strips);
     const int grp = (int)(wave % (uint32_t)a.strips);
     const RmxSample P = a.table[s];
-    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.plan[0]));
+    asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.plan[1]));
 
     const int dw = P.dst_w, dh = P.dst_h;
     const int srows = a.aux0;
@@ -111,7 +111,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     const uint64_t left = (uint64_t)((a.src + a.src_bytes) - base4);
     const uint32_t lim = left > 0xffffffffull ? 0xffffffffu : (uint32_t)left;
 
-    const int tile_w = max(P.plan[0], PX);
+    const int tile_w = max(P.plan[1], PX);  // never 0: it is the step of the tile loop
     const int ntx = (dw + tile_w - 1) / tile_w;
 
     auto make_item = [&](int tile) {

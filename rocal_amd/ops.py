@@ -79,6 +79,22 @@ def desc(n, h, w, layout, dtype, c=3):
     return TensorDesc(n, h, w, c, layout, dtype)
 
 
+NOALLOC_MAX_SAMPLES = 512  # RMX_NOALLOC_MAX_SAMPLES
+
+
+def resize_cmn_noalloc(ctx, src_desc, dst_desc, src, dst, src_roi, dst_w, dst_h, scale, bias, mirror=None, crop_roi=None,
+                       interpolation=LINEAR, flags=0, roi_type=ROI_XYWH):
+    """rmx_resize_cmn_noalloc: the fused chain resize -> CropMirrorNormalize in one call that allocates nothing (the parameter
+    table lives in a static device array). src / dst: torch CUDA tensors, the arrays are host arrays."""
+    assert src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()
+    assert src.numel() * src.element_size() >= src_desc.n * src_desc.h * src_desc.w * src_desc.c
+    esz = {FP32: 4, FP16: 2, UINT8: 1}[dst_desc.dtype]
+    assert dst.numel() * dst.element_size() >= dst_desc.n * dst_desc.h * dst_desc.w * dst_desc.c * esz
+    keep = [_arr(a, dt) for a, dt in ((src_roi, _U), (dst_w, _U), (dst_h, _U), (crop_roi, _U), (scale, _F), (bias, _F), (mirror, _U))]
+    check(_lib.lib().rmx_resize_cmn_noalloc(ctx._h, C.byref(src_desc), C.byref(dst_desc), int(interpolation), int(roi_type), C.c_uint32(flags),
+                                            C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), *[p for _, p in keep]))
+
+
 class Op:
     """One node (rmx_op). Subclasses bind create/update of a specific reference node."""
 
