@@ -63,7 +63,15 @@ __global__ void __launch_bounds__(512) rmx_table_fill_kernel(RmxRowPack pack, Rm
     for (int i = threadIdx.x; i < words; i += blockDim.x) dst[i] = src[i];
 }
 
+// Copies a freshly packed parameter table from the pinned host ring to its device slot: 16 bytes per lane, read across
+// the host link by the GPU itself. For the 4-40 KB of a table this reaches the device sooner than a copy-engine transfer
+// queued on the same stream.
+__global__ void __launch_bounds__(256) rmx_table_upload_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int n16) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += gridDim.x * blockDim.x) dst[i] = src[i];
+}
+
 struct rmx_ctx {
+    int upload_kernel = 1;        // 1: tables are uploaded by rmx_table_upload_kernel, 0: by hipMemcpyAsync
     void *scratch_ptr = nullptr;  // device address of `scratch` on this context's device
     int device = 0;
     hipStream_t stream = nullptr;
@@ -185,7 +193,14 @@ int commit_slot(rmx_op *op, int slot) {
         bytes = (sizeof(RmxSample) + sizeof(RmxSrcLayout) + op->extra_per_sample) * (size_t)op->n;
     op->slot_ragged[slot] = !op->layout.empty();
     op->slot_src_bytes[slot] = op->ragged_bytes;
-    HIP_TRY(hipMemcpyAsync(op->d_table[slot], op->h_table[slot], bytes, hipMemcpyHostToDevice, op->ctx->stream));
+    if (op->ctx->upload_kernel) {
+        const int n16 = (int)((bytes + 15) / 16);  // (the slots are allocated in whole rows of 128 bytes and 16-byte entries)
+        hipLaunchKernelGGL(rmx_table_upload_kernel, dim3((unsigned)std::min(8, (n16 + 255) / 256)), dim3(256), 0, op->ctx->stream,
+                           reinterpret_cast<const uint4 *>(op->h_table[slot]), reinterpret_cast<uint4 *>(op->d_table[slot]), n16);
+        HIP_TRY(hipGetLastError());
+    } else {
+        HIP_TRY(hipMemcpyAsync(op->d_table[slot], op->h_table[slot], bytes, hipMemcpyHostToDevice, op->ctx->stream));
+    }
     HIP_TRY(hipEventRecord(op->uploaded[slot], op->ctx->stream));
     op->cur = slot;
     return RMX_OK;
@@ -277,6 +292,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->fast_rows = tune_env("RMX_TUNE_FAST_ROWS", ctx->fast_rows, 1, 64);
         ctx->fast_lds = tune_env("RMX_TUNE_FAST_LDS", ctx->fast_lds, 2048, 48 * 1024);
         ctx->fast_wpb = tune_env("RMX_TUNE_FAST_WPB", ctx->fast_wpb, 1, 4);
+        ctx->upload_kernel = tune_env("RMX_TUNE_UPLOAD_KERNEL", ctx->upload_kernel, 0, 1);
         ctx->dma = tune_env("RMX_TUNE_DMA", ctx->dma, 0, 1);  // 0: the bilinear fast path always stages through registers
         ctx->dma_lds = tune_env("RMX_TUNE_DMA_LDS", ctx->dma_lds, 2048, 10 * 1024) & ~15;  // LDS window of a wavefront
         ctx->tri_wpb = tune_env("RMX_TUNE_TRI_WPB", ctx->tri_wpb, 1, 4);

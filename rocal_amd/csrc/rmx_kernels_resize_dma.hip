@@ -42,7 +42,6 @@ RMX_DEV float src_coord_d(int u, float ratio, float off, float lo) {
     return s;
 }
 
-constexpr int DMA_SLOTS = 10;  // load instructions per window at most: 10 x 64 pieces of 16 bytes = 10 KB
 
 // One window: a strip of destination rows x one x-tile. Every member is wave-uniform.
 struct DmaItem {
@@ -54,7 +53,6 @@ struct DmaItem {
     int ppr;         // 16-byte pieces per LDS row (margin + data + room for the right replicas)
     int nd;          // data pieces per row
     uint32_t col4;   // byte offset (from base4) of the dword that holds pixel cs, within a row
-    int ns;          // load instructions
     bool rep_l, rep_r, safe;
 };
 
@@ -120,11 +118,13 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         g.r1 = r_end;
         g.xt = tile * tile_w;
         g.tw = min(dw - g.xt, tile_w);
-        g.a_v = (int)floorf(src_coord_d(pcy + g.r0, ry, offy, fylo));
-        const int b_v = (int)floorf(src_coord_d(pcy + g.r1 - 1, ry, offy, fylo)) + 1;
+        // (wave-uniform values that come out of the vector unit's float arithmetic: into scalar registers, so that everything
+        // derived from them is scalar arithmetic)
+        g.a_v = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcy + g.r0, ry, offy, fylo)));
+        const int b_v = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcy + g.r1 - 1, ry, offy, fylo))) + 1;
         g.nrows = b_v - g.a_v + 1;
-        const int ixmin = (int)floorf(src_coord_d(pcx + g.xt, rx, offx, fxlo));
-        const int ixmax = (int)floorf(src_coord_d(pcx + g.xt + g.tw - 1, rx, offx, fxlo));
+        const int ixmin = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcx + g.xt, rx, offx, fxlo)));
+        const int ixmax = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcx + g.xt + g.tw - 1, rx, offx, fxlo)));
         g.cs = max(min(ixmin, xhi), xlo);
         const int ce = max(min(ixmax + 1, xhi), xlo);
         g.nc = ce - g.cs + 1;
@@ -136,7 +136,6 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         g.nd = (g.ph + 3 * g.nc + 15) >> 4;
         g.ppr = 1 + ((g.ph + 3 * (g.nc + 2) + 8 + 15) >> 4);
         const int tp = g.nrows * g.ppr;
-        g.ns = (tp + RMX_WAVE - 1) / RMX_WAVE;
         // every 16-byte piece of every row lies inside the batch buffer (the last rows of the last sample may not)
         const uint32_t last_row = (uint32_t)max(min(b_v, yhi), ylo) * row_stride + g.col4;
         g.safe = (uint64_t)last_row + 16ull * (uint64_t)g.nd <= (uint64_t)lim;
@@ -148,19 +147,17 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     // written over it).
     auto issue = [&](DmaItem &g, uint32_t *buf) {
         const int tp = g.nrows * g.ppr;
-        const float inv_ppr = 1.0f / (float)g.ppr;
         if (g.safe) {
-#pragma unroll
-            for (int j = 0; j < DMA_SLOTS; j++) {
-                if (j < g.ns) {
-                    const int idx = j * RMX_WAVE + lane;
-                    if (idx < tp) {
-                        const int r = (int)(((float)idx + 0.5f) * inv_ppr);  // idx / ppr, exact: idx < 2^16
-                        const int c = idx - __mul24(r, g.ppr);
+            // One load instruction per row and 64 pieces: the row's address is scalar arithmetic, a lane's piece offset is the
+            // same for every row, and consecutive lanes fill consecutive 16-byte slots from (r * ppr + c0) on.
+            for (int c0 = 0; c0 < g.ppr; c0 += RMX_WAVE) {
+                const int c = c0 + lane;
+                const uint32_t lane_off = 16u * (uint32_t)max(min(c - 1, g.nd - 1), 0);
+                if (c < g.ppr) {
+                    for (int r = 0; r < g.nrows; r++) {
                         const int ysrc = max(min(g.a_v + r, yhi), ylo);
-                        const int piece = max(min(c - 1, g.nd - 1), 0);
-                        const uint32_t off = (uint32_t)__mul24(ysrc, (int)row_stride) + g.col4 + 16u * (uint32_t)piece;
-                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(base4 + off), (lds_ptr_t)(buf + j * (RMX_WAVE * 4)), 16, 0, 0);
+                        const uint8_t *rowp = base4 + ((uint32_t)ysrc * row_stride + g.col4);
+                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(buf + (r * g.ppr + c0) * 4), 16, 0, 0);
                     }
                 }
             }
@@ -186,7 +183,6 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                 lds_u32 *dst4 = (lds_u32 *)(lds_ptr_t)(buf + 4 * idx);
                 dst4[0] = w[0]; dst4[1] = w[1]; dst4[2] = w[2]; dst4[3] = w[3];
             }
-            g.ns = 0;
         }
     };
 
