@@ -1,0 +1,247 @@
+// rocal_api_mi355x.h - public host API of the MI355X augmentation hot path: the rocAL C API entry points of the hot-path
+// operators with the reference's names, argument order, defaults and error behaviour (rocAL/include/api/rocal_api.h:83-110,
+// rocal_api_parameters.h:39-161, rocal_api_augmentation.h, rocal_api_info.h:106, rocal_api_data_transfer.h:45-66), so that a
+// program written against rocAL's headers for these operators compiles against this one and links with
+// librocal_mi355x_host.so. Like the reference's, these are extern "C" names with C++ types (std::vector, default arguments).
+// This header is self-contained: it includes nothing of the library's internals.
+//
+// Loaders, decoders and the output ring buffer are not part of the hot path. Where the reference would create a source
+// with a reader + decoder, this API takes decoded batches that already sit in device memory:
+//   rocalDeviceSource()      declares the input tensor (u8 RGB, NHWC, padded to max_height x max_width)
+//   rocalDeviceSourceFeed()  hands the next batch: device pointer + per-sample width/height
+// and an output is read through rocalTensorBuffer() / rocalTensorRoi(), or written straight into memory the caller owns
+// (rocalTensorSetBuffer, e.g. the data pointer of a torch tensor).
+#ifndef ROCAL_API_MI355X_H
+#define ROCAL_API_MI355X_H
+#include <cstddef>
+#include <vector>
+
+// rocAL/include/api/rocal_api_types.h:326-366
+enum RocalResizeScalingMode {
+    ROCAL_SCALING_MODE_DEFAULT = 0,
+    ROCAL_SCALING_MODE_STRETCH = 1,
+    ROCAL_SCALING_MODE_NOT_SMALLER = 2,
+    ROCAL_SCALING_MODE_NOT_LARGER = 3,
+    ROCAL_SCALING_MODE_MIN_MAX = 4
+};
+enum RocalResizeInterpolationType {
+    ROCAL_NEAREST_NEIGHBOR_INTERPOLATION = 0,
+    ROCAL_LINEAR_INTERPOLATION = 1,
+    ROCAL_CUBIC_INTERPOLATION = 2,
+    ROCAL_LANCZOS_INTERPOLATION = 3,
+    ROCAL_GAUSSIAN_INTERPOLATION = 4,
+    ROCAL_TRIANGULAR_INTERPOLATION = 5
+};
+
+#define ROCAL_API_CALL __attribute__((visibility("default")))
+
+typedef void *RocalContext;
+typedef void *RocalTensor;
+typedef void *RocalFloatParam;
+typedef void *RocalIntParam;
+
+// rocAL/include/api/rocal_api_types.h:112-128,151-158,208-268
+enum RocalStatus { ROCAL_OK = 0, ROCAL_CONTEXT_INVALID, ROCAL_RUNTIME_ERROR, ROCAL_UPDATE_PARAMETER_FAILED, ROCAL_INVALID_PARAMETER_TYPE };
+enum RocalProcessMode { ROCAL_PROCESS_GPU = 0, ROCAL_PROCESS_CPU = 1 };
+enum RocalTensorLayout { ROCAL_NHWC = 0, ROCAL_NCHW = 1, ROCAL_NONE = 9 };
+enum RocalTensorOutputType { ROCAL_FP32 = 0, ROCAL_FP16 = 1, ROCAL_UINT8 = 2 };
+enum RocalOutputMemType { ROCAL_MEMCPY_HOST = 0, ROCAL_MEMCPY_GPU = 1, ROCAL_MEMCPY_PINNED = 2 };
+
+/* ---- context (rocal_api.h:83-110). Only ROCAL_PROCESS_GPU exists: there is no CPU path. ---- */
+extern "C" RocalContext ROCAL_API_CALL rocalCreate(size_t batch_size, RocalProcessMode affinity, int gpu_id = 0, size_t cpu_thread_count = 1,
+                                                   size_t prefetch_queue_depth = 3, RocalTensorOutputType output_tensor_data_type = ROCAL_FP32);
+extern "C" RocalStatus ROCAL_API_CALL rocalVerify(RocalContext context);
+extern "C" RocalStatus ROCAL_API_CALL rocalRun(RocalContext context);
+extern "C" RocalStatus ROCAL_API_CALL rocalRelease(RocalContext context);
+extern "C" const char *ROCAL_API_CALL rocalGetErrorMessage(RocalContext context);
+
+/* ---- timing (rocal_api_info.h:106, rocal_api_types.h:79-84): microseconds accumulated since the last call, which resets them.
+   process_time brackets Graph::process() as the reference's does (master_graph.cpp:1015-1017): the launches of a batch and the
+   wait for them; transfer_time is the time spent in rocalToTensor; load and decode time belong to the loaders and stay 0.
+   rocalGetParameterUpdateTime (no counterpart in the reference) gives the time of the per-batch parameter renewal and node updates
+   that run before process() on the same thread (master_graph.cpp:408,1010-1013). ---- */
+struct TimingInfo {
+    long long unsigned load_time;
+    long long unsigned decode_time;
+    long long unsigned process_time;
+    long long unsigned transfer_time;
+};
+extern "C" TimingInfo ROCAL_API_CALL rocalGetTimingInfo(RocalContext rocal_context);
+extern "C" long long unsigned ROCAL_API_CALL rocalGetParameterUpdateTime(RocalContext rocal_context);
+
+/* ---- decoded batches in device memory (stands where the reference's loader modules stand) ---- */
+extern "C" RocalTensor ROCAL_API_CALL rocalDeviceSource(RocalContext context, unsigned max_width, unsigned max_height, bool is_output);
+extern "C" RocalStatus ROCAL_API_CALL rocalDeviceSourceFeed(RocalContext context, RocalTensor source, const void *device_ptr, const unsigned *roi_width,
+                                                            const unsigned *roi_height);
+extern "C" void *ROCAL_API_CALL rocalTensorBuffer(RocalTensor tensor);
+// Binds an output tensor to device memory the caller owns (at least rocalTensorDataSize bytes, 16-byte aligned), before or
+// after rocalVerify and as often as wanted between runs: the node that produces the tensor writes there directly. Stands where
+// the reference copies a finished output into the framework's tensor (rocalTensor::copy_data, rocAL/source/pipeline/tensor.cpp:419-454,
+// called from rocAL_pybind/amd/rocal/plugin/pytorch.py:118-135).
+extern "C" RocalStatus ROCAL_API_CALL rocalTensorSetBuffer(RocalContext context, RocalTensor tensor, void *device_ptr);
+// x,y,w,h per sample
+extern "C" const unsigned *ROCAL_API_CALL rocalTensorRoi(RocalTensor tensor);
+extern "C" size_t ROCAL_API_CALL rocalTensorDataSize(RocalTensor tensor);
+
+/* ---- u8 output -> float tensor (rocal_api_data_transfer.h:45-66). out_ptr is device memory: only ROCAL_MEMCPY_GPU exists. ---- */
+extern "C" RocalStatus ROCAL_API_CALL rocalToTensor(RocalContext rocal_context, void *out_ptr, RocalTensorLayout tensor_format,
+                                                    RocalTensorOutputType tensor_output_type, float multiplier0, float multiplier1, float multiplier2,
+                                                    float offset0, float offset1, float offset2, bool reverse_channels,
+                                                    RocalOutputMemType output_mem_type, int max_roi_height = 0, int max_roi_width = 0);
+
+/* ---- bounding boxes (rocal_api_meta_data.h). Metadata readers are outside the hot path: rocalEnableBoundingBoxes() stands
+   where rocalCreateCOCOReader() & co. stand (before the augmentations are added); the boxes of a batch (l,t,r,b in pixels
+   of the decoded image, `counts[i]` per sample, all samples back to back) are handed in before rocalRun() and the
+   transformed ones are read back after it, in the same layout. ---- */
+extern "C" RocalStatus ROCAL_API_CALL rocalEnableBoundingBoxes(RocalContext context);
+extern "C" RocalStatus ROCAL_API_CALL rocalSetBoundingBoxes(RocalContext context, const unsigned *counts, const float *ltrb, const int *labels);
+extern "C" unsigned ROCAL_API_CALL rocalGetBoundingBoxCount(RocalContext context, unsigned *counts);  // returns the total
+extern "C" RocalStatus ROCAL_API_CALL rocalGetBoundingBoxCords(RocalContext context, float *ltrb);
+extern "C" RocalStatus ROCAL_API_CALL rocalGetBoundingBoxLabel(RocalContext context, int *labels);
+
+/* ---- parameters (rocal_api_parameters.h:39-161) ---- */
+extern "C" void ROCAL_API_CALL rocalSetSeed(unsigned seed);
+extern "C" unsigned ROCAL_API_CALL rocalGetSeed();
+extern "C" RocalIntParam ROCAL_API_CALL rocalCreateIntUniformRand(int start, int end);
+extern "C" RocalStatus ROCAL_API_CALL rocalUpdateIntUniformRand(int start, int end, RocalIntParam updating_obj);
+extern "C" int ROCAL_API_CALL rocalGetIntValue(RocalIntParam obj);
+extern "C" float ROCAL_API_CALL rocalGetFloatValue(RocalFloatParam obj);
+extern "C" RocalFloatParam ROCAL_API_CALL rocalCreateFloatUniformRand(float start, float end);
+extern "C" RocalFloatParam ROCAL_API_CALL rocalCreateFloatParameter(float val);
+extern "C" RocalIntParam ROCAL_API_CALL rocalCreateIntParameter(int val);
+extern "C" RocalStatus ROCAL_API_CALL rocalUpdateFloatParameter(float new_val, RocalFloatParam input_obj);
+extern "C" RocalStatus ROCAL_API_CALL rocalUpdateIntParameter(int new_val, RocalIntParam input_obj);
+extern "C" RocalStatus ROCAL_API_CALL rocalUpdateFloatUniformRand(float start, float end, RocalFloatParam updating_obj);
+extern "C" RocalIntParam ROCAL_API_CALL rocalCreateIntRand(const int *values, const double *frequencies, unsigned size);
+extern "C" RocalStatus ROCAL_API_CALL rocalUpdateIntRand(const int *values, const double *frequencies, unsigned size, RocalIntParam updating_obj);
+extern "C" RocalFloatParam ROCAL_API_CALL rocalCreateFloatRand(const float *values, const double *frequencies, unsigned size);
+extern "C" RocalStatus ROCAL_API_CALL rocalUpdateFloatRand(const float *values, const double *frequencies, unsigned size, RocalFloatParam updating_obj);
+
+/* ---- augmentations (rocal_api_augmentation.h; line of each declaration given) ---- */
+extern "C" RocalTensor ROCAL_API_CALL rocalResize(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height, bool is_output,
+                                                  RocalResizeScalingMode scaling_mode = ROCAL_SCALING_MODE_STRETCH, std::vector<unsigned> max_size = {},
+                                                  unsigned resize_shorter = 0, unsigned resize_longer = 0,
+                                                  RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                  RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :67
+extern "C" RocalTensor ROCAL_API_CALL rocalResizeMirrorNormalize(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height,
+                                                                 std::vector<float> &mean, std::vector<float> &std_dev, bool is_output,
+                                                                 RocalResizeScalingMode scaling_mode = ROCAL_SCALING_MODE_STRETCH,
+                                                                 std::vector<unsigned> max_size = {}, unsigned resize_shorter = 0, unsigned resize_longer = 0,
+                                                                 RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                                 RocalIntParam mirror = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                                 RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :98
+extern "C" RocalTensor ROCAL_API_CALL rocalCropResize(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height, bool is_output,
+                                                      RocalFloatParam area = NULL, RocalFloatParam aspect_ratio = NULL, RocalFloatParam x_center_drift = NULL,
+                                                      RocalFloatParam y_center_drift = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                      RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :125
+extern "C" RocalTensor ROCAL_API_CALL rocalCropResizeFixed(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height,
+                                                           bool is_output, float area, float aspect_ratio, float x_center_drift, float y_center_drift,
+                                                           RocalTensorLayout output_layout = ROCAL_NONE,
+                                                           RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :151
+extern "C" RocalTensor ROCAL_API_CALL rocalROIResize(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height, bool is_output,
+                                                     unsigned roi_h, unsigned roi_w, float roi_pos_x = 0.0f, float roi_pos_y = 0.0f,
+                                                     RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                     RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :175
+extern "C" RocalTensor ROCAL_API_CALL rocalRotate(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam angle = NULL,
+                                                  unsigned dest_width = 0, unsigned dest_height = 0,
+                                                  RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                  RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :200
+extern "C" RocalTensor ROCAL_API_CALL rocalRotateFixed(RocalContext context, RocalTensor input, float angle, bool is_output, unsigned dest_width = 0,
+                                                       unsigned dest_height = 0, RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                       RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :220
+extern "C" RocalTensor ROCAL_API_CALL rocalBrightness(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam alpha = NULL,
+                                                      RocalFloatParam beta = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                      RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :237
+extern "C" RocalTensor ROCAL_API_CALL rocalBrightnessFixed(RocalContext context, RocalTensor input, float alpha, float beta, bool is_output,
+                                                           RocalTensorLayout output_layout = ROCAL_NONE,
+                                                           RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :253
+extern "C" RocalTensor ROCAL_API_CALL rocalContrast(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam contrast_factor = NULL,
+                                                    RocalFloatParam contrast_center = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                    RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :302
+extern "C" RocalTensor ROCAL_API_CALL rocalContrastFixed(RocalContext context, RocalTensor input, float contrast_factor, float contrast_center,
+                                                         bool is_output, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                         RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :319
+extern "C" RocalTensor ROCAL_API_CALL rocalFlip(RocalContext context, RocalTensor input, bool is_output, RocalIntParam horizonal_flag = NULL,
+                                                RocalIntParam vertical_flag = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :336
+extern "C" RocalTensor ROCAL_API_CALL rocalFlipFixed(RocalContext context, RocalTensor input, int horizonal_flag, int vertical_flag, bool is_output,
+                                                     RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :352
+extern "C" RocalTensor ROCAL_API_CALL rocalWarpAffine(RocalContext context, RocalTensor input, bool is_output, unsigned dest_height = 0,
+                                                      unsigned dest_width = 0, RocalFloatParam x0 = NULL, RocalFloatParam x1 = NULL,
+                                                      RocalFloatParam y0 = NULL, RocalFloatParam y1 = NULL, RocalFloatParam o0 = NULL,
+                                                      RocalFloatParam o1 = NULL, RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                      RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :422
+extern "C" RocalTensor ROCAL_API_CALL rocalWarpAffineFixed(RocalContext context, RocalTensor input, float x0, float x1, float y0, float y1, float o0,
+                                                           float o1, bool is_output, unsigned int dest_height = 0, unsigned int dest_width = 0,
+                                                           RocalResizeInterpolationType interpolation_type = ROCAL_LINEAR_INTERPOLATION,
+                                                           RocalTensorLayout output_layout = ROCAL_NONE,
+                                                           RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :449
+extern "C" RocalTensor ROCAL_API_CALL rocalHue(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam hue = NULL,
+                                               RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :794
+extern "C" RocalTensor ROCAL_API_CALL rocalHueFixed(RocalContext context, RocalTensor input, float hue, bool is_output,
+                                                    RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :810
+extern "C" RocalTensor ROCAL_API_CALL rocalSaturation(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam saturation = NULL,
+                                                      RocalTensorLayout output_layout = ROCAL_NONE,
+                                                      RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :826
+extern "C" RocalTensor ROCAL_API_CALL rocalSaturationFixed(RocalContext context, RocalTensor input, float saturation, bool is_output,
+                                                           RocalTensorLayout output_layout = ROCAL_NONE,
+                                                           RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :842
+extern "C" RocalTensor ROCAL_API_CALL rocalColorTwist(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam alpha = NULL,
+                                                      RocalFloatParam beta = NULL, RocalFloatParam hue = NULL, RocalFloatParam sat = NULL,
+                                                      RocalTensorLayout output_layout = ROCAL_NONE,
+                                                      RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :878
+extern "C" RocalTensor ROCAL_API_CALL rocalColorTwistFixed(RocalContext context, RocalTensor input, float alpha, float beta, float hue, float sat,
+                                                           bool is_output, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                           RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :900
+extern "C" RocalTensor ROCAL_API_CALL rocalGamma(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam gamma = NULL,
+                                                 RocalTensorLayout output_layout = ROCAL_NONE,
+                                                 RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :269
+extern "C" RocalTensor ROCAL_API_CALL rocalGammaFixed(RocalContext context, RocalTensor input, float gamma, bool is_output,
+                                                      RocalTensorLayout output_layout = ROCAL_NONE,
+                                                      RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :285
+extern "C" RocalTensor ROCAL_API_CALL rocalBlend(RocalContext context, RocalTensor input1, RocalTensor input2, bool is_output,
+                                                 RocalFloatParam ratio = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                 RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :382
+extern "C" RocalTensor ROCAL_API_CALL rocalBlendFixed(RocalContext context, RocalTensor input1, RocalTensor input2, float ratio, bool is_output,
+                                                      RocalTensorLayout output_layout = ROCAL_NONE,
+                                                      RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :399
+extern "C" RocalTensor ROCAL_API_CALL rocalColorTemp(RocalContext context, RocalTensor input, bool is_output, RocalIntParam adjustment = NULL,
+                                                     RocalTensorLayout output_layout = ROCAL_NONE,
+                                                     RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :667
+extern "C" RocalTensor ROCAL_API_CALL rocalColorTempFixed(RocalContext context, RocalTensor input, int adjustment, bool is_output,
+                                                          RocalTensorLayout output_layout = ROCAL_NONE,
+                                                          RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :683
+extern "C" RocalTensor ROCAL_API_CALL rocalExposure(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam exposure_factor = NULL,
+                                                    RocalTensorLayout output_layout = ROCAL_NONE,
+                                                    RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :763
+extern "C" RocalTensor ROCAL_API_CALL rocalExposureFixed(RocalContext context, RocalTensor input, float exposure_factor, bool is_output,
+                                                         RocalTensorLayout output_layout = ROCAL_NONE,
+                                                         RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :779
+extern "C" RocalTensor ROCAL_API_CALL rocalCropMirrorNormalize(RocalContext context, RocalTensor input, unsigned crop_height, unsigned crop_width,
+                                                               float start_x, float start_y, std::vector<float> &mean, std::vector<float> &std_dev,
+                                                               bool is_output, RocalIntParam mirror = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                               RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :925
+extern "C" RocalTensor ROCAL_API_CALL rocalCrop(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam crop_width = NULL,
+                                                RocalFloatParam crop_height = NULL, RocalFloatParam crop_depth = NULL, RocalFloatParam crop_pox_x = NULL,
+                                                RocalFloatParam crop_pos_y = NULL, RocalFloatParam crop_pos_z = NULL,
+                                                RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :952
+extern "C" RocalTensor ROCAL_API_CALL rocalCropFixed(RocalContext context, RocalTensor input, unsigned crop_width, unsigned crop_height,
+                                                     unsigned crop_depth, bool is_output, float crop_pox_x, float crop_pos_y, float crop_pos_z,
+                                                     RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :977
+extern "C" RocalTensor ROCAL_API_CALL rocalCropCenterFixed(RocalContext context, RocalTensor input, unsigned crop_width, unsigned crop_height,
+                                                           unsigned crop_depth, bool is_output, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                           RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :1000
+extern "C" RocalTensor ROCAL_API_CALL rocalResizeCropMirrorFixed(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height,
+                                                                 bool is_output, unsigned crop_h, unsigned crop_w, RocalIntParam mirror,
+                                                                 RocalTensorLayout output_layout = ROCAL_NONE,
+                                                                 RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :1022
+extern "C" RocalTensor ROCAL_API_CALL rocalResizeCropMirror(RocalContext context, RocalTensor input, unsigned dest_width, unsigned dest_height,
+                                                            bool is_output, RocalFloatParam crop_height = NULL, RocalFloatParam crop_width = NULL,
+                                                            RocalIntParam mirror = NULL, RocalTensorLayout output_layout = ROCAL_NONE,
+                                                            RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :1045
+extern "C" RocalTensor ROCAL_API_CALL rocalRandomCrop(RocalContext context, RocalTensor input, bool is_output, RocalFloatParam crop_area_factor = NULL,
+                                                      RocalFloatParam crop_aspect_ratio = NULL, RocalFloatParam crop_pos_x = NULL,
+                                                      RocalFloatParam crop_pos_y = NULL, int num_of_attempts = 20,
+                                                      RocalTensorLayout output_layout = ROCAL_NONE, RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :1066
+
+#endif  // ROCAL_API_MI355X_H

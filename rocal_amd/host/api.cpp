@@ -3,6 +3,7 @@
 // input's exactly as the reference does, adds the node and calls its init(); exceptions are caught here,
 // stored in the context, printed, and turned into a null tensor / ROCAL_RUNTIME_ERROR.
 #include "rocal_host.h"
+#include "nodes.h"
 
 #include "meta.h"
 
@@ -158,6 +159,43 @@ RocalStatus rocalDeviceSourceFeed(RocalContext p_context, RocalTensor p_source, 
         return ROCAL_RUNTIME_ERROR;
     }
     return ROCAL_OK;
+}
+
+RocalStatus rocalTensorSetBuffer(RocalContext p_context, RocalTensor p_tensor, void *device_ptr) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->bind_output(static_cast<Tensor *>(p_tensor), device_ptr);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+// rocal_api_info.cpp:90-97
+TimingInfo rocalGetTimingInfo(RocalContext p_context) {
+    TimingInfo info{0, 0, 0, 0};
+    if (!p_context) return info;
+    auto *context = static_cast<Context *>(p_context);
+    unsigned long long t[3];
+    context->master_graph->take_timing(t);
+    context->update_time_us += t[0];
+    info.process_time = t[1];
+    info.transfer_time = t[2];
+    return info;
+}
+
+long long unsigned rocalGetParameterUpdateTime(RocalContext p_context) {
+    if (!p_context) return 0;
+    auto *context = static_cast<Context *>(p_context);
+    unsigned long long t[3];
+    // (the other two timers are kept for the next rocalGetTimingInfo)
+    context->master_graph->take_timing(t);
+    context->master_graph->give_back_timing(t[1], t[2]);
+    const unsigned long long r = context->update_time_us + t[0];
+    context->update_time_us = 0;
+    return r;
 }
 
 void *rocalTensorBuffer(RocalTensor t) { return t ? static_cast<Tensor *>(t)->buffer() : nullptr; }

@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "rocal_host.h"
+#include "nodes.h"  // internals exercised directly: ParameterFactory, ParameterVX, the parameter classes
 
 namespace {
 

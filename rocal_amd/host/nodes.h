@@ -8,23 +8,7 @@
 #include "crop_params.h"
 #include "parameters.h"
 #include "pipeline.h"
-
-// rocAL/include/api/rocal_api_types.h:326-366
-enum RocalResizeScalingMode {
-    ROCAL_SCALING_MODE_DEFAULT = 0,
-    ROCAL_SCALING_MODE_STRETCH = 1,
-    ROCAL_SCALING_MODE_NOT_SMALLER = 2,
-    ROCAL_SCALING_MODE_NOT_LARGER = 3,
-    ROCAL_SCALING_MODE_MIN_MAX = 4
-};
-enum RocalResizeInterpolationType {
-    ROCAL_NEAREST_NEIGHBOR_INTERPOLATION = 0,
-    ROCAL_LINEAR_INTERPOLATION = 1,
-    ROCAL_CUBIC_INTERPOLATION = 2,
-    ROCAL_LANCZOS_INTERPOLATION = 3,
-    ROCAL_GAUSSIAN_INTERPOLATION = 4,
-    ROCAL_TRIANGULAR_INTERPOLATION = 5
-};
+#include "rocal_api_mi355x.h"  // RocalResizeScalingMode, RocalResizeInterpolationType
 
 // node_crop_mirror_normalize.cpp:34-123
 class CropMirrorNormalizeNode : public Node {

@@ -1,5 +1,7 @@
 #include "pipeline.h"
 
+#include <chrono>
+
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
@@ -219,16 +221,46 @@ void MasterGraph::build() {
 }
 
 // One batch: master_graph.cpp:408 (renew), :1010-1013 (update_parameters per node), :1015-1017 (process).
+namespace {
+struct StopWatch {
+    explicit StopWatch(double &acc) : _acc(acc), _t0(std::chrono::high_resolution_clock::now()) {}
+    ~StopWatch() { _acc += std::chrono::duration<double, std::micro>(std::chrono::high_resolution_clock::now() - _t0).count(); }
+    double &_acc;
+    std::chrono::high_resolution_clock::time_point _t0;
+};
+}  // namespace
+
+void MasterGraph::take_timing(unsigned long long out[3]) {
+    for (int i = 0; i < 3; i++) {
+        out[i] = (unsigned long long)_time_us[i];
+        _time_us[i] = 0.0;
+    }
+}
+
+void MasterGraph::bind_output(Tensor *t, void *device_ptr) {
+    if (!t || !device_ptr) THROW("null tensor or buffer")
+    if (((uintptr_t)device_ptr & 15u) != 0) THROW("an output buffer must be 16-byte aligned")
+    if (t->elided) THROW("the tensor was fused away: it is never written")
+    bool produced = false;
+    for (auto &n : _nodes) produced = produced || (!n->output().empty() && n->output()[0] == t);
+    if (!produced) THROW("the tensor is not the output of a node of this context")
+    t->swap_handle(device_ptr);
+}
+
 void MasterGraph::run() {
     if (!_built) THROW("rocalVerify must be called before rocalRun")
-    ParameterFactory::instance()->renew_parameters();
-    for (auto &n : _nodes) n->update_parameters();
+    {
+        StopWatch w(_time_us[0]);
+        ParameterFactory::instance()->renew_parameters();
+        for (auto &n : _nodes) n->update_parameters();
+    }
     if (_meta_graph && _input_meta) {
         if (_input_meta->size() != _batch_size) THROW("bounding boxes were given for " + TOSTR(_input_meta->size()) + " samples, the batch has " + TOSTR(_batch_size))
         // an empty instance when nodes will fill it, a copy when no node touches the boxes
         _output_meta = _input_meta->clone(_meta_graph->_meta_nodes.empty());
         _meta_graph->process(_input_meta, _output_meta);
     }
+    StopWatch w(_time_us[1]);
     _graph->process();
 }
 
@@ -245,6 +277,7 @@ void MasterGraph::to_tensor(void *out_ptr, RocalTensorlayout format, float multi
                             float offset1, float offset2, bool reverse_channels, RocalTensorDataType output_data_type, unsigned max_roi_height,
                             unsigned max_roi_width) {
     if (!_built) THROW("rocalVerify must be called before rocalToTensor")
+    StopWatch w(_time_us[2]);
     if (_outputs.size() != 1) THROW("Cannot copy, Multiple output tensors present in the list")
     Tensor *src = _outputs[0];
     const TensorInfo &info = src->info();

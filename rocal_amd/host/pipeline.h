@@ -165,6 +165,15 @@ class MasterGraph {
     void set_input_meta_data(std::shared_ptr<MetaDataBatch> m) { _input_meta = m; }
     std::shared_ptr<MetaDataBatch> output_meta_data() { return _output_meta; }
     size_t batch_size() const { return _batch_size; }
+    // Accumulated microseconds since the last call, which resets them (TimingDbg::get_timing, include/pipeline/timing_debug.h:72-82):
+    // [0] parameter renewal + node updates, [1] Graph::process (master_graph.cpp:1015-1017), [2] to_tensor.
+    void take_timing(unsigned long long out[3]);
+    void give_back_timing(unsigned long long process_us, unsigned long long convert_us) {
+        _time_us[1] += (double)process_us;
+        _time_us[2] += (double)convert_us;
+    }
+    // an output tensor written straight into caller-owned device memory (Tensor::swap_handle, tensor.cpp:478-489)
+    void bind_output(Tensor *t, void *device_ptr);
     const std::vector<Tensor *> &outputs() const { return _outputs; }
     bool built() const { return _built; }
 
@@ -178,6 +187,7 @@ class MasterGraph {
     std::shared_ptr<BoundingBoxGraph> _meta_graph;
     std::shared_ptr<MetaDataBatch> _input_meta, _output_meta;
     bool _built = false;
+    double _time_us[3] = {0.0, 0.0, 0.0};
     // the conversion op of to_tensor(), rebuilt when the requested format changes
     rmx_op *_to_tensor_op = nullptr;
     unsigned _to_tensor_key[4] = {0, 0, 0, 0};
@@ -187,5 +197,6 @@ struct Context {
     Context(size_t batch_size, int gpu_id, void *stream) : master_graph(new MasterGraph(batch_size, gpu_id, stream)) {}
     std::unique_ptr<MasterGraph> master_graph;
     std::string error;
+    unsigned long long update_time_us = 0;  // parameter-update time read off by rocalGetTimingInfo, kept for rocalGetParameterUpdateTime
     void capture_error(const std::string &e) { error = e; }
 };

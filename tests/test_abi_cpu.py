@@ -52,3 +52,25 @@ def test_missing_library_fails_loudly(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "nope.so"))
     with pytest.raises(_lib.RmxError, match="not built"):
         _lib.lib()
+
+
+def test_public_api_header_stands_alone(tmp_path):
+    """include/rocal_api_mi355x.h compiles with include/ as the only search path of this repository, and the caller program of the GPU
+    tests names nothing outside it."""
+    import subprocess
+    src = tmp_path / "only_public.cpp"
+    src.write_text('#include "rocal_api_mi355x.h"\n#include "rocal_mi355x.h"\nint main() { TimingInfo t{}; (void)t; return rocalGetSeed() == 0u ? 0 : 1; }\n')
+    r = subprocess.run(["g++", "-std=c++17", "-fsyntax-only", "-I", os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    caller = open(os.path.join(ROOT, "tests", "cpp", "api_caller.cpp")).read()
+    includes = re.findall(r'#include\s+"([^"]+)"', caller)
+    assert includes == ["rocal_api_mi355x.h"]
+    # every rocal* entry point the public header declares is exported by the host library
+    text = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "rocal_api_mi355x.h")).read(), flags=re.S)
+    declared = sorted(set(re.findall(r"ROCAL_API_CALL\s+(rocal\w+)\s*\(", text)))
+    assert len(declared) >= 70
+    host = os.path.join(ROOT, "rocal_amd", "lib", "librocal_mi355x_host.so")
+    assert os.path.exists(host), "build the host layer first: make -C rocal_amd/host"
+    syms = subprocess.run(["nm", "-D", "--defined-only", host], capture_output=True, text=True).stdout
+    missing = [d for d in declared if (" T " + d + "\n") not in syms]
+    assert not missing, missing

@@ -127,6 +127,42 @@ def test_random_resized_crop_colour_cmn_runs_as_one_kernel(tmp_path, scenario):
         assert np.array_equal(roi[:, 2:], crop[:, 2:])
 
 
+def test_caller_built_against_the_public_header_alone(tmp_path):
+    """tests/cpp/api_caller.cpp sees include/rocal_api_mi355x.h and nothing else of this repository: CropResize -> ColorTwist ->
+    CropMirrorNormalize, two batches, the output bound to memory the caller allocated (rocalTensorSetBuffer), the timers of
+    rocalGetTimingInfo. Same expected values as the three reference nodes run one after the other."""
+    img = _image()
+    img.tofile(tmp_path / "input.bin")
+    with open(tmp_path / "meta.txt", "w") as f:
+        f.write("%d %d %d\n" % (N, H, W))
+        for w, h in ROIS:
+            f.write("%d %d\n" % (w, h))
+    exe = os.path.join(ROOT, "rocal_amd", "lib", "api_caller")
+    print("api_caller", flush=True)
+    p = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, (p.returncode, p.stdout, p.stderr)
+    assert "intermediates_elided 1" in p.stdout and p.stdout.strip().endswith("ok")
+    t = dict(zip(*[iter(p.stdout.split("timing_us ")[1].split("\n")[0].split())] * 2))
+    assert int(t["process"]) > 0 and int(t["update"]) > 0 and int(t["load"]) == 0 and int(t["transfer"]) == 0
+    assert "timing_after_reset 0" in p.stdout
+    s = orc.FParam.simple
+    window = np.stack([orc.random_crop(s(0.5), s(1.2), s(0.3), s(0.7), w, h) for w, h in ROIS])
+    full = np.full(N, 64, np.uint32)
+    mid = orc.resize(img, window, full, full, 64, 64, interp=orc.LINEAR)
+    mid_w, mid_h = np.minimum(window[:, 2], 64), np.minimum(window[:, 3], 64)
+    one = lambda v: np.full(N, v, np.float32)
+    mid_roi = np.stack([np.zeros(N), np.zeros(N), mid_w, mid_h], -1).astype(np.uint32)
+    mid = orc.color_twist(mid, mid_roi, one(1.2), one(8.0), one(40.0), one(1.3))
+    crop = np.stack([orc.fixed_crop(int(w), int(h), 56, 56, anchor=(0.5, 0.5)) for w, h in zip(mid_w, mid_h)])
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    mirrors = _coin_batches(2)
+    for b in range(2):
+        got = np.fromfile(tmp_path / ("out_b%d.bin" % b), dtype=np.float16).reshape(N, 3, 56, 56)
+        _same(got, orc.crop_mirror_normalize(mid, crop, scale, bias, mirrors[b], 56, 56, orc.NCHW, orc.FP16), "caller batch %d" % b)
+        roi = np.loadtxt(tmp_path / ("roi_b%d.txt" % b), dtype=np.int64).reshape(N, 4)
+        assert np.array_equal(roi[:, 2:], crop[:, 2:])
+
+
 def test_resize_colortwist_flip_chain_with_intermediate_tensors(tmp_path):
     img, outs, _ = _run("chain", tmp_path, 2, [(np.uint8, (N, 32, 40, 3))] * 2)
     dw, dh = np.full(N, 40, np.uint32), np.full(N, 32, np.uint32)
