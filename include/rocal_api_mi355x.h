@@ -83,6 +83,10 @@ extern "C" RocalStatus ROCAL_API_CALL rocalTensorSetBuffer(RocalContext context,
 extern "C" const unsigned *ROCAL_API_CALL rocalTensorRoi(RocalTensor tensor);
 extern "C" size_t ROCAL_API_CALL rocalTensorDataSize(RocalTensor tensor);
 
+/* ---- tensors the caller wants to read after a run (rocal_api_data_transfer.h:75): called before rocalVerify, as the Python
+   pipeline does for what define_graph returns; a tensor created with is_output = true is an output already. ---- */
+extern "C" void ROCAL_API_CALL rocalSetOutputs(RocalContext p_context, unsigned int num_of_outputs, std::vector<RocalTensor> &output_images);
+
 /* ---- u8 output -> float tensor (rocal_api_data_transfer.h:45-66). out_ptr is device memory: only ROCAL_MEMCPY_GPU exists. ---- */
 extern "C" RocalStatus ROCAL_API_CALL rocalToTensor(RocalContext rocal_context, void *out_ptr, RocalTensorLayout tensor_format,
                                                     RocalTensorOutputType tensor_output_type, float multiplier0, float multiplier1, float multiplier2,

@@ -161,6 +161,13 @@ RocalStatus rocalDeviceSourceFeed(RocalContext p_context, RocalTensor p_source, 
     return ROCAL_OK;
 }
 
+void rocalSetOutputs(RocalContext p_context, unsigned int num_of_outputs, std::vector<RocalTensor> &output_tensors) {
+    if (!p_context) THROW("Invalid rocal context passed to rocalSetOutputs")
+    auto *context = static_cast<Context *>(p_context);
+    if (num_of_outputs > output_tensors.size()) THROW("rocalSetOutputs: fewer tensors than announced")
+    for (unsigned i = 0; i < num_of_outputs; i++) context->master_graph->set_output(static_cast<Tensor *>(output_tensors[i]));
+}
+
 RocalStatus rocalTensorSetBuffer(RocalContext p_context, RocalTensor p_tensor, void *device_ptr) {
     if (!p_context) return ROCAL_CONTEXT_INVALID;
     auto *context = static_cast<Context *>(p_context);

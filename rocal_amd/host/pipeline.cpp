@@ -203,6 +203,14 @@ Tensor *MasterGraph::create_tensor(const TensorInfo &info, bool is_output) {
 
 // rocalVerify: plan chains, create every node's op on the user thread, then give every tensor that is
 // written by a launch a device buffer (the reference's ring buffer / virtual tensors).
+void MasterGraph::set_output(Tensor *t) {
+    if (!t) THROW("null output tensor")
+    if (_built) THROW("outputs must be set before rocalVerify")
+    if (t->is_output) return;
+    t->is_output = true;
+    _outputs.push_back(t);
+}
+
 void MasterGraph::build() {
     if (_built) THROW("graph already built")
     for (auto &n : _nodes) _graph->add(n.get());

@@ -154,6 +154,7 @@ class MasterGraph {
     }
     void build();
     void run();
+    void set_output(Tensor *t);  // master_graph.cpp:337-349
     // master_graph.cpp:514-856: converts the single u8 output tensor into a float tensor in caller memory
     void to_tensor(void *out_ptr, RocalTensorlayout format, float multiplier0, float multiplier1, float multiplier2, float offset0, float offset1,
                    float offset2, bool reverse_channels, RocalTensorDataType output_data_type, unsigned max_roi_height, unsigned max_roi_width);

@@ -1,0 +1,58 @@
+// Plain-C doorway for Python (ctypes) onto the entry points that take C++ types, standing where the reference's pybind
+// module stands (rocAL_pybind/rocal_pybind.cpp): vectors travel as pointer + length. Every other rocal* entry point takes
+// PODs only and is called by ctypes directly.
+#include <vector>
+
+#include "rocal_api_mi355x.h"
+
+#define PY_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+std::vector<float> vec(const float *p, unsigned n) { return p ? std::vector<float>(p, p + n) : std::vector<float>(); }
+}  // namespace
+
+PY_API RocalTensor rocalpy_resize(RocalContext ctx, RocalTensor in, unsigned dest_width, unsigned dest_height, bool is_output, int scaling_mode,
+                                  const unsigned *max_size, unsigned n_max_size, unsigned resize_shorter, unsigned resize_longer, int interpolation,
+                                  int layout, int dtype) {
+    std::vector<unsigned> ms(max_size, max_size + (max_size ? n_max_size : 0));
+    return rocalResize(ctx, in, dest_width, dest_height, is_output, (RocalResizeScalingMode)scaling_mode, ms, resize_shorter, resize_longer,
+                       (RocalResizeInterpolationType)interpolation, (RocalTensorLayout)layout, (RocalTensorOutputType)dtype);
+}
+
+PY_API RocalTensor rocalpy_resize_mirror_normalize(RocalContext ctx, RocalTensor in, unsigned dest_width, unsigned dest_height, const float *mean,
+                                                   unsigned n_mean, const float *std_dev, unsigned n_std, bool is_output, int scaling_mode,
+                                                   const unsigned *max_size, unsigned n_max_size, unsigned resize_shorter, unsigned resize_longer,
+                                                   int interpolation, RocalIntParam mirror, int layout, int dtype) {
+    std::vector<float> m = vec(mean, n_mean), s = vec(std_dev, n_std);
+    std::vector<unsigned> ms(max_size, max_size + (max_size ? n_max_size : 0));
+    return rocalResizeMirrorNormalize(ctx, in, dest_width, dest_height, m, s, is_output, (RocalResizeScalingMode)scaling_mode, ms, resize_shorter,
+                                      resize_longer, (RocalResizeInterpolationType)interpolation, mirror, (RocalTensorLayout)layout,
+                                      (RocalTensorOutputType)dtype);
+}
+
+PY_API RocalTensor rocalpy_crop_mirror_normalize(RocalContext ctx, RocalTensor in, unsigned crop_height, unsigned crop_width, float start_x,
+                                                 float start_y, const float *mean, unsigned n_mean, const float *std_dev, unsigned n_std,
+                                                 bool is_output, RocalIntParam mirror, int layout, int dtype) {
+    std::vector<float> m = vec(mean, n_mean), s = vec(std_dev, n_std);
+    return rocalCropMirrorNormalize(ctx, in, crop_height, crop_width, start_x, start_y, m, s, is_output, mirror, (RocalTensorLayout)layout,
+                                    (RocalTensorOutputType)dtype);
+}
+
+PY_API int rocalpy_set_outputs(RocalContext ctx, unsigned n, RocalTensor *tensors) {
+    try {
+        std::vector<RocalTensor> v(tensors, tensors + n);
+        rocalSetOutputs(ctx, n, v);
+    } catch (...) {
+        return 1;
+    }
+    return 0;
+}
+
+PY_API void rocalpy_timing(RocalContext ctx, unsigned long long out[5]) {
+    out[4] = rocalGetParameterUpdateTime(ctx);
+    const TimingInfo t = rocalGetTimingInfo(ctx);
+    out[0] = t.load_time;
+    out[1] = t.decode_time;
+    out[2] = t.process_time;
+    out[3] = t.transfer_time;
+}

@@ -1,0 +1,114 @@
+"""Pipeline of the Python API (rocAL_pybind/amd/rocal/pipeline.py:66-170): owns the context, is the `with` scope in which the
+fn.* calls add nodes, marks outputs, builds and runs. Readers and decoders are outside the hot path: a pipeline here takes
+its decoded batches from device memory (device_source / feed)."""
+from . import backend, types
+
+b = backend.Backend()
+
+
+class Pipeline:
+    _current_pipeline = None
+
+    def __init__(self, batch_size=-1, num_threads=0, device_id=0, seed=1, exec_pipelined=True, prefetch_queue_depth=2, exec_async=True,
+                 bytes_per_sample=0, rocal_cpu=False, max_streams=-1, default_cuda_stream_priority=0, tensor_layout=types.NCHW,
+                 reverse_channels=False, mean=None, std=None, tensor_dtype=types.FLOAT, output_memory_type=None):
+        if rocal_cpu:
+            raise Exception("Failed creating the pipeline: this build has no CPU path (rocal_cpu=True)")
+        self._handle = b.rocalCreate(batch_size, types.GPU, device_id, num_threads, prefetch_queue_depth, tensor_dtype)
+        if b.getStatus(self._handle) != types.OK:
+            raise Exception("Failed creating the pipeline")
+        self._batch_size = batch_size
+        self._device_id = device_id
+        self._seed = seed
+        self._tensor_layout = tensor_layout
+        self._tensor_dtype = tensor_dtype
+        # pipeline.py:100-103: what copyToExternalTensor applies to a u8 output
+        self._multiplier = list(map(lambda x: 1 / x, std)) if std else [1.0, 1.0, 1.0]
+        self._offset = list(map(lambda x, y: -(x / y), mean, std)) if mean and std else [0.0, 0.0, 0.0]
+        self._reverse_channels = reverse_channels
+        self._output_memory_type = output_memory_type if output_memory_type else types.DEVICE_MEMORY
+        self._outputs = []
+        self.set_seed(self._seed)
+
+    def __enter__(self):
+        Pipeline._current_pipeline = self
+        return self
+
+    def __exit__(self, exception_type, exception_value, traceback):
+        Pipeline._current_pipeline = None
+
+    def set_seed(self, seed=0):
+        return b.setSeed(seed)
+
+    def create_int_param(self, value=1):
+        return b.createIntParameter(value)
+
+    def create_float_param(self, value=1):
+        return b.createFloatParameter(value)
+
+    def update_int_param(self, value=1, param=1):
+        b.updateIntParameter(value, param)
+
+    def update_float_param(self, value=1, param=1):
+        b.updateFloatParameter(value, param)
+
+    def get_int_value(self, param):
+        return b.getIntValue(param)
+
+    def get_float_value(self, param):
+        return b.getFloatValue(param)
+
+    def get_handle(self):
+        return self._handle
+
+    def set_outputs(self, *output_list):
+        self._outputs = list(output_list)
+        b.setOutputs(self._handle, len(output_list), output_list)
+
+    def build(self):
+        status = b.rocalVerify(self._handle)
+        if status != types.OK:
+            raise RuntimeError("Verify graph failed: " + b.getErrorMessage(self._handle))
+        return self
+
+    def rocal_run(self):
+        status = b.rocalRun(self._handle)
+        if status != types.OK:
+            raise RuntimeError("rocalRun failed: " + b.getErrorMessage(self._handle))
+        return status
+
+    def copyToExternalTensor(self, array, multiplier, offset, reverse_channels, tensor_format, tensor_dtype, max_roi_height=0, max_roi_width=0):
+        import ctypes
+        b.rocalToTensor(self._handle, ctypes.c_void_p(array.data_ptr()), tensor_format, tensor_dtype, multiplier[0], multiplier[1], multiplier[2],
+                        offset[0], offset[1], offset[2], reverse_channels, self._output_memory_type, max_roi_height, max_roi_width)
+
+    def timing_info(self):
+        return b.getTimingInfo(self._handle)
+
+    # ---- decoded batches in device memory (where the reference has readers and decoders)
+    def device_source(self, max_width, max_height, is_output=False):
+        return b.deviceSource(self._handle, max_width, max_height, is_output)
+
+    def feed(self, source, tensor, widths, heights):
+        """tensor: a torch CUDA uint8 tensor [N, max_height, max_width, 3]; widths / heights: the valid size of each image."""
+        assert tensor.is_cuda and tensor.is_contiguous()
+        self._fed = tensor  # kept alive until the next batch
+        status = b.deviceSourceFeed(self._handle, source, tensor.data_ptr(), widths, heights)
+        if status != types.OK:
+            raise RuntimeError("feed failed: " + b.getErrorMessage(self._handle))
+
+    def bind_output(self, output, tensor):
+        """The node that produces `output` writes straight into `tensor` (a torch CUDA tensor the caller owns): no copy afterwards."""
+        assert tensor.is_cuda and tensor.is_contiguous() and tensor.numel() * tensor.element_size() >= b.tensorDataSize(output)
+        self._bound = getattr(self, "_bound", {})
+        self._bound[output] = tensor
+        if b.tensorSetBuffer(self._handle, output, tensor.data_ptr()) != types.OK:
+            raise RuntimeError("bind_output failed: " + b.getErrorMessage(self._handle))
+
+    def output_roi(self, output):
+        return b.tensorRoi(output, self._batch_size)
+
+    def release(self):
+        if self._handle:
+            b.rocalRelease(self._handle)
+            self._handle = None
