@@ -221,6 +221,14 @@ extern "C" RocalTensor ROCAL_API_CALL rocalExposure(RocalContext context, RocalT
 extern "C" RocalTensor ROCAL_API_CALL rocalExposureFixed(RocalContext context, RocalTensor input, float exposure_factor, bool is_output,
                                                          RocalTensorLayout output_layout = ROCAL_NONE,
                                                          RocalTensorOutputType output_datatype = ROCAL_UINT8);  // :779
+// Normalize and Transpose on image tensors (rocal_api_augmentation.h: rocalNormalize, rocalTranspose). axes / perm name the axes of
+// the tensor without its batch axis: 0 height, 1 width, 2 channels. Normalize: axes {0,1} or {0,1,2}; an empty mean / std_dev is
+// computed per sample. Transpose: {0,1,2}, {2,0,1}, {1,0,2}, {2,1,0} with the output layout the permutation produces.
+extern "C" RocalTensor ROCAL_API_CALL rocalNormalize(RocalContext context, RocalTensor input, std::vector<unsigned> &axes, std::vector<float> &mean,
+                                                     std::vector<float> &std_dev, bool is_output, float scale = 1.0, float shift = 0.0,
+                                                     RocalTensorOutputType output_datatype = ROCAL_FP32);
+extern "C" RocalTensor ROCAL_API_CALL rocalTranspose(RocalContext context, RocalTensor input, std::vector<unsigned> perm, bool is_output,
+                                                     RocalTensorLayout output_layout = ROCAL_NONE);
 extern "C" RocalTensor ROCAL_API_CALL rocalCropMirrorNormalize(RocalContext context, RocalTensor input, unsigned crop_height, unsigned crop_width,
                                                                float start_x, float start_y, std::vector<float> &mean, std::vector<float> &std_dev,
                                                                bool is_output, RocalIntParam mirror = NULL, RocalTensorLayout output_layout = ROCAL_NONE,

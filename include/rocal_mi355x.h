@@ -215,6 +215,27 @@ RMX_API int rmx_update_blend(rmx_op *op, const uint32_t *src_roi, const float *r
 /* process step of a two-input node (Blend): as rmx_op_launch, with the second source batch. */
 RMX_API int rmx_op_launch2(rmx_op *op, const void *src1, const void *src2, void *dst);
 
+/* ---- Normalize: replaces vxExtRppNormalize (rocAL/source/augmentations/effects_augmentations/node_normalize.cpp:31-113) for image
+ *      tensors: per sample, out = (x - mean) / stddev * scale + shift with the statistics taken over the axes of axis_mask
+ *      (bit 0 height, bit 1 width, bit 2 channels): 3 = one mean / stddev per channel, 7 = one per sample; other masks are
+ *      outside the hot path. mean and / or stddev NULL: computed on the device from the sample's window (exact integer moments,
+ *      population standard deviation; a zero deviation gives out = shift); else n_stats (1 or 3) given values, as the node
+ *      replicates its vectors. The arithmetic lives in RPP; the law is the one stated here: one fp32 FMA per value with
+ *      a = scale / stddev and b = fma(-mean, a, shift). ---- */
+RMX_API int rmx_create_normalize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out);
+RMX_API int rmx_update_normalize(rmx_op *op, const uint32_t *src_roi, uint32_t axis_mask, const float *mean, const float *stddev,
+                                 uint32_t n_stats, float scale, float shift);
+
+/* ---- Transpose: replaces vxExtRppTranspose (rocAL/source/augmentations/geometry_augmentations/node_transpose.cpp:31-48) for image
+ *      tensors. perm holds the three axes (0 height, 1 width, 2 channels) of the u8 [N,H,W,C] source in output order; on images the
+ *      channel axis stays at the back or goes to the front (:52-53): {0,1,2} copy, {2,0,1} planes [N,C,H,W], {1,0,2} height and
+ *      width swapped [N,W,H,C], {2,1,0} both [N,C,W,H]. The destination descriptor gives the padded size of the output's two
+ *      image axes (for the swapping permutations h >= source w and w >= source h) and its layout must be the one the
+ *      permutation produces; its dtype may differ from u8 (values are converted). ---- */
+RMX_API int rmx_create_transpose(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, const uint32_t *perm /*[3]*/,
+                                 int roi_type, rmx_op **out);
+RMX_API int rmx_update_transpose(rmx_op *op, const uint32_t *src_roi);
+
 /* ---- WarpAffine: replaces vxExtRppWarpAffine (node_warp_affine.cpp:61-62). affine is [N][6] in
  *      rocAL's fill order x0,y0,x1,y1,o0,o1 (:43-48), read as M=[[x0,x1,o0],[y0,y1,o1]] mapping
  *      destination to source about the ROI / output centres. Out-of-ROI samples give 0. ---- */

@@ -174,6 +174,19 @@ def color_temperature(img, roi_xywh, adjustment, flags=0, layout=NHWC, dtype=UIN
     return out
 
 
+def normalize(img, roi_xywh, axis_mask=3, mean=None, stddev=None, scale=1.0, shift=0.0, layout=NHWC, dtype=FP32, flags=0):
+    roi_xywh = _u32(roi_xywh)
+    n, h, w, c = img.shape
+    out, d = _alloc_dst(n, c, h, w, layout, dtype)
+    s = _src(img)
+    m = _f32(mean) if mean is not None else None
+    sd = _f32(stddev) if stddev is not None else None
+    n_stats = len(m) if m is not None else (len(sd) if sd is not None else 0)
+    lib().orc_normalize(C.byref(s), _p(roi_xywh), C.c_uint(axis_mask), _p(m) if m is not None else None, _p(sd) if sd is not None else None,
+                        C.c_uint(n_stats), C.c_float(scale), C.c_float(shift), C.byref(d), C.c_uint(flags))
+    return out
+
+
 def blend(img1, img2, roi_xywh, ratio, flags=0, layout=NHWC, dtype=UINT8):
     assert img1.shape == img2.shape
     roi_xywh, ratio = _u32(roi_xywh), _f32(ratio)

@@ -488,6 +488,53 @@ void orc_blend(const orc_src *src1, const orc_src *src2, const uint32_t *roi, co
     }
 }
 
+/* Normalize (vxExtRppNormalize, effects_augmentations/node_normalize.cpp:31-113) for image tensors; law DEFINED here (the arithmetic
+ * lives in RPP): statistics over height and width (axis_mask 3: per channel) or height, width and channels (7: per sample), from
+ * exact integer moments: mean = sum / count, stddev = sqrt(sum (x - mean)^2 / count) in double, then fp32
+ * a = scale / stddev (0 when stddev is 0), b = fmaf(-mean, a, shift), out = fmaf(x, a, b). */
+void orc_normalize(const orc_src *src, const uint32_t *roi, unsigned axis_mask, const float *mean, const float *stddev, unsigned n_stats,
+                   float scale, float shift, const orc_dst *dst, unsigned flags) {
+#pragma omp parallel for schedule(dynamic)
+    for (int n = 0; n < src->n; n++) {
+        int x0 = (int)roi[n * 4], y0 = (int)roi[n * 4 + 1], w = (int)roi[n * 4 + 2], h = (int)roi[n * 4 + 3];
+        unsigned long long sum[3] = {0, 0, 0}, sq[3] = {0, 0, 0};
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const uint8_t *p = src_px(src, n, y0 + y, x0 + x);
+                for (int c = 0; c < 3; c++) {
+                    sum[c] += p[c];
+                    sq[c] += (unsigned)p[c] * p[c];
+                }
+            }
+        float a[3], b[3];
+        for (int c = 0; c < 3; c++) {
+            double cnt = (double)w * (double)h, s1 = (double)sum[c], s2 = (double)sq[c];
+            if (axis_mask == 7u) {
+                cnt *= 3.0;
+                s1 = (double)(sum[0] + sum[1] + sum[2]);
+                s2 = (double)(sq[0] + sq[1] + sq[2]);
+            }
+            float m = mean ? mean[n_stats == 3 ? c : 0] : 0.0f, sd = stddev ? stddev[n_stats == 3 ? c : 0] : 1.0f;
+            if (cnt > 0.0) {
+                const double md = mean ? (double)m : s1 / cnt;
+                if (!mean) m = (float)md;
+                if (!stddev) {
+                    double var = (s2 - 2.0 * md * s1 + cnt * md * md) / cnt;
+                    if (var < 0.0) var = 0.0;
+                    sd = (float)sqrt(var);
+                }
+            }
+            a[c] = sd != 0.0f ? scale / sd : 0.0f;
+            b[c] = fmaf(-m, a[c], shift);
+        }
+        for (int y = 0; y < h; y++)
+            for (int x = 0; x < w; x++) {
+                const uint8_t *p = src_px(src, n, y0 + y, x0 + x);
+                for (int c = 0; c < 3; c++) store(dst, dst_index(dst, n, c, y, x), fmaf((float)p[c], a[c], b[c]), flags);
+            }
+    }
+}
+
 /* hue in degrees -> shift in sextants, reduced to [0,6] */
 static float hue_shift_sextants(float hue_deg, unsigned flags) {
     if (flags & ORC_F_HUE_INT_TRUNC) hue_deg = (float)((int)hue_deg % 360);

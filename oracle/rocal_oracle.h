@@ -36,6 +36,8 @@
  *   orc_resize (nearest)       law DEFINED here (floor of the half-pixel-centre coordinate + 0.5); the restatement is
  *                              checked against hand-written indices (identity, 2x / 3x down, 2x / 3x replication, ROI and
  *                              mirror); against RPP it is parity unpinned.
+ *   orc_normalize              law DEFINED here (PARITY UNPINNED against RPP); the restatement is checked against numpy's mean / std in
+ *                              float64, a constant image (out = shift) and a two-valued image with hand-computed statistics.
  *   orc_color_twist/hue/sat    restatement checked on all 2^24 RGB triples against the same HSV round trip written
  *                              with true divisions in numpy (5 parameter sets: at most one level apart, < 0.3 % of
  *                              values differ), identity, grey fixed points, 360-periodicity, colorsys. Against RPP the
@@ -126,6 +128,9 @@ void orc_gamma(const orc_src *src, const uint32_t *roi_xywh, const float *gamma,
 void orc_exposure(const orc_src *src, const uint32_t *roi_xywh, const float *factor, const orc_dst *dst, unsigned flags);
 void orc_color_temperature(const orc_src *src, const uint32_t *roi_xywh, const int32_t *adjustment, const orc_dst *dst,
                            unsigned flags);
+/* axis_mask 3 (height, width) or 7 (height, width, channels); mean / stddev NULL = computed; n_stats 1 or 3 given values */
+void orc_normalize(const orc_src *src, const uint32_t *roi_xywh, unsigned axis_mask, const float *mean, const float *stddev, unsigned n_stats,
+                   float scale, float shift, const orc_dst *dst, unsigned flags);
 void orc_blend(const orc_src *src1, const orc_src *src2, const uint32_t *roi_xywh, const float *ratio, const orc_dst *dst,
                unsigned flags);
 /* HSV colour twist; hue in degrees. */

@@ -73,6 +73,10 @@ _SIGS = {
     "rmx_update_rotate": [_vp, _vp, _vp, _vp, _vp],
     "rmx_create_to_tensor": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.POINTER(_vp)],
     "rmx_update_to_tensor": [_vp, _vp, _vp, C.c_int],
+    "rmx_create_normalize": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
+    "rmx_update_normalize": [_vp, _vp, C.c_uint32, _vp, _vp, C.c_uint32, C.c_float, C.c_float],
+    "rmx_create_transpose": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), _vp, C.c_int, C.POINTER(_vp)],
+    "rmx_update_transpose": [_vp, _vp],
     "rmx_copy_bytes": [_vp, _vp, _vp, C.c_size_t],
     "rmx_resize_cmn_noalloc": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
 }

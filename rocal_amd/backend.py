@@ -42,6 +42,8 @@ _SIGS = {
     "rocalpy_resize": (_vp, [_vp, _vp, _u, _u, _b, _i, _vp, _u, _u, _u, _i, _i, _i]),
     "rocalpy_resize_mirror_normalize": (_vp, [_vp, _vp, _u, _u, _vp, _u, _vp, _u, _b, _i, _vp, _u, _u, _u, _i, _vp, _i, _i]),
     "rocalpy_crop_mirror_normalize": (_vp, [_vp, _vp, _u, _u, _f, _f, _vp, _u, _vp, _u, _b, _vp, _i, _i]),
+    "rocalpy_normalize": (_vp, [_vp, _vp, _vp, _u, _vp, _u, _vp, _u, _b, _f, _f, _i]),
+    "rocalpy_transpose": (_vp, [_vp, _vp, _vp, _u, _b, _i]),
     "rocalpy_set_outputs": (_i, [_vp, _u, _vp]), "rocalpy_timing": (None, [_vp, _vp]),
 }
 
@@ -234,6 +236,14 @@ class Backend:
 
     def blend(self, handle, inp1, inp2, is_output, ratio, layout, dtype):
         return host().rocalBlend(handle, inp1, inp2, is_output, ratio, layout, dtype)
+
+    def normalize(self, handle, inp, axes, mean, std_dev, is_output, scale, shift, dtype):
+        (ax, na), (m, nm), (s, ns) = _uarr(axes), _farr(mean), _farr(std_dev)
+        return host().rocalpy_normalize(handle, inp, ax, na, m if nm else None, nm, s if ns else None, ns, is_output, scale, shift, dtype)
+
+    def transpose(self, handle, inp, perm, is_output, layout):
+        p, n = _uarr(perm)
+        return host().rocalpy_transpose(handle, inp, p, n, is_output, layout)
 
     def crop(self, handle, inp, is_output, crop_width, crop_height, crop_depth, pos_x, pos_y, pos_z, layout, dtype):
         return host().rocalCrop(handle, inp, is_output, crop_width, crop_height, crop_depth, pos_x, pos_y, pos_z, layout, dtype)

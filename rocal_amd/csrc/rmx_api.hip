@@ -38,7 +38,7 @@ int fail(int code, const char *fmt, ...) {
 
 enum OpKind {
     OP_CMN = 1, OP_CROP, OP_FLIP, OP_RESIZE, OP_COLOR_TWIST, OP_BRIGHTNESS, OP_CONTRAST, OP_HUE,
-    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE, OP_TO_TENSOR, OP_GAMMA, OP_EXPOSURE, OP_COLOR_TEMPERATURE, OP_BLEND
+    OP_SATURATION, OP_WARP_AFFINE, OP_ROTATE, OP_TO_TENSOR, OP_GAMMA, OP_EXPOSURE, OP_COLOR_TEMPERATURE, OP_BLEND, OP_NORMALIZE, OP_TRANSPOSE
 };
 
 constexpr int TABLE_RING = 4;  // updates in flight before the host has to wait on an old upload
@@ -123,6 +123,8 @@ struct rmx_op {
     int fast_aux1 = 0;                                               // aux1 of fn_fast
     bool fast_needs_src16 = false;                                   // fn_fast also wants a 16-byte aligned source base
     uint64_t algo_bytes = 0;
+    int stats_mode = 0, stats_per_channel = 1;  // Normalize: what is computed on the device (bit 0 mean, bit 1 standard deviation)
+    float stats_scale = 1.0f, stats_shift = 0.0f;
     rmx::KernelFn lds_fn[2] = {};  // kernels whose static LDS size has been asked of the runtime ([0] general, [1] fast)
     int lds_static[2] = {};
 };
@@ -425,6 +427,15 @@ static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *
     if (blocks == 0 || blocks > 0x7fffffffull) return fail(RMX_ERR_INVALID, "grid of %llu workgroups is out of range", (unsigned long long)blocks);
     a.wpb = wpb;
     a.nblocks = (uint32_t)blocks;
+    if (op->kind == OP_NORMALIZE) {
+        // moments of every sample's window (when asked for), then the FMA constants into the rows the streaming pass reads;
+        // the side table of the slot holds the given statistics (6 floats per sample) and, behind them, the 64-bit counters
+        const float *given = reinterpret_cast<const float *>(extra);
+        unsigned long long *counters = reinterpret_cast<unsigned long long *>(const_cast<uint8_t *>(extra) + (size_t)op->n * 24);
+        rmx::launch_stats(op->ctx->stream, a, counters, const_cast<RmxSample *>(table), given, op->stats_mode, op->stats_per_channel, op->stats_scale,
+                          op->stats_shift, op->stats_mode != 0);
+        HIP_TRY(hipGetLastError());
+    }
     hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
     HIP_TRY(hipGetLastError());
     return RMX_OK;
@@ -482,7 +493,7 @@ static int create_k1(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const r
 }
 
 static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const float *bias, const uint32_t *hflip, const uint32_t *vflip,
-                     bool per_sample_scale = true, bool channel_reverse = false) {
+                     bool per_sample_scale = true, bool channel_reverse = false, int *open_slot = nullptr) {
     RmxSample *t;
     int slot = next_slot(op, &t);
     if (slot < 0) return RMX_ERR_HIP;
@@ -526,6 +537,10 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
         op->fast_wpb = op->waves_per_block;
         op->fast_needs_src16 = false;
     }
+    if (open_slot) {  // the caller fills the side table of the slot and commits it
+        *open_slot = slot;
+        return RMX_OK;
+    }
     return commit_slot(op, slot);
 }
 
@@ -566,6 +581,98 @@ int rmx_update_to_tensor(rmx_op *op, const float *multiplier, const float *offse
     if (!op || op->kind != OP_TO_TENSOR) return fail(RMX_ERR_INVALID, "op is not a ToTensor node");
     if (!multiplier || !offset) return fail(RMX_ERR_INVALID, "multiplier and offset (3 floats each) are required");
     return update_k1(op, nullptr, multiplier, offset, nullptr, nullptr, false, reverse_channels != 0);
+}
+
+/* ------------------------------------------------------------------ Normalize */
+
+int rmx_create_normalize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
+    // side table per sample: 6 floats of given statistics + 6 counters of 8 bytes
+    int rc = make_op(ctx, OP_NORMALIZE, src, dst, roi_type, out, 72);
+    if (rc) return rc;
+    (*out)->norm = true;
+    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, true, false, &(*out)->kernel_name);
+    return RMX_OK;
+}
+
+int rmx_update_normalize(rmx_op *op, const uint32_t *src_roi, uint32_t axis_mask, const float *mean, const float *stddev, uint32_t n_stats,
+                         float scale, float shift) {
+    if (!op || op->kind != OP_NORMALIZE) return fail(RMX_ERR_INVALID, "op is not a Normalize node");
+    if (axis_mask != 3u && axis_mask != 7u)
+        return fail(RMX_ERR_UNSUPPORTED, "axis mask %u: images are normalised over height and width (3) or height, width and channels (7)", axis_mask);
+    if ((mean || stddev) && n_stats != 1 && n_stats != 3) return fail(RMX_ERR_INVALID, "given statistics hold 1 or 3 values (n_stats = %u)", n_stats);
+    if (stddev)
+        for (uint32_t k = 0; k < n_stats; k++)
+            if (stddev[k] == 0.0f) return fail(RMX_ERR_INVALID, "standard deviation %u is 0", k);
+    int slot = -1;
+    int rc = update_k1(op, src_roi, nullptr, nullptr, nullptr, nullptr, true, false, &slot);
+    if (rc) return rc;
+    float *given = reinterpret_cast<float *>(slot_extra(op, op->h_table[slot]));
+    for (int i = 0; i < op->n; i++)
+        for (int c = 0; c < 3; c++) {
+            given[(size_t)i * 6 + c] = mean ? mean[n_stats == 3 ? c : 0] : 0.0f;
+            given[(size_t)i * 6 + 3 + c] = stddev ? stddev[n_stats == 3 ? c : 0] : 1.0f;
+        }
+    op->stats_mode = (mean ? 0 : 1) | (stddev ? 0 : 2);
+    op->stats_per_channel = axis_mask == 3u ? 1 : 0;
+    op->stats_scale = scale;
+    op->stats_shift = shift;
+    // the moments pass reads every source byte once more when something is computed
+    if (op->stats_mode) op->algo_bytes += op->algo_bytes / (1 + dtype_size(op->dst.dtype));
+    return commit_slot(op, slot);
+}
+
+/* ------------------------------------------------------------------ Transpose */
+
+int rmx_create_transpose(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, const uint32_t *perm, int roi_type, rmx_op **out) {
+    if (out) *out = nullptr;
+    if (!perm) return fail(RMX_ERR_INVALID, "perm (3 axes) is required");
+    const uint32_t p = perm[0] * 100 + perm[1] * 10 + perm[2];
+    if (!src || !dst) return fail(RMX_ERR_INVALID, "descriptor is NULL");
+    // channels stay last (NHWC-shaped output) or go to the front (NCHW-shaped output); height and width keep or swap places
+    const bool swap = p == 102 || p == 210;
+    if (p != 12 && p != 201 && !swap)
+        return fail(RMX_ERR_UNSUPPORTED, "permutation {%u,%u,%u}: on images the channel axis goes to the front or stays at the back", perm[0], perm[1], perm[2]);
+    const int want_layout = (p == 12 || p == 102) ? RMX_NHWC : RMX_NCHW;
+    if (dst->layout != want_layout) return fail(RMX_ERR_INVALID, "permutation {%u,%u,%u} produces a %s tensor", perm[0], perm[1], perm[2], want_layout == RMX_NHWC ? "channels-last" : "channels-first");
+    if (swap ? (dst->h < src->w || dst->w < src->h) : (dst->h < src->h || dst->w < src->w))
+        return fail(RMX_ERR_INVALID, "destination of %u x %u cannot hold the permuted %u x %u source", dst->w, dst->h, src->w, src->h);
+    int rc = make_op(ctx, OP_TRANSPOSE, src, dst, roi_type, out);
+    if (rc) return rc;
+    (*out)->aux1 = swap ? 1 : 0;
+    if (swap) (*out)->fn = rmx::select_transpose_kernel(dst->dtype, dst->layout, &(*out)->kernel_name);
+    else (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, false, false, &(*out)->kernel_name);
+    return RMX_OK;
+}
+
+int rmx_update_transpose(rmx_op *op, const uint32_t *src_roi) {
+    if (!op || op->kind != OP_TRANSPOSE) return fail(RMX_ERR_INVALID, "op is not a Transpose node");
+    if (!op->aux1) return update_k1(op, src_roi, nullptr, nullptr, nullptr, nullptr);  // a layout change of the streaming kernel
+    RmxSample *t;
+    int slot = next_slot(op, &t);
+    if (slot < 0) return RMX_ERR_HIP;
+    uint64_t bytes = 0;
+    int max_w = 1, max_h = 1;
+    for (int i = 0; i < op->n; i++) {
+        RmxSample &s = t[i];
+        int rc = read_roi(op, src_roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
+        if (rc) return rc;
+        s.src_w = std::min<int32_t>(s.src_w, (int32_t)op->dst.h);  // the window's width becomes the output's height
+        s.src_h = std::min<int32_t>(s.src_h, (int32_t)op->dst.w);
+        s.dst_w = s.src_h;
+        s.dst_h = s.src_w;
+        s.flags = 0;
+        bytes += (uint64_t)s.src_w * s.src_h * 3 * (1 + dtype_size(op->dst.dtype));
+        max_w = std::max(max_w, (int)s.src_w);
+        max_h = std::max(max_h, (int)s.src_h);
+    }
+    op->algo_bytes = bytes;
+    const int tiles_x = (max_w + 31) / 32, tiles_y = (max_h + 31) / 32;
+    op->strips = tiles_x * tiles_y;
+    op->aux0 = tiles_x;
+    op->lds_per_wave = 0;
+    op->waves_per_block = 4;
+    op->fn_fast = nullptr;
+    return commit_slot(op, slot);
 }
 
 /* ------------------------------------------------------------------ K2 family */

@@ -146,7 +146,6 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     // pieces behind the row's data repeat a neighbouring data piece (their content is never read before a replica is
     // written over it).
     auto issue = [&](DmaItem &g, uint32_t *buf) {
-        const int tp = g.nrows * g.ppr;
         if (g.safe) {
             // One load instruction per row and 64 pieces: the row's address is scalar arithmetic, a lane's piece offset is the
             // same for every row, and consecutive lanes fill consecutive 16-byte slots from (r * ppr + c0) on.
@@ -163,6 +162,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
             }
         } else {
             // the window touches the last bytes of the batch buffer: bounds-checked byte loads, stored by the lanes
+            const int tp = g.nrows * g.ppr;
             for (int idx = lane; idx < tp; idx += RMX_WAVE) {
                 const int r = idx / g.ppr;
                 const int c = idx - r * g.ppr;

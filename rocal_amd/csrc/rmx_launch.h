@@ -15,6 +15,10 @@ KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, 
 KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name);
 KernelFn select_point_kernel(int kind, int dtype, int layout, bool fast, const char **name);
+KernelFn select_transpose_kernel(int dtype, int layout, const char **name);
 KernelFn select_warp_kernel(int interp, int dtype, int layout, const char **name);
+// Normalize: (reduce: zero + per-sample integer moments,) then the FMA constants into the rows of `table` (device memory)
+void launch_stats(hipStream_t stream, const RmxKArgs &a, unsigned long long *counters, RmxSample *table, const float *given, int mode, int per_channel,
+                  float scale, float shift, bool reduce);
 void launch_copy(hipStream_t stream, const void *src, void *dst, size_t nbytes, int num_cus);
 }  // namespace rmx

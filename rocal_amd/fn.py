@@ -183,3 +183,13 @@ def color_temp(*inputs, adjustment_value=50, device=None, output_layout=types.NH
 
 def blend(*inputs, ratio=None, device=None, output_layout=types.NHWC, output_dtype=types.UINT8):
     return b.blend(_handle(), inputs[0], inputs[1], False, _fparam(ratio), output_layout, output_dtype)
+
+
+# ---- fn.py: normalize (axes, mean, stddev, scale, shift) and transpose (perm) on image tensors
+def normalize(*inputs, axes=[], mean=[], stddev=[], scale=1.0, shift=0.0, output_dtype=types.FLOAT):
+    """axes: the reduced axes (0 height, 1 width, 2 channels); empty mean / stddev are computed per sample."""
+    return b.normalize(_handle(), inputs[0], axes, mean, stddev, False, scale, shift, output_dtype)
+
+
+def transpose(*inputs, perm=[], output_layout=types.NHWC, output_dtype=types.UINT8):
+    return b.transpose(_handle(), inputs[0], perm, False, output_layout)

@@ -567,6 +567,31 @@ RocalTensor rocalGamma(RocalContext c, RocalTensor in, bool is_output, RocalFloa
 RocalTensor rocalGammaFixed(RocalContext c, RocalTensor in, float gamma, bool is_output, RocalTensorLayout layout, RocalTensorOutputType dtype) {
     return add_op<GammaNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](GammaNode &n) { n.init(gamma); });
 }
+// rocal_api_augmentation.cpp:2288-2308: same shape and layout as the input, the requested type
+RocalTensor rocalNormalize(RocalContext c, RocalTensor in, std::vector<unsigned> &axes, std::vector<float> &mean, std::vector<float> &std_dev, bool is_output,
+                           float scale, float shift, RocalTensorOutputType dtype) {
+    const auto layout = in ? (RocalTensorLayout) static_cast<Tensor *>(in)->info().layout() : ROCAL_NHWC;
+    return add_op<NormalizeNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](NormalizeNode &n) { n.init(axes, mean, std_dev, scale, shift); });
+}
+
+// rocal_api_augmentation.cpp:2349-2378: the dims follow the permutation, the layout is the one asked for
+RocalTensor rocalTranspose(RocalContext c, RocalTensor in, std::vector<unsigned> perm, bool is_output, RocalTensorLayout output_layout) {
+    const char *err = nullptr;
+    unsigned w = 0, h = 0;
+    if (c && in) {
+        const TensorInfo &info = static_cast<Tensor *>(in)->info();
+        if (perm.size() != 3) {
+            err = "Transpose permutation must match with the input dims";
+        } else {
+            const bool swap = (perm == std::vector<unsigned>{2, 1, 0}) || (perm == std::vector<unsigned>{1, 0, 2});
+            w = (unsigned)(swap ? info.max_shape()[1] : info.max_shape()[0]);
+            h = (unsigned)(swap ? info.max_shape()[0] : info.max_shape()[1]);
+        }
+    }
+    const auto dtype = in ? (RocalTensorOutputType) static_cast<Tensor *>(in)->info().data_type() : ROCAL_UINT8;
+    return add_op<TransposeNode>(c, in, is_output, output_layout, dtype, Dims::SET, w, h, err, [&](TransposeNode &n) { n.init(perm); });
+}
+
 RocalTensor rocalExposure(RocalContext c, RocalTensor in, bool is_output, RocalFloatParam exposure_factor, RocalTensorLayout layout,
                           RocalTensorOutputType dtype) {
     return add_op<ExposureNode>(c, in, is_output, layout, dtype, Dims::KEEP, 0, 0, nullptr, [&](ExposureNode &n) { n.init(F(exposure_factor)); });

@@ -257,6 +257,13 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         RocalTensor other = rocalResize(ctx, src, 40, 32, true, ROCAL_SCALING_MODE_STRETCH, {}, 0, 0, ROCAL_NEAREST_NEIGHBOR_INTERPOLATION);
         outs.push_back(other);
         outs.push_back(rocalBlendFixed(ctx, other, mid, 0.25f, true));
+    } else if (scenario == "normalize_transpose") {
+        std::vector<unsigned> hw{0, 1}, hwc{0, 1, 2};
+        std::vector<float> none, m3{10.0f, 20.0f, 30.0f}, s3{2.0f, 4.0f, 8.0f};
+        outs.push_back(rocalNormalize(ctx, src, hw, none, none, true));                       // per-channel statistics of every window, fp32
+        outs.push_back(rocalNormalize(ctx, src, hwc, m3, s3, true, 3.0f, 1.0f, ROCAL_FP16));  // given statistics, scale and shift
+        outs.push_back(rocalTranspose(ctx, src, {1, 0, 2}, true, ROCAL_NHWC));                // [N, W, H, C]
+        outs.push_back(rocalTranspose(ctx, src, {2, 0, 1}, true, ROCAL_NCHW));                // [N, C, H, W]
     } else if (scenario == "to_tensor") {
         outs.push_back(rocalResize(ctx, src, 40, 32, true));
     } else if (scenario == "errors") {

@@ -639,6 +639,55 @@ void GammaNode::update_node() {
     check(rmx_update_gamma(_node, roi.data(), _gamma.values().data()), "rmx_update_gamma");
 }
 
+NormalizeNode::NormalizeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs) : Node(inputs, outputs) {}
+
+void NormalizeNode::init(std::vector<unsigned> &axes, std::vector<float> &mean, std::vector<float> &std_dev, float scale, float shift) {
+    _mean = mean;
+    _std_dev = std_dev;
+    _scale = scale;
+    _shift = shift;
+    for (unsigned d = 0; d < axes.size(); d++) _axis_mask |= (1 << axes[d]);
+}
+
+void NormalizeNode::create_node() {
+    if (_mean.size() && _std_dev.size() && _mean.size() != _std_dev.size()) THROW("Normalize: mean and stddev must hold the same number of values")
+    for (float v : _std_dev)
+        if (v == 0.0f) THROW("Normalize: standard deviation value cannot be 0")
+    RMX_COLOR_CREATE(rmx_create_normalize)
+}
+
+void NormalizeNode::update_node() {
+    const auto roi = roi_as_array(_inputs[0]->info().roi());
+    const unsigned n_stats = (unsigned)(_mean.size() ? _mean.size() : _std_dev.size());
+    check(rmx_update_normalize(_node, roi.data(), (uint32_t)_axis_mask, _mean.size() ? _mean.data() : nullptr, _std_dev.size() ? _std_dev.data() : nullptr,
+                               n_stats, _scale, _shift),
+          "rmx_update_normalize");
+}
+
+TransposeNode::TransposeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs) : Node(inputs, outputs) {}
+void TransposeNode::init(std::vector<unsigned> perm) { _perm = perm; }
+
+void TransposeNode::create_node() {
+    if (_node) return;
+    if (_perm.size() != 3) THROW("Transpose permutation must match with the input dims")
+    rmx_tensor_desc s = _inputs[0]->info().desc(), d = _outputs[0]->info().desc();
+    check(rmx_create_transpose(_graph->get(), &s, &d, _perm.data(), (int)_inputs[0]->info().roi_type(), &_node), "rmx_create_transpose");
+}
+
+// node_transpose.cpp:50-66: the output ROI swaps width and height when the permutation does
+void TransposeNode::update_node() {
+    const Roi2DCords *src = _inputs[0]->info().roi();
+    const bool swap = (_perm == std::vector<unsigned>{2, 1, 0}) || (_perm == std::vector<unsigned>{1, 0, 2});
+    std::vector<uint32_t> w(_batch_size), h(_batch_size);
+    for (size_t i = 0; i < _batch_size; i++) {
+        w[i] = swap ? src[i].xywh.h : src[i].xywh.w;
+        h[i] = swap ? src[i].xywh.w : src[i].xywh.h;
+    }
+    _outputs[0]->update_tensor_roi(w, h);
+    const auto roi = roi_as_array(src);
+    check(rmx_update_transpose(_node, roi.data()), "rmx_update_transpose");
+}
+
 ExposureNode::ExposureNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs)
     : Node(inputs, outputs), _exposure_factor(EXPOSURE_FACTOR_RANGE[0], EXPOSURE_FACTOR_RANGE[1]) {}
 void ExposureNode::init(float exposure_factor) { _exposure_factor.set_param(exposure_factor); }

@@ -291,6 +291,37 @@ class GammaNode : public Node {
     static constexpr float GAMMA_RANGE[2] = {0.3f, 7.00f};
 };
 
+// effects_augmentations/node_normalize.cpp:28-123: mean / standard deviation over the axes of `axes`, given or computed (an empty
+// vector = computed), then scale and shift. Image tensors: axes {0,1} (per channel) or {0,1,2} (per sample).
+class NormalizeNode : public Node {
+   public:
+    NormalizeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(std::vector<unsigned> &axes, std::vector<float> &mean, std::vector<float> &std_dev, float scale, float shift);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    int _axis_mask = 0;
+    std::vector<float> _mean, _std_dev;
+    float _scale = 1.0f, _shift = 0.0f;
+};
+
+// geometry_augmentations/node_transpose.cpp:28-83: perm = the input's axes (batch axis left out) in output order
+class TransposeNode : public Node {
+   public:
+    TransposeNode(const std::vector<Tensor *> &inputs, const std::vector<Tensor *> &outputs);
+    void init(std::vector<unsigned> perm);
+
+   protected:
+    void create_node() override;
+    void update_node() override;
+
+   private:
+    std::vector<unsigned> _perm;
+};
+
 // node_exposure.cpp:28-60 (range node_exposure.h:42)
 class ExposureNode : public Node {
    public:

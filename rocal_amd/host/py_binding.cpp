@@ -38,6 +38,17 @@ PY_API RocalTensor rocalpy_crop_mirror_normalize(RocalContext ctx, RocalTensor i
                                     (RocalTensorOutputType)dtype);
 }
 
+PY_API RocalTensor rocalpy_normalize(RocalContext ctx, RocalTensor in, const unsigned *axes, unsigned n_axes, const float *mean, unsigned n_mean,
+                                     const float *std_dev, unsigned n_std, bool is_output, float scale, float shift, int dtype) {
+    std::vector<unsigned> ax(axes, axes + (axes ? n_axes : 0));
+    std::vector<float> m = vec(mean, n_mean), s = vec(std_dev, n_std);
+    return rocalNormalize(ctx, in, ax, m, s, is_output, scale, shift, (RocalTensorOutputType)dtype);
+}
+
+PY_API RocalTensor rocalpy_transpose(RocalContext ctx, RocalTensor in, const unsigned *perm, unsigned n_perm, bool is_output, int layout) {
+    return rocalTranspose(ctx, in, std::vector<unsigned>(perm, perm + (perm ? n_perm : 0)), is_output, (RocalTensorLayout)layout);
+}
+
 PY_API int rocalpy_set_outputs(RocalContext ctx, unsigned n, RocalTensor *tensors) {
     try {
         std::vector<RocalTensor> v(tensors, tensors + n);

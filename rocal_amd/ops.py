@@ -310,6 +310,34 @@ class ColorTemperature(Op):
         self._update("rmx_update_color_temperature", (src_roi, _U), (adjustment, np.int32))
 
 
+class Normalize(Op):
+    """Per-sample normalisation over height and width (axis_mask 3) or height, width and channels (7); mean / stddev None = computed."""
+    _create = "rmx_create_normalize"
+
+    def update(self, src_roi, axis_mask=3, mean=None, stddev=None, scale=1.0, shift=0.0):
+        roi, proi = _arr(src_roi, _U)
+        m, pm = _arr(mean, _F)
+        s, ps = _arr(stddev, _F)
+        n_stats = m.size if m is not None else (s.size if s is not None else 0)
+        if m is not None and s is not None:
+            assert m.size == s.size
+        check(_lib.lib().rmx_update_normalize(self._h, proi, int(axis_mask), pm, ps, int(n_stats), float(scale), float(shift)))
+
+
+class Transpose(Op):
+    """perm: the source's (height, width, channels) axes in output order: (0,1,2), (2,0,1), (1,0,2) or (2,1,0)."""
+
+    def __init__(self, ctx, src_desc, dst_desc, perm, roi_type=ROI_XYWH):
+        self.ctx = ctx
+        self.src_desc, self.dst_desc = src_desc, dst_desc
+        self._h = C.c_void_p()
+        p = np.ascontiguousarray(perm, np.uint32)
+        check(_lib.lib().rmx_create_transpose(ctx._h, C.byref(src_desc), C.byref(dst_desc), p.ctypes.data_as(C.c_void_p), int(roi_type), C.byref(self._h)))
+
+    def update(self, src_roi=None):
+        self._update("rmx_update_transpose", (src_roi, _U))
+
+
 class Blend(Op):
     """Two source batches of one shape; launch(src1, src2, dst)."""
     _create = "rmx_create_blend"

@@ -124,6 +124,15 @@ def test_flip_warp_rotate_crop(rec):
     assert rec.calls[-1] == ("randomCrop", "H", "in", False, ("FU", 0.08, 1.0), ("FU", 0.75, 1.333333), None, None, 20, NHWC, U8)
 
 
+def test_normalize_and_transpose(rec):
+    fn.normalize("in")
+    assert rec.calls[-1] == ("normalize", "H", "in", [], [], [], False, 1.0, 0.0, types.FLOAT)
+    fn.normalize("in", axes=[0, 1], mean=[1.0], stddev=[2.0], scale=3.0, shift=4.0, output_dtype=types.FLOAT16)
+    assert rec.calls[-1] == ("normalize", "H", "in", [0, 1], [1.0], [2.0], False, 3.0, 4.0, types.FLOAT16)
+    fn.transpose("in", perm=[2, 0, 1], output_layout=types.NCHW)
+    assert rec.calls[-1] == ("transpose", "H", "in", [2, 0, 1], False, types.NCHW)
+
+
 def test_fn_needs_a_current_pipeline(monkeypatch):
     monkeypatch.setattr(pipeline.Pipeline, "_current_pipeline", None)
     with pytest.raises(RuntimeError, match="with pipeline"):

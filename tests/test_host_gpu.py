@@ -251,6 +251,23 @@ def test_tensor_read_as_a_second_input_is_not_fused_away(tmp_path):
         _same(o[2][0], orc.blend(other, mid, whole, np.full(N, 0.25, np.float32)), "blend with the resized tensor as second input")
 
 
+def test_normalize_and_transpose_nodes(tmp_path):
+    """rocalNormalize (computed per-channel statistics; given statistics with scale and shift) and rocalTranspose ({1,0,2} and
+    {2,0,1}) on the ragged source: values from the oracle / numpy, output ROIs swapped where the permutation swaps."""
+    img, outs, _ = _run("normalize_transpose", tmp_path, 4, [(np.float32, (N, H, W, 3)), (np.float16, (N, H, W, 3)), (np.uint8, (N, W, H, 3)),
+                                                             (np.uint8, (N, 3, H, W))])
+    e0 = orc.normalize(img, _roi(), axis_mask=3, layout=orc.NHWC, dtype=orc.FP32)
+    e1 = orc.normalize(img, _roi(), axis_mask=7, mean=[10.0, 20.0, 30.0], stddev=[2.0, 4.0, 8.0], scale=3.0, shift=1.0, layout=orc.NHWC, dtype=orc.FP16)
+    for o in outs:
+        for i, (w, h) in enumerate(ROIS):
+            _same(o[0][0][i, :h, :w], e0[i, :h, :w], "normalize, computed statistics, sample %d" % i)
+            _same(o[1][0][i, :h, :w], e1[i, :h, :w], "normalize, given statistics, sample %d" % i)
+            _same(o[2][0][i, :w, :h], np.ascontiguousarray(img[i, :h, :w].transpose(1, 0, 2)), "transpose {1,0,2}, sample %d" % i)
+            _same(o[3][0][i, :, :h, :w], np.ascontiguousarray(img[i, :h, :w].transpose(2, 0, 1)), "transpose {2,0,1}, sample %d" % i)
+        assert np.array_equal(o[2][1][:, 2:], np.array([[h, w] for w, h in ROIS]))  # width and height swapped
+        assert np.array_equal(o[3][1][:, 2:], np.array([[w, h] for w, h in ROIS]))
+
+
 def test_to_tensor_of_the_u8_output(tmp_path):
     """rocalToTensor (rocal_api_data_transfer.cpp:30-52 -> MasterGraph::to_tensor): planar fp16 with reversed
     channels of the whole output, then an interleaved fp32 tensor of its top-left max_roi corner."""

@@ -265,3 +265,51 @@ def test_color_twist_reciprocal_form_within_one_level_of_division_form_on_all_rg
     if (alpha, beta, hue, sat) == TWIST_SETS[0]:
         # identity parameters: the round trip reproduces every input triple to within one level
         assert np.abs(out - rgb.astype(np.int32)).max() <= 1
+
+
+# ------------------------------------------------------------------ normalize: numpy statistics, hand-computed cases
+
+def test_normalize_matches_numpy_statistics():
+    rng = np.random.default_rng(31)
+    n, h, w = 3, 20, 27
+    img = _img(n, h, w, rng)
+    roi = np.array([[0, 0, w, h], [3, 2, 11, 9], [5, 5, 1, 7]], np.uint32)
+    for mask in (3, 7):
+        out = orc.normalize(img, roi, axis_mask=mask, scale=2.0, shift=-0.5)
+        for i in range(n):
+            x0, y0, ww, hh = [int(v) for v in roi[i]]
+            win = img[i, y0:y0 + hh, x0:x0 + ww].astype(np.float64)
+            axes = (0, 1) if mask == 3 else (0, 1, 2)
+            mu, sd = win.mean(axis=axes, keepdims=True), win.std(axis=axes, keepdims=True)  # population standard deviation
+            with np.errstate(divide="ignore", invalid="ignore"):
+                exp = np.where(sd > 0, (win - mu) / sd * 2.0 - 0.5, -0.5)
+            assert np.abs(out[i, :hh, :ww] - exp).max() < 2e-4, (mask, i)
+    # given statistics: one value, and one per channel
+    out = orc.normalize(img, roi, mean=[100.0], stddev=[50.0])
+    assert np.abs(out[0] - (img[0].astype(np.float64) - 100.0) / 50.0).max() < 1e-5
+    out = orc.normalize(img, roi, mean=[10.0, 20.0, 30.0], stddev=[2.0, 4.0, 8.0], scale=3.0, shift=1.0)
+    exp = (img[0].astype(np.float64) - [10.0, 20.0, 30.0]) / [2.0, 4.0, 8.0] * 3.0 + 1.0
+    assert np.abs(out[0] - exp).max() < 1e-4
+    # a given mean with a computed deviation: the deviation is taken around the GIVEN mean
+    out = orc.normalize(img, roi[:1], mean=[0.0], axis_mask=7)
+    rms = np.sqrt((img[0].astype(np.float64) ** 2).mean())
+    assert np.abs(out[0] - img[0] / rms).max() < 1e-5
+
+
+def test_normalize_hand_computed_cases():
+    # constant image: deviation 0 -> every value becomes the shift
+    img = np.full((1, 4, 6, 3), 77, np.uint8)
+    out = orc.normalize(img, _full(1, 4, 6), shift=0.25)
+    assert (out == 0.25).all()
+    # half 10, half 30 in every channel: mean 20, deviation 10 -> -1 and +1 exactly
+    img = np.empty((1, 4, 6, 3), np.uint8)
+    img[:, :, :3] = 10
+    img[:, :, 3:] = 30
+    out = orc.normalize(img, _full(1, 4, 6))
+    assert (out[0, :, :3] == -1.0).all() and (out[0, :, 3:] == 1.0).all()
+    # channels 0 / 100 / 200, all axes: mean 100, deviation sqrt(20000/3)
+    img = np.zeros((1, 2, 2, 3), np.uint8)
+    img[..., 1], img[..., 2] = 100, 200
+    out = orc.normalize(img, _full(1, 2, 2), axis_mask=7)
+    assert np.allclose(out[0, 0, 0], [-100 / math.sqrt(20000 / 3), 0.0, 100 / math.sqrt(20000 / 3)], atol=1e-6)
+    assert abs(out[0, 0, 0, 1]) < 1e-6  # fma(x, a, fma(-mean, a, 0)): the rounding of mean * a is all that is left
