@@ -82,7 +82,7 @@ def build_case(cfg, ctx, n=None):
                 op.update_cmn(c["roi"], dw, dw, scale, bias, c["mirror"])
             else:
                 rng = np.random.default_rng(99000 + j)
-                roi = np.array([wl.rrc_window(rng, int(c["H"][i]), int(c["W"][i])) for i in range(n)], np.uint32)
+                roi = wl.random_crop_dec_windows(99000 + j, c["H"], c["W"])
                 op.update_cmn(roi, dw, dw, scale, bias, (rng.random(n) < 0.5).astype(np.uint32))
         update(0)
 

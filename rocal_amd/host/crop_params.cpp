@@ -137,3 +137,82 @@ void RocalRandomCropParam::update_array() {
         y2_arr_val[i] = y1_arr_val[i] + ch;
     }
 }
+
+// ---- decoder-side random crop ----
+
+RocalRandomCropDecParam::RocalRandomCropDecParam(AspectRatioRange aspect, AreaRange area, int64_t /*seed: unused by rocAL too*/, int num_attempts,
+                                                 int batch_size)
+    : _aspect_ratio_range(aspect),
+      _aspect_ratio_log_dis(std::log(aspect.first), std::log(aspect.second)),
+      _area_dis(area.first, area.second),
+      _seeds(batch_size),
+      _num_attempts(num_attempts),
+      _batch_size(batch_size) {}
+
+// parameter_random_crop_decoder.cpp:42-100. Kept from the reference because they decide the result: integer
+// products compared against a float area, float->int truncation of the side limits, roundf of the square roots,
+// the ratio test on the ROUNDED sides, the fallback that shrinks both sides by sqrt(scale) one after the other
+// (the second product sees the already shrunk width), and both position draws even when their range is a single value.
+CropWindow RocalRandomCropDecParam::window_for(const Shape &shape, std::mt19937 &gen) {
+    if (shape.size() != 2) THROW("RocalRandomCropDecParam: shape must be {height, width}")
+    CropWindow crop;
+    const int H = (int)shape[0], W = (int)shape[1];
+    if (W <= 0 || H <= 0) return crop;
+    const float min_wh = _aspect_ratio_range.first, max_wh = _aspect_ratio_range.second;
+    const float max_hw = 1 / _aspect_ratio_range.first;
+    const float min_area = W * H * _area_dis.a();
+    const int max_w = std::max<int>(1, H * max_wh);
+    const int max_h = std::max<int>(1, W * max_hw);
+    if (H * max_w < min_area) {  // too wide for any window of the smallest area
+        crop.set_shape(H, max_w);
+    } else if (W * max_h < min_area) {  // too tall
+        crop.set_shape(max_h, W);
+    } else {
+        int left = _num_attempts;
+        for (; left > 0; left--) {
+            const float scale = _area_dis(gen);
+            const size_t whole = (size_t)(H * W);
+            const float target = scale * whole;
+            float ratio = std::exp(_aspect_ratio_log_dis(gen));
+            const int w = std::max(1, (int)std::roundf(sqrtf(target * ratio)));
+            const int h = std::max(1, (int)std::roundf(sqrtf(target / ratio)));
+            crop.set_shape(h, w);
+            ratio = (float)w / h;
+            if (w <= W && h <= H && ratio >= min_wh && ratio <= max_wh) break;
+        }
+        if (left <= 0) {
+            const float max_area = _area_dis.b() * W * H;
+            const float ratio = (float)W / H;
+            if (ratio > max_wh)
+                crop.set_shape(H, max_w);
+            else if (ratio < min_wh)
+                crop.set_shape(max_h, W);
+            else
+                crop.set_shape(H, W);
+            const float scale = std::min(1.0f, max_area / (crop.W * crop.H));
+            crop.W = std::max<int>(1, crop.W * std::sqrt(scale));
+            crop.H = std::max<int>(1, crop.H * std::sqrt(scale));
+        }
+    }
+    crop.x = std::uniform_int_distribution<int>(0, W - crop.W)(gen);
+    crop.y = std::uniform_int_distribution<int>(0, H - crop.H)(gen);
+    return crop;
+}
+
+CropWindow RocalRandomCropDecParam::generate_crop_window(const Shape &shape, int instance) {
+    if (instance < 0 || instance >= _batch_size) THROW("RocalRandomCropDecParam: instance outside the batch")
+    // one engine per thread, re-seeded per sample (parameter_random_crop_decoder.cpp:103-106)
+    static thread_local std::mt19937 gen;
+    gen.seed(_seeds[instance]);
+    return window_for(shape, gen);
+}
+
+void RocalRandomCropDecParam::generate_random_seeds() {
+    ParameterFactory::instance()->generate_seed();
+    generate_seeds_from(ParameterFactory::instance()->get_seed());
+}
+
+void RocalRandomCropDecParam::generate_seeds_from(unsigned master_seed) {
+    std::seed_seq seq{master_seed};
+    seq.generate(_seeds.begin(), _seeds.end());
+}

@@ -2,11 +2,15 @@
 //   CropParam            rocAL/include/parameters/parameter_crop.h:36-92
 //   RocalCropParam       rocAL/source/parameters/parameter_rocal_crop.cpp:44-85   (fixed / anchored / factor crops)
 //   RocalRandomCropParam rocAL/source/parameters/parameter_random_crop.cpp:44-100 (area + aspect-ratio crops)
+//   RocalRandomCropDecParam rocAL/source/parameters/parameter_random_crop_decoder.cpp:42-112 (the decoder-side
+//                        random-resized-crop law: retries, fallback, integer position, one seed per sample)
 // The windows feed the crop ROI argument of rmx_update_*(); the arithmetic (truncations, nearbyintf,
 // number and order of random draws) is the part that has to agree with the reference.
 #pragma once
 #include <cmath>
 #include <cstdint>
+#include <random>
+#include <utility>
 #include <vector>
 
 #include "parameters.h"
@@ -83,4 +87,38 @@ class RocalRandomCropParam : public CropParam {
     static constexpr float AREA_FACTOR_RANGE[2] = {0.08f, 0.99f};
     static constexpr float ASPECT_RATIO_RANGE[2] = {0.7500f, 1.333f};
     Parameter<float> *area_factor, *aspect_ratio;
+};
+
+// Window of the decoder-side random crop: x, y, then height and width (parameter_random_crop_decoder.h:29-39).
+struct CropWindow {
+    unsigned x = 0, y = 0, H = 1, W = 1;
+    CropWindow() = default;
+    CropWindow(unsigned x1, unsigned y1, unsigned h, unsigned w) : x(x1), y(y1), H(h), W(w) {}
+    void set_shape(unsigned h, unsigned w) { H = h, W = w; }
+};
+
+typedef std::vector<size_t> Shape;  // {height, width}
+using AspectRatioRange = std::pair<float, float>;
+using AreaRange = std::pair<float, float>;
+
+// Random-resized-crop windows as rocAL's fused decoders draw them (parameter_random_crop_decoder.h:45-71): the
+// engine is re-seeded per sample from a per-batch seed list, so a sample's window depends on its slot only.
+// The draws per window are: up to num_attempts pairs (area fraction, log aspect ratio), then x, then y.
+class RocalRandomCropDecParam {
+   public:
+    explicit RocalRandomCropDecParam(AspectRatioRange aspect_ratio_range = {3.0f / 4, 4.0f / 3}, AreaRange area_range = {0.08f, 1.0f},
+                                     int64_t seed = 0, int num_attempts = 10, int batch_size = 256);
+    CropWindow generate_crop_window(const Shape &shape, int instance);
+    // Renews the factory's master seed from the random device and expands it (parameter_random_crop_decoder.cpp:108-112).
+    void generate_random_seeds();
+    // The same expansion from a given master seed: reproducible batches.
+    void generate_seeds_from(unsigned master_seed);
+    const std::vector<int> &seeds() const { return _seeds; }
+
+   private:
+    CropWindow window_for(const Shape &shape, std::mt19937 &gen);
+    AspectRatioRange _aspect_ratio_range;
+    std::uniform_real_distribution<float> _aspect_ratio_log_dis, _area_dis;
+    std::vector<int> _seeds;
+    int _num_attempts, _batch_size;
 };

@@ -1,8 +1,10 @@
 // Plain-C doorway for Python (ctypes) onto the entry points that take C++ types, standing where the reference's pybind
 // module stands (rocAL_pybind/rocal_pybind.cpp): vectors travel as pointer + length. Every other rocal* entry point takes
 // PODs only and is called by ctypes directly.
+#include <cstdio>
 #include <vector>
 
+#include "crop_params.h"
 #include "rocal_api_mi355x.h"
 
 #define PY_API extern "C" __attribute__((visibility("default")))
@@ -66,4 +68,26 @@ PY_API void rocalpy_timing(RocalContext ctx, unsigned long long out[5]) {
     out[1] = t.decode_time;
     out[2] = t.process_time;
     out[3] = t.transfer_time;
+}
+
+// Windows of the decoder-side random-resized crop for a batch of image shapes (hw = height,width pairs), from a
+// master seed: what rocAL's fused decoders draw per sample (parameter_random_crop_decoder.cpp:42-112).
+// Writes x,y,w,h per sample and returns 0, or -1 with the message left for rocalGetErrorMessage-style callers on stderr.
+PY_API int rocalpy_random_crop_dec_windows(unsigned master_seed, unsigned n, const unsigned *hw, float aspect_lo, float aspect_hi, float area_lo,
+                                           float area_hi, int num_attempts, unsigned *xywh) {
+    try {
+        RocalRandomCropDecParam law({aspect_lo, aspect_hi}, {area_lo, area_hi}, 0, num_attempts, (int)n);
+        law.generate_seeds_from(master_seed);
+        for (unsigned i = 0; i < n; i++) {
+            const CropWindow w = law.generate_crop_window({hw[2 * i], hw[2 * i + 1]}, (int)i);
+            xywh[4 * i + 0] = w.x;
+            xywh[4 * i + 1] = w.y;
+            xywh[4 * i + 2] = w.W;
+            xywh[4 * i + 3] = w.H;
+        }
+        return 0;
+    } catch (const std::exception &e) {
+        fprintf(stderr, "rocalpy_random_crop_dec_windows: %s\n", e.what());
+        return -1;
+    }
 }

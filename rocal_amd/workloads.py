@@ -20,49 +20,22 @@ def smooth_noise(rng, n, h, w, sigma=3.0):
     return out
 
 
-def fast_smooth_noise(rng, n, h, w):
-    """Cheap smooth field for full-size batches: low-resolution noise upsampled bilinearly."""
-    out = np.empty((n, h, w, 3), np.uint8)
-    gh, gw = h // 8 + 2, w // 8 + 2
-    ys = np.linspace(0, gh - 1.001, h, dtype=np.float32)
-    xs = np.linspace(0, gw - 1.001, w, dtype=np.float32)
-    y0, x0 = ys.astype(np.int32), xs.astype(np.int32)
-    wy, wx = (ys - y0)[:, None, None], (xs - x0)[None, :, None]
-    for i in range(n):
-        g = rng.random((gh, gw, 3), dtype=np.float32) * 255.0
-        a = g[y0][:, x0] * (1 - wx) + g[y0][:, x0 + 1] * wx
-        b = g[y0 + 1][:, x0] * (1 - wx) + g[y0 + 1][:, x0 + 1] * wx
-        out[i] = np.rint(a * (1 - wy) + b * wy).astype(np.uint8)
+def random_crop_dec_windows(master_seed, H, W, area=(0.08, 1.0), ratio=(3.0 / 4.0, 4.0 / 3.0), attempts=10):
+    """Random-resized-crop windows (x, y, w, h per sample) drawn by the host layer's RocalRandomCropDecParam, the law of
+    rocAL's fused decoders (rocAL/source/parameters/parameter_random_crop_decoder.cpp:42-112): per-sample engines seeded from
+    seed_seq{master_seed}, area fraction uniform, aspect ratio log-uniform, rounded sides, ten attempts, fallback, uniform
+    integer position."""
+    import ctypes as C
+    from . import backend
+    n = len(H)
+    hw = np.ascontiguousarray(np.stack([np.asarray(H), np.asarray(W)], axis=1), dtype=np.uint32)
+    out = np.empty((n, 4), np.uint32)
+    fn = backend.host().rocalpy_random_crop_dec_windows
+    fn.restype = C.c_int
+    fn.argtypes = [C.c_uint, C.c_uint, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int, C.c_void_p]
+    if fn(int(master_seed) & 0xFFFFFFFF, n, hw.ctypes.data, ratio[0], ratio[1], area[0], area[1], attempts, out.ctypes.data) != 0:
+        raise RuntimeError("rocalpy_random_crop_dec_windows failed")
     return out
-
-
-def rrc_window(rng, H, W, area=(0.08, 1.0), ratio=(3.0 / 4.0, 4.0 / 3.0), attempts=10):
-    """Random-resized-crop window law of rocAL's decoder-side generator
-    (rocAL/source/parameters/parameter_random_crop_decoder.cpp:42-100): area fraction uniform,
-    aspect ratio log-uniform, rounded sides, retry, centre-ish fallback, uniform integer position."""
-    min_r, max_r = ratio
-    w = h = None
-    for _ in range(attempts):
-        scale = np.float32(rng.uniform(area[0], area[1]))
-        target = scale * np.float32(H * W)
-        r = np.float32(math.exp(rng.uniform(math.log(min_r), math.log(max_r))))
-        cw = max(1, int(np.round(np.sqrt(target * r))))
-        ch = max(1, int(np.round(np.sqrt(target / r))))
-        rr = cw / ch
-        if cw <= W and ch <= H and min_r <= rr <= max_r:
-            w, h = cw, ch
-            break
-    if w is None:
-        rr = W / H
-        if rr > max_r:
-            h, w = H, max(1, int(H * max_r))
-        elif rr < min_r:
-            h, w = max(1, int(W / min_r)), W
-        else:
-            h, w = H, W
-    x = int(rng.integers(0, W - w + 1))
-    y = int(rng.integers(0, H - h + 1))
-    return x, y, w, h
 
 
 def config0(n=128, seed=1234):
@@ -74,17 +47,17 @@ def config0(n=128, seed=1234):
     return dict(img=img, crop=crop, mirror=mirror, out_h=224, out_w=224)
 
 
-def config1(n=256, seed=1235, hw_range=(240, 640), smooth="fast"):
-    """RandomResizedCrop + CMN, ragged batch -> 224x224 fp16 NCHW."""
+def config1(n=256, seed=1235, hw_range=(240, 640), sigma=3.0):
+    """RandomResizedCrop + CMN, ragged batch -> 224x224 fp16 NCHW. Pixels: Gaussian-blurred uniform noise; windows: the
+    decoder-side random-crop law with master seed `seed`."""
     rng = np.random.default_rng(seed)
     hmax = wmax = hw_range[1]
     H = rng.integers(hw_range[0], hw_range[1] + 1, n)
     W = rng.integers(hw_range[0], hw_range[1] + 1, n)
     img = np.zeros((n, hmax, wmax, 3), np.uint8)
-    gen = fast_smooth_noise if smooth == "fast" else smooth_noise
     for i in range(n):
-        img[i, :H[i], :W[i]] = gen(rng, 1, int(H[i]), int(W[i]))[0]
-    roi = np.array([rrc_window(rng, int(H[i]), int(W[i])) for i in range(n)], np.uint32)
+        img[i, :H[i], :W[i]] = smooth_noise(rng, 1, int(H[i]), int(W[i]), sigma)[0]
+    roi = random_crop_dec_windows(seed, H, W)
     mirror = (rng.random(n) < 0.5).astype(np.uint32)
     return dict(img=img, roi=roi, mirror=mirror, out_h=224, out_w=224, H=H, W=W)
 
@@ -110,11 +83,10 @@ def inverse_affine(theta_deg, scale, tx, ty):
     return m
 
 
-def config3(n=128, seed=1237, size=512, smooth="fast"):
+def config3(n=128, seed=1237, size=512, sigma=3.0):
     """WarpAffine: rotation +-30 deg, scale 0.9..1.1, translation +-16 px; u8 NHWC size x size."""
     rng = np.random.default_rng(seed)
-    gen = fast_smooth_noise if smooth == "fast" else smooth_noise
-    img = gen(rng, n, size, size)
+    img = smooth_noise(rng, n, size, size, sigma)
     roi = np.tile(np.array([0, 0, size, size], np.uint32), (n, 1))
     affine = np.empty((n, 6), np.float32)
     for i in range(n):
@@ -124,12 +96,11 @@ def config3(n=128, seed=1237, size=512, smooth="fast"):
     return dict(img=img, roi=roi, affine=affine, out_h=size, out_w=size)
 
 
-def config4(n=32, seed=1238, src_hw=(1080, 1920), dst_hw=(360, 640), smooth="fast"):
+def config4(n=32, seed=1238, src_hw=(1080, 1920), dst_hw=(360, 640), sigma=3.0):
     """Triangular downscale of large images + normalise + mirror -> fp16 NCHW."""
     rng = np.random.default_rng(seed)
     h, w = src_hw
-    gen = fast_smooth_noise if smooth == "fast" else smooth_noise
-    img = gen(rng, n, h, w)
+    img = smooth_noise(rng, n, h, w, sigma)
     sp = rng.random((n, h, w))
     img[sp < 0.025] = 0
     img[sp > 0.975] = 255

@@ -159,3 +159,143 @@ def test_box_laws_known_answers():
     # overlap measure: intersection over the first box's area, or over the union
     assert meta.overlap((0, 0, 10, 10), (5, 5, 15, 15)) == 0.25
     assert abs(meta.overlap((0, 0, 10, 10), (5, 5, 15, 15), True) - 25.0 / 175.0) < 1e-7
+
+
+# ---- decoder-side random-resized-crop law (RocalRandomCropDecParam) ----
+# The C++ class draws with libstdc++'s distributions. The expectation below restates those algorithms from their published
+# definitions over the oracle's generator: generate_canonical<float,24> on a 32-bit engine (one draw, divided by 2^32 in
+# float arithmetic, 1.0 replaced by the float below it) and uniform_int_distribution<int> on a 32-bit engine (Lemire's
+# multiply-shift with rejection). libm supplies logf / expf / sqrtf / roundf, as it does for the C++ class.
+
+def _libm():
+    import ctypes as C
+    m = C.CDLL("libm.so.6")
+    for f in ("logf", "expf", "sqrtf", "roundf"):
+        getattr(m, f).restype = C.c_float
+        getattr(m, f).argtypes = [C.c_float]
+    return m
+
+
+class _StdDraws:
+    def __init__(self, seed):
+        self.g = orc.MT19937(int(seed) & 0xFFFFFFFF)
+        self.draws = 0
+
+    def raw(self):
+        self.draws += 1
+        return self.g.next()
+
+    def canonical(self):
+        r = np.float32(self.raw()) / np.float32(4294967296.0)
+        return np.nextafter(np.float32(1), np.float32(0)) if r >= np.float32(1) else r
+
+    def real(self, a, b):
+        a, b = np.float32(a), np.float32(b)
+        return np.float32(np.float32(self.canonical() * np.float32(b - a)) + a)
+
+    def integer(self, lo, hi):
+        rng_ = hi - lo + 1
+        prod = self.raw() * rng_
+        low = prod & 0xFFFFFFFF
+        if low < rng_:
+            thresh = ((1 << 32) - rng_) % rng_
+            while low < thresh:
+                prod = self.raw() * rng_
+                low = prod & 0xFFFFFFFF
+        return lo + (prod >> 32)
+
+
+def _dec_window(seed, H, W, area=(0.08, 1.0), ratio=(3.0 / 4.0, 4.0 / 3.0), attempts=10):
+    m, f32 = _libm(), np.float32
+    d = _StdDraws(seed)
+    lo_r, hi_r = f32(ratio[0]), f32(ratio[1])
+    log_lo, log_hi = f32(m.logf(lo_r)), f32(m.logf(hi_r))
+    a_lo, a_hi = f32(area[0]), f32(area[1])
+    max_hw = f32(1) / lo_r
+    min_area = f32(W * H) * a_lo
+    max_w = max(1, int(f32(H) * hi_r))
+    max_h = max(1, int(f32(W) * max_hw))
+    if f32(H * max_w) < min_area:
+        h, w = H, max_w
+    elif f32(W * max_h) < min_area:
+        h, w = max_h, W
+    else:
+        for _ in range(attempts):
+            scale = d.real(a_lo, a_hi)
+            target = f32(scale * f32(H * W))
+            r = f32(m.expf(d.real(log_lo, log_hi)))
+            w = max(1, int(m.roundf(m.sqrtf(f32(target * r)))))
+            h = max(1, int(m.roundf(m.sqrtf(f32(target / r)))))
+            rr = f32(w) / f32(h)
+            if w <= W and h <= H and lo_r <= rr <= hi_r:
+                break
+        else:
+            max_area = f32(f32(a_hi * f32(W)) * f32(H))
+            rr = f32(W) / f32(H)
+            if rr > hi_r:
+                h, w = H, max_w
+            elif rr < lo_r:
+                h, w = max_h, W
+            else:
+                h, w = H, W
+            s = min(f32(1), max_area / f32(w * h))
+            rs = f32(m.sqrtf(s))
+            w = max(1, int(f32(w) * rs))
+            h = max(1, int(f32(h) * rs))
+    x = d.integer(0, W - w)
+    y = d.integer(0, H - h)
+    return (x, y, w, h), d.draws
+
+
+def _host_windows(seed, shapes, **kw):
+    from rocal_amd import workloads as wl
+    return wl.random_crop_dec_windows(seed, [s[0] for s in shapes], [s[1] for s in shapes], **kw)
+
+
+def test_decoder_crop_windows_follow_the_reference_law():
+    rng = np.random.default_rng(8)
+    shapes = [(int(rng.integers(240, 641)), int(rng.integers(240, 641))) for _ in range(256)]
+    shapes += [(1, 1), (2, 3), (3, 2), (5, 5), (7, 1), (1, 9), (16, 4000), (4000, 16)]
+    seeds = orc.seed_seq_generate([1235], len(shapes))
+    got = _host_windows(1235, shapes)
+    retried = 0
+    for i, (H, W) in enumerate(shapes):
+        exp, draws = _dec_window(seeds[i], H, W)
+        assert tuple(int(v) for v in got[i]) == exp, "sample %d (%dx%d)" % (i, H, W)
+        retried += draws > 4
+    assert retried >= 20  # the retry branch is exercised (about a fifth of ImageNet-like shapes need a second attempt)
+    x, y, w, h = got[:, 0].astype(int), got[:, 1].astype(int), got[:, 2].astype(int), got[:, 3].astype(int)
+    Hs, Ws = np.array([s[0] for s in shapes]), np.array([s[1] for s in shapes])
+    assert np.all(w >= 1) and np.all(h >= 1) and np.all(x + w <= Ws) and np.all(y + h <= Hs)
+
+
+def test_decoder_crop_windows_hand_computed_cases():
+    # Too wide (H=10, W=1000): max width = int(10 * 4/3) = 13; 10*13 = 130 < 0.08*10000 = 800 -> 10 x 13 without any
+    # attempt; y has a single possible value. Too tall is the transpose: max height = int(10 / 0.75) = 13.
+    got = _host_windows(7, [(10, 1000), (1000, 10)])
+    assert got[0, 2:].tolist() == [13, 10] and got[0, 1] == 0 and 0 <= got[0, 0] <= 987
+    assert got[1, 2:].tolist() == [10, 13] and got[1, 0] == 0 and 0 <= got[1, 1] <= 987
+    # A degenerate law (area exactly 1, ratio exactly 1) on a square image: sqrt(H*W) = H, the whole image, at (0, 0).
+    got = _host_windows(7, [(64, 64), (300, 300)], area=(1.0, 1.0), ratio=(1.0, 1.0))
+    assert got.tolist() == [[0, 0, 64, 64], [0, 0, 300, 300]]
+    # The same law on a 2:1 image can never satisfy h <= H: after ten attempts the fallback takes the side limits
+    # (ratio 2 > 1 -> H x int(H*1)), area scale min(1, W*H / (H*H)) = 1 -> a centred-law square of side H, x uniform.
+    got = _host_windows(7, [(100, 200)], area=(1.0, 1.0), ratio=(1.0, 1.0))
+    assert got[0, 2:].tolist() == [100, 100] and got[0, 1] == 0 and 0 <= got[0, 0] <= 100
+    # Fallback with shrink: area at most 0.25 of a 2:1 image, ratio exactly 1, attempts 0 -> H x H scaled by
+    # sqrt(0.25*200*100 / (100*100)) = sqrt(0.5): width int(100*0.70710677) = 70, then height int(100*0.70710677) = 70.
+    got = _host_windows(7, [(100, 200)], area=(0.25, 0.25), ratio=(1.0, 1.0), attempts=0)
+    assert got[0, 2:].tolist() == [70, 70]
+
+
+def test_decoder_crop_windows_statistics():
+    # Large sample on one shape: the area fraction is uniform on [0.08, 1] conditioned on fitting, the position uniform.
+    n = 4000
+    got = _host_windows(99, [(480, 640)] * n).astype(np.float64)
+    frac = got[:, 2] * got[:, 3] / (480 * 640)
+    ratio = got[:, 2] / got[:, 3]
+    assert 0.079 <= frac.min() and frac.max() <= 1.0
+    assert np.all(ratio >= 0.75 - 1e-6) and np.all(ratio <= 4 / 3 + 1e-6)
+    assert abs(np.mean(np.log(ratio))) < 0.05      # log-uniform about 1 (fit conditioning leaves a small tilt)
+    free = 640 - got[:, 2]
+    assert abs(np.mean(got[free > 50, 0] / free[free > 50]) - 0.5) < 0.03
