@@ -53,7 +53,7 @@ def host():
     global _HOST
     if _HOST is None:
         _lib.lib()  # the C-ABI library first: one HIP runtime instance for both
-        path = os.path.join(os.path.dirname(_lib.LIB_PATH), "librocal_mi355x_host.so")
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "librocal_mi355x_host.so")
         if not os.path.exists(path):
             raise _lib.RmxError(-1, "host library not built: %s is missing (run `make -C rocal_amd/host`)" % path)
         h = C.CDLL(path)

@@ -81,7 +81,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -297,6 +297,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->upload_kernel = tune_env("RMX_TUNE_UPLOAD_KERNEL", ctx->upload_kernel, 0, 1);
         ctx->dma = tune_env("RMX_TUNE_DMA", ctx->dma, 0, 1);  // 0: the bilinear fast path always stages through registers
         ctx->dma_lds = tune_env("RMX_TUNE_DMA_LDS", ctx->dma_lds, 2048, 10 * 1024) & ~15;  // LDS window of a wavefront
+        ctx->dma_group = tune_env("RMX_TUNE_DMA_GROUP", ctx->dma_group, 0, 16);  // windows per wavefront, 0: chosen per batch
         ctx->tri_wpb = tune_env("RMX_TUNE_TRI_WPB", ctx->tri_wpb, 1, 4);
         ctx->warp_passes = tune_env("RMX_TUNE_WARP_PASSES", ctx->warp_passes, 1, 8);
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
@@ -343,8 +344,8 @@ const char *rmx_op_plan(const rmx_op *op) {
     static thread_local char buf[256];
     if (!op) return "";
     if (op->fn_fast)
-        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d waves_per_block=%d fast=1",
-                 (long long)op->n * op->fast_strips, op->fast_strips, op->fast_rows, op->fast_lds, op->fast_wpb);
+        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d waves_per_block=%d fast=1 group=%d",
+                 (long long)op->n * op->fast_strips, op->fast_strips, op->fast_rows, op->fast_lds, op->fast_wpb, std::max(1, op->fast_aux1));
     else
         snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=0",
                  (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block);
@@ -978,9 +979,13 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 op->fast_name = dname;
                 op->fast_lds = (need_max + 15) / 16 * 16;
                 op->fast_rows = rows;
-                op->fast_strips = std::max(1, (max_dh + rows - 1) / rows);
+                // A wavefront works through `group` windows (of `rows` destination rows) below each other per x-tile, so that the
+                // tile's x taps are computed once for all of them; as many as still leave about four wavefronts per SIMD.
+                const long windows = (long)op->n * ((max_dh + rows - 1) / rows);
+                const int group = op->ctx->dma_group ? op->ctx->dma_group : (int)std::max<long>(1, std::min<long>(8, windows / 4096));
+                op->fast_strips = std::max(1, (max_dh + rows * group - 1) / (rows * group));
                 op->fast_wpb = std::max(1, std::min(op->ctx->fast_wpb, (op->ctx->max_lds_per_block - kStaticLdsMax) / std::max(1, op->fast_lds)));
-                op->fast_aux1 = 0;
+                op->fast_aux1 = group;
             }
         }
     }

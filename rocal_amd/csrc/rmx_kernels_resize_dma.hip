@@ -26,6 +26,10 @@
 
 #include <type_traits>
 
+#ifndef RMX_DMA_NT
+#define RMX_DMA_NT (sizeof(T) == 2)  // fp16: streaming stores
+#endif
+
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_dma[];
@@ -43,17 +47,27 @@ RMX_DEV float src_coord_d(int u, float ratio, float off, float lo) {
 }
 
 
-// One window: a strip of destination rows x one x-tile. Every member is wave-uniform.
-struct DmaItem {
-    int r0, r1;      // destination rows [r0, r1)
-    int xt, tw;      // destination columns [xt, xt + tw)
-    int a_v, nrows;  // virtual source rows a_v .. a_v + nrows - 1 (clamped into the window when fetched)
+// A wave-uniform value that the vector unit produced (float arithmetic has no scalar form), moved into a scalar register
+// by an instruction the optimiser cannot look through: everything derived from it stays scalar arithmetic. (The
+// readfirstlane builtin is folded away for values known to be uniform, and the dependants then run on the vector unit.)
+// The compiler does not see inside the statement, so the wait states this chip wants around the instruction are spelled
+// out: one between a vector instruction that writes the source register and the read of it, five before a vector memory
+// instruction may read the scalar result (two before a vector ALU instruction may).
+RMX_DEV int to_sgpr(int v) {
+    int r;
+    asm("s_nop 0\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(r) : "v"(v));
+    return r;
+}
+
+// One x-tile of a wavefront's rows: destination columns [xt, xt + tw) and the source columns they read. Wave-uniform.
+struct DmaTile {
+    int xt, tw;
     int cs, nc;      // source columns cs .. cs + nc - 1
     int ph;          // byte phase of pixel cs inside its dword
     int ppr;         // 16-byte pieces per LDS row (margin + data + room for the right replicas)
     int nd;          // data pieces per row
     uint32_t col4;   // byte offset (from base4) of the dword that holds pixel cs, within a row
-    bool rep_l, rep_r, safe;
+    bool rep_l, rep_r;
 };
 
 // CHAIN: a colour node between the (quantised) resize and the normalisation, see chain_colour().
@@ -74,10 +88,10 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.plan[1]));
 
     const int dw = P.dst_w, dh = P.dst_h;
-    const int srows = a.aux0;
-    const int r_begin = grp * srows;
+    const int wrows = a.aux0;                        // destination rows of one window
+    const int r_begin = grp * wrows * max(a.aux1, 1);  // this wavefront: max(aux1, 1) windows below each other
     if (r_begin >= dh || dw <= 0) return;
-    const int r_end = min(r_begin + srows, dh);
+    const int r_end = min(r_begin + wrows * max(a.aux1, 1), dh);
     const bool hf = (P.flags & RMX_S_HFLIP) != 0;
 
     const int xlo = P.src_x, ylo = P.src_y;
@@ -89,7 +103,9 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     const int pcx = P.pc_x, pcy = P.pc_y;
 
     T *dimg = reinterpret_cast<T *>(a.dst) + (size_t)s * 3 * a.dst_h * a.dst_w;
-    uint32_t *lds = rmx_lds_dma + (size_t)wib * (a.lds_bytes >> 2);
+    // (the wavefront's index inside its workgroup comes from a lane id: wave-uniform, but only a scalar register says so)
+    const uint32_t slice_off = (uint32_t)to_sgpr((int)((uint32_t)wib * (uint32_t)a.lds_bytes));
+    lds_u8 *bufb = (lds_u8 *)(lds_ptr_t)rmx_lds_dma + slice_off;
 
     float sc[3], bi[3];
 #pragma unroll
@@ -102,8 +118,11 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     const ColorTables *ctab = reinterpret_cast<const ColorTables *>(chain_tables);
     if constexpr (CHAIN == CHAIN_TWIST) color_tables_fill(reinterpret_cast<ColorTables *>(chain_tables), lane);
 
-    uint32_t row_stride;
-    const uint8_t *simg = sample_base(a, s, row_stride);
+    uint32_t row_stride_v;
+    const uint8_t *simg_v = sample_base(a, s, row_stride_v);
+    const uint32_t row_stride = (uint32_t)to_sgpr((int)row_stride_v);
+    const uint8_t *simg = reinterpret_cast<const uint8_t *>(((uint64_t)(uint32_t)to_sgpr((int)((uintptr_t)simg_v >> 32)) << 32) |
+                                                            (uint32_t)to_sgpr((int)(uint32_t)(uintptr_t)simg_v));
     const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
     const uint8_t *base4 = simg - skew;
     const uint64_t left = (uint64_t)((a.src + a.src_bytes) - base4);
@@ -112,22 +131,15 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     const int tile_w = max(P.plan[1], PX);  // never 0: it is the step of the tile loop
     const int ntx = (dw + tile_w - 1) / tile_w;
 
-    auto make_item = [&](int tile) {
-        DmaItem g;
-        g.r0 = r_begin;
-        g.r1 = r_end;
+    // ---- geometry of an x-tile and of a window of it (all wave-uniform)
+    auto tile_geom = [&](int tile) {
+        DmaTile g;
         g.xt = tile * tile_w;
         g.tw = min(dw - g.xt, tile_w);
-        // (wave-uniform values that come out of the vector unit's float arithmetic: into scalar registers, so that everything
-        // derived from them is scalar arithmetic)
-        g.a_v = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcy + g.r0, ry, offy, fylo)));
-        const int b_v = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcy + g.r1 - 1, ry, offy, fylo))) + 1;
-        g.nrows = b_v - g.a_v + 1;
-        const int ixmin = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcx + g.xt, rx, offx, fxlo)));
-        const int ixmax = __builtin_amdgcn_readfirstlane((int)floorf(src_coord_d(pcx + g.xt + g.tw - 1, rx, offx, fxlo)));
+        const int ixmin = to_sgpr((int)floorf(src_coord_d(pcx + g.xt, rx, offx, fxlo)));
+        const int ixmax = to_sgpr((int)floorf(src_coord_d(pcx + g.xt + g.tw - 1, rx, offx, fxlo)));
         g.cs = max(min(ixmin, xhi), xlo);
-        const int ce = max(min(ixmax + 1, xhi), xlo);
-        g.nc = ce - g.cs + 1;
+        g.nc = max(min(ixmax + 1, xhi), xlo) - g.cs + 1;
         g.rep_l = ixmin < xlo;
         g.rep_r = ixmax + 1 > xhi;
         const uint32_t colb = (uint32_t)g.cs * 3u + skew;
@@ -135,38 +147,40 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         g.col4 = colb & ~3u;
         g.nd = (g.ph + 3 * g.nc + 15) >> 4;
         g.ppr = 1 + ((g.ph + 3 * (g.nc + 2) + 8 + 15) >> 4);
-        const int tp = g.nrows * g.ppr;
-        // every 16-byte piece of every row lies inside the batch buffer (the last rows of the last sample may not)
-        const uint32_t last_row = (uint32_t)max(min(b_v, yhi), ylo) * row_stride + g.col4;
-        g.safe = (uint64_t)last_row + 16ull * (uint64_t)g.nd <= (uint64_t)lim;
         return g;
     };
-
-    // Starts the window's transfer into `buf`. A piece is 16 bytes at a dword-aligned address; the margin piece and the
-    // pieces behind the row's data repeat a neighbouring data piece (their content is never read before a replica is
-    // written over it).
-    auto issue = [&](DmaItem &g, uint32_t *buf) {
-        if (g.safe) {
-            // One load instruction per row and 64 pieces: the row's address is scalar arithmetic, a lane's piece offset is the
-            // same for every row, and consecutive lanes fill consecutive 16-byte slots from (r * ppr + c0) on.
+    // Starts the transfer of the window of destination rows [r0, r1) into the LDS slice and returns its first (virtual)
+    // source row; sets nrows. A piece is 16 bytes at a dword-aligned address; the margin piece and the pieces behind the row's
+    // data repeat a neighbouring data piece (their content is never read before a replica is written over it).
+    int nrows = 0;
+    auto issue = [&](const DmaTile &g, int r0, int r1) {
+        const int a_v = to_sgpr((int)floorf(src_coord_d(pcy + r0, ry, offy, fylo)));
+        const int b_v = to_sgpr((int)floorf(src_coord_d(pcy + r1 - 1, ry, offy, fylo))) + 1;
+        nrows = b_v - a_v + 1;
+        // every 16-byte piece of every row lies inside the batch buffer (the last rows of the last sample may not)
+        const uint32_t last_row = (uint32_t)max(min(b_v, yhi), ylo) * row_stride + g.col4;
+        const bool safe = (uint64_t)last_row + 16ull * (uint64_t)g.nd <= (uint64_t)lim;
+        if (safe) {
+            // One load instruction per row and 64 pieces: the row's address and its LDS slot are scalar arithmetic, a lane
+            // only adds its piece offset, the same for every row; consecutive lanes fill consecutive 16-byte slots.
             for (int c0 = 0; c0 < g.ppr; c0 += RMX_WAVE) {
                 const int c = c0 + lane;
                 const uint32_t lane_off = 16u * (uint32_t)max(min(c - 1, g.nd - 1), 0);
                 if (c < g.ppr) {
-                    for (int r = 0; r < g.nrows; r++) {
-                        const int ysrc = max(min(g.a_v + r, yhi), ylo);
+                    for (int r = 0; r < nrows; r++) {
+                        const int ysrc = max(min(a_v + r, yhi), ylo);
                         const uint8_t *rowp = base4 + ((uint32_t)ysrc * row_stride + g.col4);
-                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(buf + (r * g.ppr + c0) * 4), 16, 0, 0);
+                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(bufb + (r * g.ppr + c0) * 16), 16, 0, 0);
                     }
                 }
             }
         } else {
             // the window touches the last bytes of the batch buffer: bounds-checked byte loads, stored by the lanes
-            const int tp = g.nrows * g.ppr;
+            const int tp = nrows * g.ppr;
             for (int idx = lane; idx < tp; idx += RMX_WAVE) {
                 const int r = idx / g.ppr;
                 const int c = idx - r * g.ppr;
-                const int ysrc = max(min(g.a_v + r, yhi), ylo);
+                const int ysrc = max(min(a_v + r, yhi), ylo);
                 const int piece = max(min(c - 1, g.nd - 1), 0);
                 const uint32_t off = (uint32_t)ysrc * row_stride + g.col4 + 16u * (uint32_t)piece;
                 uint32_t w[4];
@@ -180,56 +194,64 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     }
                     w[i] = v;
                 }
-                lds_u32 *dst4 = (lds_u32 *)(lds_ptr_t)(buf + 4 * idx);
+                lds_u32 *dst4 = (lds_u32 *)(bufb + 16 * idx);
                 dst4[0] = w[0]; dst4[1] = w[1]; dst4[2] = w[2]; dst4[3] = w[3];
             }
         }
+        return a_v;
     };
-
-    // x taps of a tile: byte offset of the left neighbour inside an LDS row (dword part and byte phase) and the weights
+    // A lane's x taps in a tile: byte offset of the left neighbour inside an LDS row (dword part and byte phase), weights
     uint32_t bo4[PX], bsh[PX];
     float wx[PX], omx[PX];
-    int L = 1, G = 1, lr = 0, gl = 0, t0 = 0;
+    int G = 1, lr = 0, x0 = 0;
     bool lane_on = false;
-    auto taps = [&](const DmaItem &g) {
-        L = g.tw / PX;
-        G = RMX_WAVE / L;
+    auto taps = [&](const DmaTile &g) {
+        const int L = g.tw / PX;  // lanes per destination row
+        G = RMX_WAVE / L;         // destination rows per pass
         lr = lane / L;
-        gl = lane - lr * L;
-        t0 = g.xt + gl * PX;
+        const int t0 = g.xt + (lane - lr * L) * PX;
         lane_on = lr < G;
 #pragma unroll
         for (int k = 0; k < PX; k++) {
-            float sx = src_coord_d(pcx + t0 + k, rx, offx, fxlo);
-            float fx = floorf(sx);
+            const float sx = src_coord_d(pcx + t0 + k, rx, offx, fxlo);
+            const float fx = floorf(sx);
             wx[k] = sx - fx;
             omx[k] = 1.0f - wx[k];
             const uint32_t b = (uint32_t)(16 + g.ph + 3 * ((int)fx - g.cs));
             bo4[k] = b & ~3u;
             bsh[k] = b & 3u;
         }
+        x0 = hf ? (dw - t0 - PX) : t0;
     };
 
-    for (int tile = 0; tile < ntx; tile++) {
-        uint32_t *buf = lds;
-        DmaItem cur = make_item(tile);
-        wave_sync();  // the blend of the tile before has read the window for the last time
-        issue(cur, buf);
-        taps(cur);  // while the loads are in flight
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // The wavefront's windows, tile by tile and top to bottom inside a tile. The stores of a window's last pass are held back
+    // in registers until the next window's loads have been started (the LDS slice is free once the blend has read it):
+    // memory operations of a wavefront complete in issue order, so the wait for those loads, which allows the DEFERRED
+    // youngest operations (the held-back stores) to be outstanding, never waits for a store to reach memory.
+    constexpr bool DEFER = sizeof(T) <= 2;  // (an fp32 run is 24 registers: stored at once)
+    constexpr int DEFERRED = 3;             // store instructions of one packed group of 1- and 2-byte elements, both layouts
+    int tile = 0, r0 = r_begin;
+    DmaTile g = tile_geom(0);
+    int a_v = issue(g, r0, min(r0 + wrows, r_end));
+    taps(g);  // while the loads are in flight
+    bool held = false;
+    for (;;) {
+        const int r1 = min(r0 + wrows, r_end);
+        // The compiler does not order LDS reads behind the loads into LDS: await them explicitly, between two fences.
+        if (DEFER && held) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(DEFERRED) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         wave_sync();
-        const int pitch_b = cur.ppr * 16;
-        lds_u8 *bufb = (lds_u8 *)(lds_ptr_t)buf;
+        const int pitch_b = g.ppr * 16;
         // clamp-to-edge: the pixel before the window's first column repeats it, the two after its last column repeat that
-        if (cur.rep_l || cur.rep_r) {
-            for (int rr = lane; rr < cur.nrows; rr += RMX_WAVE) {
-                lds_u8 *row = bufb + rr * pitch_b + 16 + cur.ph;
-                if (cur.rep_l) {
+        if (g.rep_l || g.rep_r) {
+            for (int rr = lane; rr < nrows; rr += RMX_WAVE) {
+                lds_u8 *row = bufb + rr * pitch_b + 16 + g.ph;
+                if (g.rep_l) {
 #pragma unroll
                     for (int b = 0; b < 3; b++) row[b - 3] = row[b];
                 }
-                if (cur.rep_r) {
-                    lds_u8 *lastpx = row + 3 * (cur.nc - 1);
+                if (g.rep_r) {
+                    lds_u8 *lastpx = row + 3 * (g.nc - 1);
 #pragma unroll
                     for (int b = 0; b < 3; b++) lastpx[3 + b] = lastpx[6 + b] = lastpx[b];
                 }
@@ -238,14 +260,17 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         }
 
         // ---- blend, epilogue, store: G rows per pass
-        const int x0 = hf ? (dw - t0 - PX) : t0;
-        for (int rs = cur.r0; rs < cur.r1; rs += G) {
+        PackedGroup<T> packed;
+        bool packed_on = false;
+        int packed_r = 0;
+        for (int rs = r0; rs < r1; rs += G) {
             const int r = rs + lr;
-            if (lane_on && r < cur.r1) {
+            const bool on = lane_on && r < r1;
+            if (on) {
                 float sy = src_coord_d(pcy + r, ry, offy, fylo);
                 float fy = floorf(sy);
                 float wy = sy - fy;
-                const lds_u8 *row0 = bufb + ((int)fy - cur.a_v) * pitch_b;
+                const lds_u8 *row0 = bufb + ((int)fy - a_v) * pitch_b;
                 const lds_u8 *row1 = row0 + pitch_b;
                 const float omy = 1.0f - wy;
                 float v[3][PX];
@@ -262,6 +287,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     float o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte0(br) * wy * wx[k])));
                     float o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte1(br) * wy * wx[k])));
                     if constexpr (QUANT) {
+                        // (a convex blend of bytes stays inside 0..255: rounding is the whole u8 store rule here)
                         o0 = __builtin_rintf(o0); o1 = __builtin_rintf(o1); o2 = __builtin_rintf(o2);
                     }
                     chain_colour<CHAIN>(o0, o1, o2, cp, sh2, sh4, ctab);
@@ -270,11 +296,38 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     }
                     v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
                 }
-                PackedGroup<T> packed;
                 pack_group<T, LAYOUT>(v, hf, packed);
-                store_packed<T, LAYOUT, sizeof(T) == 2>(dimg, a.dst_h, a.dst_w, r, x0, packed);  // fp16: streaming stores
+            }
+            if (DEFER && rs + G >= r1) {  // the window's last pass: held back
+                packed_on = on;
+                packed_r = r;
+            } else if (on) {
+                store_packed<T, LAYOUT, RMX_DMA_NT>(dimg, a.dst_h, a.dst_w, r, x0, packed);
             }
         }
+
+        // ---- the next window: its loads first, then the held-back stores
+        int nr0 = r0 + wrows, ntile = tile;
+        if (nr0 >= r_end) {
+            nr0 = r_begin;
+            ntile = tile + 1;
+        }
+        const bool more = ntile < ntx;
+        DmaTile ng = g;
+        wave_sync();  // the blend has read the LDS slice for the last time
+        if (more) {
+            if (ntile != tile) ng = tile_geom(ntile);
+            a_v = issue(ng, nr0, min(nr0 + wrows, r_end));
+        }
+        asm volatile("" ::: "memory");  // the held-back stores are issued after those loads, not before
+        if (DEFER && packed_on) store_packed<T, LAYOUT, RMX_DMA_NT>(dimg, a.dst_h, a.dst_w, packed_r, x0, packed);
+        asm volatile("" ::: "memory");
+        if (!more) break;
+        held = true;
+        if (ntile != tile) taps(ng);  // while the loads are in flight
+        g = ng;
+        tile = ntile;
+        r0 = nr0;
     }
 }
 

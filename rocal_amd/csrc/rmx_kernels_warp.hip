@@ -15,6 +15,10 @@
 
 #include <type_traits>
 
+#ifndef RMX_WARP_NT
+#define RMX_WARP_NT false
+#endif
+
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_warp[];
@@ -257,7 +261,7 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
             if (packed_ok && cnt == PX) {
                 PackedGroup<T> packed;
                 pack_group_dir<T, LAYOUT, false>(v, packed);
-                store_packed<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
+                store_packed<T, LAYOUT, RMX_WARP_NT>(dimg, a.dst_h, a.dst_w, y, x0, packed);
             } else {
                 store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, v, false);
             }
