@@ -362,7 +362,7 @@ def measured_traffic(cfg, kernel):
     return rec["fetch_bytes"] + rec["write_bytes"]
 
 
-def run_config(cfg, ctx, steps, warmup, with_cpu, rotating_only=False):
+def run_config(cfg, ctx, steps, warmup, with_cpu, rotating_only=False, ramp_ms=RAMP_MS):
     import torch
     op, src, dst, n, cpu_fn, update_fn = build_case(cfg, ctx)
     srcs = src if isinstance(src, tuple) else (src,)
@@ -371,7 +371,7 @@ def run_config(cfg, ctx, steps, warmup, with_cpu, rotating_only=False):
     copies = max(2, -(-ROTATE_BYTES // max(algo, 1)))
     pairs = [(srcs, dst)] + [(tuple(t.clone() for t in srcs), torch.empty_like(dst)) for _ in range(copies - 1)]
     launchers = [_launcher(op, sp, d) for sp, d in pairs]
-    ramp_launches, ramp_ms = clock_ramp(launchers)
+    ramp_launches, ramp_ms = clock_ramp(launchers, ramp_ms) if ramp_ms > 0 else (0, 0.0)
     ms_kernel, ms_step = time_loop(launchers, steps, warmup)          # rotating: the reported figure
     ms_warm = ms_kernel
     if not rotating_only:
@@ -420,6 +420,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--rotating-only", action="store_true", help="only the ramp and the rotating timed loop: every launch of the process is of the "
                     "reported kind, so a rocprofv3 kernel summary of this command averages the same thing")
+    ap.add_argument("--ramp-ms", type=float, default=RAMP_MS, help="length of the untimed clock ramp (0 for counter runs, which only count)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build measures ONE GPU (the path shards trivially by sample; no multi-GPU figure is produced). "
@@ -430,7 +431,7 @@ def main():
     from rocal_amd import ops
     ctx = ops.Context(0)
     ceiling = copy_ceiling(ctx)
-    res = run_config(args.config, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only)
+    res = run_config(args.config, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only, args.ramp_ms)
     res["metric"] = "images/s + HBM GB/s (% peak), RandomResizedCrop+CMN 224^2 fp16, batch 256" if args.config == 1 else "images/s"
     res["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
     res["roofline"]["frac_of_copy_ceiling"] = round(res["roofline"]["achieved"] / ceiling, 4)
@@ -438,7 +439,7 @@ def main():
         allres = {args.config: res}
         for cfg in sorted(WORKLOADS):
             if cfg != args.config:
-                allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only)
+                allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only, args.ramp_ms)
                 allres[cfg]["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
                 print("config %d: %s" % (cfg, json.dumps(allres[cfg])), file=sys.stderr)
         os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
