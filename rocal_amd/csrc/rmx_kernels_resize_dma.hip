@@ -6,20 +6,23 @@
 // (rmx_kernels_resize_fast.hip), but the source window travels from global memory straight into LDS
 // (global_load_lds_dwordx4: 16 bytes per lane, no vector register, no unpacking, no LDS store instruction):
 //   1. LDS holds the raw packed-RGB rows. A row is a sequence of 16-byte pieces: piece 0 is a margin for the left
-//      edge replica, pieces 1.. are the row's bytes from the dword that holds the window's first pixel. (row, piece)
-//      pairs form one flat index space dealt to the 64 lanes; every load instruction fills 1 KB of LDS. The compiler
-//      does not order LDS reads behind such loads, so arrival is awaited with an explicit s_waitcnt vmcnt(0) between
-//      two wavefront fences; the x taps are computed while the loads are in flight;
+//      edge replica, pieces 1.. are the row's bytes from the dword that holds the window's first pixel. One load
+//      instruction per source row and 64 pieces; the row's address and LDS slot are scalar arithmetic. The compiler
+//      does not order LDS reads behind such loads, so arrival is awaited with an explicit s_waitcnt between two
+//      wavefront fences; the x taps of a tile are computed while its first window's loads are in flight;
 //   2. the blend reads a tap pair (two packed pixels, 6 bytes at any byte phase) as three aligned dwords and
 //      realigns them with two v_alignbyte; every value and every operation after that is the general kernel's,
-//      operation for operation (bit-identical results).
+//      operation for operation (bit-identical results);
+//   3. the stores of a window's last pass wait in registers until the next window's loads have been started, so that
+//      the wait for those loads (operations of a wavefront complete in issue order) never waits for a store.
 // Against the staged kernel this trades about 25 staging instructions per 4 source pixels for 4 realignments per
-// destination pixel (the vector-instruction count stays within 3 %), frees the registers the staged loads occupy and
-// needs a quarter less LDS (3 bytes per pixel instead of 4). Measured on the RandomResizedCrop batch with every launch
-// reading and writing buffers that were not touched for a gigabyte: 33.9 us against 36.4 us; replayed on one
-// cache-resident pair both take 29.5 us. Tried and measured slower: two windows per wavefront with the next strip's loads
-// in flight during the blend (38-41 us: 12 KB of LDS per wavefront leaves 13 wavefronts per CU), all LDS reads of a pass
-// issued before its arithmetic (129 registers, 3 wavefronts per SIMD), register budgets of 96 and 80 (spills).
+// destination pixel, frees the registers the staged loads occupy and needs a quarter less LDS (3 bytes per pixel
+// instead of 4). Measured on the RandomResizedCrop batch (256 images to 224 x 224 fp16) with every launch reading and
+// writing buffers that were not touched for a gigabyte: 32.1 us against 36.4 us; replayed on one cache-resident pair
+// 26.3 against 29.4 us. Tried and measured slower: two LDS windows per wavefront with the next window's loads in flight
+// during the blend (38-41 us: 12 KB of LDS per wavefront leaves 13 wavefronts per CU), all LDS reads of a pass issued
+// before its arithmetic (129 registers, 3 wavefronts per SIMD), register budgets of 96 and 80 (spills), several windows
+// below each other per wavefront (fewer instructions, but too few wavefronts to fill the chip evenly).
 #include "rmx_device.h"
 #include "rmx_color_math.h"
 #include "rmx_launch.h"
