@@ -81,7 +81,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 8, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -1362,7 +1362,9 @@ static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, con
         if (std::isfinite(bw) && std::isfinite(bh)) {
             bw = std::min(bw, (double)s.src_w + 1);
             bh = std::min(bh, (double)s.src_h + 1);
-            worst_box = std::max(worst_box, (std::ceil(bw / 4) * 4 + 4) * bh);
+            // (boxes of up to 60 dwords per row are staged at a pitch of 60, see the kernel)
+            const double pitch = std::ceil(bw / 4) * 4 + 4;
+            worst_box = std::max(worst_box, (pitch <= 60.0 ? 60.0 : pitch) * bh);
         }
     }
     op->algo_bytes = bytes;

@@ -22,8 +22,10 @@
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_warp[];
+typedef __attribute__((address_space(3))) uint32_t lds_u32;  // explicit LDS pointers: 32-bit address arithmetic
 
 constexpr int WTW = 32, WTH = 16;  // destination tile: 4 lanes x 8 px wide, 16 rows per pass
+constexpr int WFP = 60;            // fixed LDS pitch (dwords) of boxes that fit it
 
 RMX_DEV uint32_t load_px_global(const uint8_t *p) {
     return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
@@ -99,7 +101,11 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const bool empty = bw <= 0 || bh <= 0;
     // staged box: bw columns + the repeated last one, bh rows + the repeated last one
     const int items = (max(bw, 0) + 1 + 3) >> 2;
-    const int pitch = items * 4;
+    // Boxes of at most WFP - 1 columns (every tile of a map that does not minify) are staged at ONE pitch, known to the
+    // compiler: the address of a tap is two instructions (a 24-bit multiply-add and a shift-add) and the row below is an
+    // offset inside the read instruction. 15 items: an odd number of 16-byte items spreads the rows over the LDS banks.
+    const bool fixed = items * 4 <= WFP;
+    const int pitch = fixed ? WFP : items * 4;
     const int total = (bh + 1) * items;
     const bool use_lds = !empty && total <= 16 * RMX_WAVE && (size_t)(bh + 1) * pitch * 4 <= (size_t)a.lds_bytes;
 
@@ -108,8 +114,21 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const int cnt = min(PX, dw - x0);
     const float xr0 = (float)x0 - dcx;
 
+    if (empty) {
+        // every pixel of the tile maps outside the ROI: the fill value
+        float z[3][PX];
+#pragma unroll
+        for (int c = 0; c < 3; c++)
+#pragma unroll
+            for (int k = 0; k < PX; k++) z[c][k] = 0.0f;
+        for (int pass = 0; pass < passes; pass++) {
+            const int y = Y0 + pass * WTH + lr;
+            if (y < dh && cnt > 0) store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, y, x0, cnt, z, false);
+        }
+        return;
+    }
     if (!use_lds) {
-        // empty box (every pixel is outside the ROI) or a box too large for the slice: per-pixel gathers from global memory
+        // a box too large for the slice: per-pixel gathers from global memory
         for (int pass = 0; pass < passes; pass++) {
             const int y = Y0 + pass * WTH + lr;
             if (y >= dh || cnt <= 0) continue;
@@ -213,10 +232,17 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     }
 
     // ---- gather and blend, branch-free
-    const int boff = by0 * pitch + bx0;  // dword offset of source pixel (0, 0) relative to the slice (may be "negative")
-    const uint32_t xspan = (uint32_t)(xhi - xlo), yspan = (uint32_t)(yhi - ylo);
-    auto gather = [&](auto chk) {
+    // LDS byte address of source pixel (0, 0): the slice's base minus the box origin (may lie below the slice)
+    const int lbase0 = (int)(uint32_t)(uintptr_t)(lds_u32 *)lds - 4 * (by0 * pitch + bx0);
+    // pixels whose floor lies inside the ROI: xlo <= s < xhi + 1 (and not NaN), tested on the clamped coordinate
+    // (upper bounds: the float just below xhi + 1, a positive number, so one step down in its bit pattern)
+    const float cx_lo = (float)xlo, cx_hi = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, (float)(xhi + 1)) - 1u);
+    const float cy_lo = (float)ylo, cy_hi = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, (float)(yhi + 1)) - 1u);
+    int lbase_v = lbase0;  // the same in a vector register: the multiply-add takes only one scalar operand
+    asm volatile("" : "+v"(lbase_v));
+    auto gather = [&](auto chk, auto fix) {
         constexpr bool CHECK = decltype(chk)::value;
+        constexpr bool FIXED = decltype(fix)::value;
         for (int pass = 0; pass < passes; pass++) {
             const int y = Y0 + pass * WTH + lr;
             if (y >= dh || cnt <= 0) continue;
@@ -232,19 +258,39 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
                     sx += 0.5f;
                     sy += 0.5f;
                 }
+                bool inb = true;
+                if constexpr (CHECK) {
+                    // Clamped into the ROI (a NaN becomes the lower bound): equal to the coordinate exactly when the pixel is
+                    // inside, and an address inside the staged box also when it is not (the box holds the ROI's border
+                    // wherever the tile reaches beyond it).
+                    const float qx = __builtin_fminf(__builtin_fmaxf(sx, cx_lo), cx_hi);
+                    const float qy = __builtin_fminf(__builtin_fmaxf(sy, cy_lo), cy_hi);
+                    inb = qx == sx && qy == sy;
+                    sx = qx;
+                    sy = qy;
+                }
                 const int ix0 = floor_i32(sx), iy0 = floor_i32(sy);
-                const bool inb = !CHECK || ((uint32_t)(ix0 - xlo) <= xspan && (uint32_t)(iy0 - ylo) <= yspan && sx == sx && sy == sy);
-                // (an address inside the slice also for pixels outside the ROI, whose coordinates can be anything)
-                const uint32_t *t0p = lds + (inb ? (__mul24(iy0, pitch) + ix0 - boff) : 0);
+                const lds_u32 *t0p, *t1p;
+                if constexpr (FIXED) {
+                    // byte address: a 24-bit multiply-add of the row onto the (scalar) slice base, a shift-add of the column
+                    // (spelled out: left to itself the compiler makes a shift, a multiply and a three-way add of it)
+                    uint32_t rowb, adr;
+                    asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(rowb) : "v"(iy0), "s"(WFP * 4), "v"(lbase_v));
+                    asm("v_lshl_add_u32 %0, %1, 2, %2" : "=v"(adr) : "v"(ix0), "v"(rowb));
+                    t0p = (const lds_u32 *)adr;
+                    t1p = t0p + WFP;
+                } else {
+                    t0p = (const lds_u32 *)(uint32_t)(((uint32_t)(__mul24(iy0, pitch) + ix0) << 2) + (uint32_t)lbase0);
+                    t1p = t0p + pitch;
+                }
                 float o0, o1, o2;
                 if constexpr (NEAREST) {
                     const uint32_t tl = t0p[0];
                     o0 = ubyte0(tl); o1 = ubyte1(tl); o2 = ubyte2(tl);
                 } else {
                     const uint32_t tl = t0p[0], tr = t0p[1];
-                    const uint32_t *t1p = t0p + pitch;
                     const uint32_t bl = t1p[0], br = t1p[1];
-                    // sx - floor(sx): exact for the non-negative coordinates of pixels inside the ROI
+                    // s - floor(s): exact for the non-negative coordinates of pixels inside the ROI
                     const float wx = __builtin_amdgcn_fractf(sx), wy = __builtin_amdgcn_fractf(sy);
                     const float omx = 1.0f - wx, omy = 1.0f - wy;
                     const float w00 = omy * omx, w01 = omy * wx, w10 = wy * omx;
@@ -267,8 +313,13 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
             }
         }
     };
-    if (all_in) gather(std::false_type{});
-    else gather(std::true_type{});
+    if (fixed) {
+        if (all_in) gather(std::false_type{}, std::true_type{});
+        else gather(std::true_type{}, std::true_type{});
+    } else {
+        if (all_in) gather(std::false_type{}, std::false_type{});
+        else gather(std::true_type{}, std::false_type{});
+    }
 }
 
 template <bool NEAREST>
