@@ -74,66 +74,90 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
         // source column of group pixel 0 (mirror reads the mirrored run and reverses it)
         const int sx0 = x1 + (hf ? (cw - gx - cnt) : gx);
         if constexpr (FAST) {
-            constexpr int NI = 4;  // row steps in flight
-            for (int rb = r0 + lr; rb < r1 && active; rb += NI * G) {
-                const uint32_t *q[NI];
-                uint32_t ph[NI];
-                bool safe = true;
+            // One row step of a lane: 8 pixels = 24 source bytes, fetched as a 16- and a 12-byte load from the dword below them.
+            auto row_ptr = [&](int r, uint32_t &ph) {
+                const int sy = y1 + (vf ? (ch - 1 - r) : r);
+                const uint8_t *p = simg + (size_t)sy * row_stride + (size_t)sx0 * 3;
+                ph = (uint32_t)((uintptr_t)p & 3u);
+                return reinterpret_cast<const uint32_t *>(p - ph);
+            };
+            auto finish = [&](int r, const uint32_t (&w)[6]) {
+                float v[3][PX];
+                unpack8(w, v);
+                if (chrev) {
 #pragma unroll
-                for (int i = 0; i < NI; i++) {
-                    const int r = min(rb + i * G, r1 - 1);  // steps beyond the strip repeat its last row (never stored)
-                    const int sy = y1 + (vf ? (ch - 1 - r) : r);
-                    const uint8_t *p = simg + (size_t)sy * row_stride + (size_t)sx0 * 3;
-                    ph[i] = (uint32_t)((uintptr_t)p & 3u);
-                    q[i] = reinterpret_cast<const uint32_t *>(p - ph[i]);
-                    safe = safe && ((const uint8_t *)(q[i] + 7) <= buf_end);
+                    for (int k = 0; k < PX; k++) {
+                        const float t = v[0][k];
+                        v[0][k] = v[2][k];
+                        v[2][k] = t;
+                    }
                 }
-                uint32_t w[NI][6];
-                if (safe) {
-                    u32x4_a4 t[NI];
-                    u32x3_a4 u[NI];
+                if constexpr (NORM) {
+#pragma unroll
+                    for (int c = 0; c < 3; c++)
+#pragma unroll
+                        for (int k = 0; k < PX; k++) v[c][k] = __builtin_fmaf(v[c][k], sc[c], bi[c]);
+                }
+                PackedGroup<T> packed;
+                pack_group<T, LAYOUT>(v, hf, packed);
+                if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT, RMX_K1_NT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
+                else store_packed<T, LAYOUT, RMX_K1_NT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+            };
+            // every wide load of this wavefront's strip stays inside the batch buffer (the first and the last row bound the rest)
+            bool lane_safe = true;
+            if (active) {
+                uint32_t ph;
+                lane_safe = (const uint8_t *)(row_ptr(r0, ph) + 7) <= buf_end && (const uint8_t *)(row_ptr(r1 - 1, ph) + 7) <= buf_end;
+            }
+            if (__builtin_amdgcn_ballot_w64(!lane_safe) == 0) {
+                // Software pipeline over batches of NI row steps: the loads of the next batch are issued BEFORE the stores of the
+                // current one. Memory operations of a wavefront complete in issue order, so the wait for a batch's loads then
+                // leaves the stores of the batch before (and the loads of the batch after) outstanding: a wavefront has reads
+                // and writes in flight at the same time, instead of all wavefronts of a launch reading first and writing after.
+                constexpr int NI = 2;
+                u32x4_a4 ta[NI], tb[NI];
+                u32x3_a4 ua[NI], ub[NI];
+                uint32_t pa[NI], pb[NI];
+                auto issue = [&](int base, u32x4_a4 (&t)[NI], u32x3_a4 (&u)[NI], uint32_t (&ph)[NI]) {
+                    if (active) {
+#pragma unroll
+                        for (int i = 0; i < NI; i++) {
+                            const uint32_t *q = row_ptr(min(base + lr + i * G, r1 - 1), ph[i]);  // steps beyond the strip repeat its last row (never stored)
+                            t[i] = *reinterpret_cast<const u32x4_a4 *>(q);
+                            u[i] = *reinterpret_cast<const u32x3_a4 *>(q + 4);
+                        }
+                    }
+                };
+                auto consume = [&](int base, const u32x4_a4 (&t)[NI], const u32x3_a4 (&u)[NI], const uint32_t (&ph)[NI]) {
 #pragma unroll
                     for (int i = 0; i < NI; i++) {
-                        t[i] = *reinterpret_cast<const u32x4_a4 *>(q[i]);
-                        u[i] = *reinterpret_cast<const u32x3_a4 *>(q[i] + 4);
+                        const int r = base + lr + i * G;
+                        if (active && r < r1) {
+                            const uint32_t d[7] = {t[i].x, t[i].y, t[i].z, t[i].w, u[i].x, u[i].y, u[i].z};
+                            uint32_t w[6];
+#pragma unroll
+                            for (int j = 0; j < 6; j++) w[j] = __builtin_amdgcn_alignbyte(d[j + 1], d[j], ph[i]);
+                            finish(r, w);
+                        }
                     }
-#pragma unroll
-                    for (int i = 0; i < NI; i++) {
-                        const uint32_t d[7] = {t[i].x, t[i].y, t[i].z, t[i].w, u[i].x, u[i].y, u[i].z};
-#pragma unroll
-                        for (int j = 0; j < 6; j++) w[i][j] = __builtin_amdgcn_alignbyte(d[j + 1], d[j], ph[i]);
+                };
+                const int step = NI * G;
+                issue(r0, ta, ua, pa);
+                for (int base = r0; base < r1; base += 2 * step) {
+                    if (base + step < r1) issue(base + step, tb, ub, pb);
+                    consume(base, ta, ua, pa);
+                    if (base + step < r1) {
+                        if (base + 2 * step < r1) issue(base + 2 * step, ta, ua, pa);
+                        consume(base + step, tb, ub, pb);
                     }
-                } else {
-                    // last bytes of the batch buffer: the bounds-checked loader
-#pragma unroll
-                    for (int i = 0; i < NI; i++)
-                        load_realigned<7>(reinterpret_cast<const uint8_t *>(q[i]) + ph[i], buf_end, w[i]);
                 }
-#pragma unroll
-                for (int i = 0; i < NI; i++) {
-                    const int r = rb + i * G;
-                    if (r < r1) {
-                        float v[3][PX];
-                        unpack8(w[i], v);
-                        if (chrev) {
-#pragma unroll
-                            for (int k = 0; k < PX; k++) {
-                                const float t = v[0][k];
-                                v[0][k] = v[2][k];
-                                v[2][k] = t;
-                            }
-                        }
-                        if constexpr (NORM) {
-#pragma unroll
-                            for (int c = 0; c < 3; c++)
-#pragma unroll
-                                for (int k = 0; k < PX; k++) v[c][k] = __builtin_fmaf(v[c][k], sc[c], bi[c]);
-                        }
-                        PackedGroup<T> packed;
-                        pack_group<T, LAYOUT>(v, hf, packed);
-                        if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT, RMX_K1_NT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
-                        else store_packed<T, LAYOUT, RMX_K1_NT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
-                    }
+            } else {
+                // last bytes of the batch buffer: the bounds-checked loader, row by row
+                for (int r = r0 + lr; r < r1 && active; r += G) {
+                    uint32_t ph, w[6];
+                    const uint32_t *q = row_ptr(r, ph);
+                    load_realigned<7>(reinterpret_cast<const uint8_t *>(q) + ph, buf_end, w);
+                    finish(r, w);
                 }
             }
         } else {
