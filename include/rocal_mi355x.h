@@ -94,6 +94,11 @@ RMX_API int rmx_op_destroy(rmx_op *op);
  * (rocAL/source/loaders/image/image_read_and_decode.cpp:165-390, circular_buffer.cpp:88-133): a C1 batch is
  * 315 MB padded for about 80 MB of pixels. */
 RMX_API int rmx_op_set_ragged_source(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights, uint64_t buffer_bytes);
+/* The same with a row stride per image (bytes, >= width*3; NULL: width*3). A loader that starts every image at a multiple of 4
+ * bytes and pads its rows to a multiple of 4 bytes gives the bilinear resize its streaming kernel (source rows straight into
+ * LDS), which needs every row of the batch to start at the same byte phase; the padding is at most 3 bytes per row. */
+RMX_API int rmx_op_set_ragged_source_strided(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights,
+                                             const uint32_t *row_strides, uint64_t buffer_bytes);
 /* Algorithmic bytes of the last update: sum of source-window bytes + destination bytes. */
 RMX_API uint64_t rmx_op_algorithmic_bytes(const rmx_op *op);
 /* Launch plan of the last update as text (waves, strips, LDS per wave ...), for logs and benchmarks. */

@@ -38,6 +38,7 @@ _SIGS = {
     "rmx_op_kernel_name": [_vp],
     "rmx_op_plan": [_vp],
     "rmx_op_set_ragged_source": [_vp, _vp, _vp, _vp, C.c_uint64],
+    "rmx_op_set_ragged_source_strided": [_vp, _vp, _vp, _vp, _vp, C.c_uint64],
     "rmx_create_crop_mirror_normalize": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],
     "rmx_update_crop_mirror_normalize": [_vp, _vp, _vp, _vp, _vp],
     "rmx_create_crop": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.POINTER(_vp)],

@@ -458,6 +458,11 @@ int rmx_op_launch2(rmx_op *op, const void *src1, const void *src2, void *dst) {
 /* ------------------------------------------------------------------ ragged sources */
 
 int rmx_op_set_ragged_source(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights, uint64_t buffer_bytes) {
+    return rmx_op_set_ragged_source_strided(op, offsets, widths, heights, nullptr, buffer_bytes);
+}
+
+int rmx_op_set_ragged_source_strided(rmx_op *op, const uint64_t *offsets, const uint32_t *widths, const uint32_t *heights, const uint32_t *row_strides,
+                                     uint64_t buffer_bytes) {
     if (!op) return fail(RMX_ERR_INVALID, "op is NULL");
     if (op->kind == OP_BLEND) return fail(RMX_ERR_UNSUPPORTED, "a Blend node reads two padded tensors of one shape; ragged sources are not supported");
     if (!offsets && !widths && !heights) {  // back to one padded tensor
@@ -470,12 +475,15 @@ int rmx_op_set_ragged_source(rmx_op *op, const uint64_t *offsets, const uint32_t
     for (int i = 0; i < op->n; i++) {
         if (widths[i] == 0 || heights[i] == 0 || widths[i] > op->src.w || heights[i] > op->src.h)
             return fail(RMX_ERR_INVALID, "sample %d: image of %u x %u is empty or exceeds the %u x %u of the source descriptor", i, widths[i], heights[i], op->src.w, op->src.h);
-        const uint64_t bytes = (uint64_t)widths[i] * heights[i] * 3;
+        const uint32_t stride = row_strides ? row_strides[i] : widths[i] * 3u;
+        if (stride < widths[i] * 3u) return fail(RMX_ERR_INVALID, "sample %d: row stride %u is shorter than a row of %u pixels", i, stride, widths[i]);
+        // (the last row need not be padded)
+        const uint64_t bytes = (uint64_t)stride * (heights[i] - 1) + (uint64_t)widths[i] * 3;
         if (offsets[i] > buffer_bytes || bytes > buffer_bytes - offsets[i])
             return fail(RMX_ERR_INVALID, "sample %d: %llu bytes at offset %llu do not fit the buffer of %llu bytes", i, (unsigned long long)bytes, (unsigned long long)offsets[i],
                         (unsigned long long)buffer_bytes);
         l[i].offset = offsets[i];
-        l[i].row_stride = widths[i] * 3u;
+        l[i].row_stride = stride;
         l[i].rows = heights[i];
     }
     op->layout.swap(l);

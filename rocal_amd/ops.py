@@ -155,8 +155,9 @@ class Op:
         shape = (d.n, d.c, d.h, d.w) if d.layout == NCHW else (d.n, d.h, d.w, d.c)
         return t.full(shape, fill, dtype=torch_dtype(d.dtype), device="cuda:%d" % self.ctx.device)
 
-    def set_ragged_source(self, offsets, widths, heights, buffer_bytes):
-        """The batch's images lie tightly packed at byte `offsets` of one buffer (None, None, None: padded tensor again)."""
+    def set_ragged_source(self, offsets, widths, heights, buffer_bytes, row_strides=None):
+        """The batch's images lie packed at byte `offsets` of one buffer, rows `row_strides` bytes apart (default: width*3, no
+        padding at all); offsets None: padded tensor again."""
         if offsets is None:
             check(_lib.lib().rmx_op_set_ragged_source(self._h, None, None, None, 0))
             self._ragged_bytes = None
@@ -165,8 +166,13 @@ class Op:
         o = np.ascontiguousarray(offsets, np.uint64)
         w = np.ascontiguousarray(widths, np.uint32)
         h = np.ascontiguousarray(heights, np.uint32)
-        check(_lib.lib().rmx_op_set_ragged_source(self._h, o.ctypes.data_as(C.c_void_p), w.ctypes.data_as(C.c_void_p), h.ctypes.data_as(C.c_void_p),
-                                                  int(buffer_bytes)))
+        if row_strides is None:
+            check(_lib.lib().rmx_op_set_ragged_source(self._h, o.ctypes.data_as(C.c_void_p), w.ctypes.data_as(C.c_void_p), h.ctypes.data_as(C.c_void_p),
+                                                      int(buffer_bytes)))
+        else:
+            st = np.ascontiguousarray(row_strides, np.uint32)
+            check(_lib.lib().rmx_op_set_ragged_source_strided(self._h, o.ctypes.data_as(C.c_void_p), w.ctypes.data_as(C.c_void_p),
+                                                              h.ctypes.data_as(C.c_void_p), st.ctypes.data_as(C.c_void_p), int(buffer_bytes)))
 
     @property
     def algorithmic_bytes(self):

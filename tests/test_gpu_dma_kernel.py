@@ -138,3 +138,45 @@ def test_ragged_source_with_dword_row_strides(ctx):
         got = out.cpu().numpy()
         for i in range(n):
             assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp[i, :, :dh[i], :dw[i]].view(np.uint16)), "sample %d, odd=%s" % (i, odd)
+
+
+def test_ragged_source_with_padded_rows(ctx):
+    """Packed images of any width whose rows the loader pads to a multiple of 4 bytes (a row stride per image): the streaming
+    kernel, bit-identical to the oracle on the padded tensor; a stride shorter than a row is refused."""
+    rng = np.random.default_rng(6)
+    n = 6
+    widths = np.array([61, 100, 37, 127, 85, 11], np.uint32)
+    heights = np.array([50, 33, 80, 64, 21, 9], np.uint32)
+    strides = (3 * widths + 3) // 4 * 4
+    offsets, parts, pos = [], [], 0
+    padded = np.zeros((n, 80, 128, 3), np.uint8)
+    for i in range(n):
+        h, w, st = int(heights[i]), int(widths[i]), int(strides[i])
+        im = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+        padded[i, :h, :w] = im
+        rows = rng.integers(0, 256, (h, st), dtype=np.uint8)  # the padding bytes hold anything
+        rows[:, :3 * w] = im.reshape(h, 3 * w)
+        offsets.append(pos)
+        parts.append(rows.reshape(-1))
+        pos += h * st
+    packed = np.concatenate(parts)
+    roi = np.array([[0, 0, widths[i], heights[i]] for i in range(n)], np.uint32)
+    roi[1] = (10, 5, 80, 20)
+    dw = np.array([48, 64, 40, 128, 8, 24], np.uint32)
+    dh = np.array([40, 30, 90, 50, 30, 18], np.uint32)
+    mirror = np.array([1, 0, 0, 1, 1, 0], np.uint32)
+    scale, bias = _scale_bias(n)
+    exp = orc.resize(padded, roi, dw, dh, 90, 128, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                     flags=orc.F_QUANTIZE_U8)
+    op = ops.Resize(ctx, ops.desc(n, 80, 128, ops.NHWC, ops.UINT8), ops.desc(n, 90, 128, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+    op.set_ragged_source(np.array(offsets, np.uint64), widths, heights, packed.size, row_strides=strides)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert op.kernel_name == "rmx_resize_dma_kernel"
+    out = op.alloc_output()
+    op.launch(_gpu(packed), out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    for i in range(n):
+        assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp[i, :, :dh[i], :dw[i]].view(np.uint16)), "sample %d" % i
+    with pytest.raises(Exception, match="row stride"):
+        op.set_ragged_source(np.array(offsets, np.uint64), widths, heights, packed.size, row_strides=3 * widths - 1)
