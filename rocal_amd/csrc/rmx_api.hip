@@ -105,6 +105,7 @@ struct rmx_op {
     std::vector<float> lut_gamma;         // Gamma: the exponent each cached table was built for (NaN = none yet)
     std::vector<uint8_t> lut_cache;       // Gamma: last table of every sample (256 powf per table are worth keeping)
     std::vector<RmxSrcLayout> layout;     // ragged source (empty: one padded tensor); copied behind the rows on every update
+    std::vector<uint32_t> layout_w;       // image widths of the ragged source (a row stride may include padding)
     uint64_t ragged_bytes = 0;            // extent of the ragged source buffer
     bool slot_ragged[TABLE_RING] = {};    // what the table slot was committed with
     uint64_t slot_src_bytes[TABLE_RING] = {};
@@ -209,7 +210,7 @@ int commit_slot(rmx_op *op, int slot) {
 }
 
 // image size of sample i: its own when the source is ragged, the padded tensor's otherwise
-inline uint32_t sample_w(const rmx_op *op, int i) { return op->layout.empty() ? op->src.w : op->layout[i].row_stride / 3u; }
+inline uint32_t sample_w(const rmx_op *op, int i) { return op->layout.empty() ? op->src.w : op->layout_w[i]; }
 inline uint32_t sample_h(const rmx_op *op, int i) { return op->layout.empty() ? op->src.h : op->layout[i].rows; }
 
 // ROI in the caller's convention -> x,y,w,h clipped to the padded source tensor.
@@ -467,6 +468,7 @@ int rmx_op_set_ragged_source_strided(rmx_op *op, const uint64_t *offsets, const 
     if (op->kind == OP_BLEND) return fail(RMX_ERR_UNSUPPORTED, "a Blend node reads two padded tensors of one shape; ragged sources are not supported");
     if (!offsets && !widths && !heights) {  // back to one padded tensor
         op->layout.clear();
+        op->layout_w.clear();
         op->ragged_bytes = 0;
         return RMX_OK;
     }
@@ -487,6 +489,7 @@ int rmx_op_set_ragged_source_strided(rmx_op *op, const uint64_t *offsets, const 
         l[i].rows = heights[i];
     }
     op->layout.swap(l);
+    op->layout_w.assign(widths, widths + op->n);
     op->ragged_bytes = buffer_bytes;
     return RMX_OK;
 }

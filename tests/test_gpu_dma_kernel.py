@@ -180,3 +180,17 @@ def test_ragged_source_with_padded_rows(ctx):
         assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp[i, :, :dh[i], :dw[i]].view(np.uint16)), "sample %d" % i
     with pytest.raises(Exception, match="row stride"):
         op.set_ragged_source(np.array(offsets, np.uint64), widths, heights, packed.size, row_strides=3 * widths - 1)
+    # windows are clipped to the image, not to the padded row: image 2 is 37 pixels wide in rows of 112 bytes (37.3 pixels)
+    op.set_ragged_source(np.array(offsets, np.uint64), widths, heights, packed.size, row_strides=strides)
+    wide = roi.copy()
+    wide[:, 2] = 1000
+    op.update_cmn(wide, dw, dh, scale, bias, mirror)
+    op.launch(_gpu(packed), out)
+    ctx.sync()
+    full = np.array([[0, 0, widths[i], heights[i]] for i in range(n)], np.uint32)
+    full[1] = (10, 5, widths[1] - 10, 20)
+    exp2 = orc.resize(padded, full, dw, dh, 90, 128, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                      flags=orc.F_QUANTIZE_U8)
+    got = out.cpu().numpy()
+    for i in range(n):
+        assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp2[i, :, :dh[i], :dw[i]].view(np.uint16)), "clipped window, sample %d" % i
