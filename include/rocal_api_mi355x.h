@@ -73,6 +73,22 @@ extern "C" long long unsigned ROCAL_API_CALL rocalGetParameterUpdateTime(RocalCo
 extern "C" RocalTensor ROCAL_API_CALL rocalDeviceSource(RocalContext context, unsigned max_width, unsigned max_height, bool is_output);
 extern "C" RocalStatus ROCAL_API_CALL rocalDeviceSourceFeed(RocalContext context, RocalTensor source, const void *device_ptr, const unsigned *roi_width,
                                                             const unsigned *roi_height);
+// A source fed by a loader through a ring of PACKED batches (stands where the loader's CircularBuffer and its padded
+// [N, Hmax, Wmax, 3] staging stand: rocAL/source/loaders/circular_buffer.cpp:88-160, image_read_and_decode.cpp:165-390).
+// The loader places every decoded image of a batch into pinned host memory (rocalPackedSourcePlaceImage returns where the
+// image's first row goes and the row stride to use: width*3 rounded up to a multiple of 4) and pushes the batch, which starts
+// ONE asynchronous copy of the bytes written; rocalRun() consumes the oldest pushed batch of every packed source.
+// queue_depth slots (>= 2) of slot_bytes each (0: every image at max size). Place and push may run on a loader thread while
+// another thread calls rocalRun: place blocks while the ring is full.
+extern "C" RocalTensor ROCAL_API_CALL rocalPackedSource(RocalContext context, unsigned max_width, unsigned max_height, bool is_output,
+                                                        unsigned queue_depth, size_t slot_bytes);
+extern "C" unsigned char *ROCAL_API_CALL rocalPackedSourcePlaceImage(RocalContext context, RocalTensor source, unsigned index, unsigned width,
+                                                                     unsigned height, unsigned *row_stride);
+extern "C" RocalStatus ROCAL_API_CALL rocalPackedSourcePush(RocalContext context, RocalTensor source);
+// Blocks the caller until a pushed batch is waiting (the consumer side of a loader thread); rocalRun() on an empty ring
+// returns an error instead of blocking.
+extern "C" RocalStatus ROCAL_API_CALL rocalPackedSourceWait(RocalContext context, RocalTensor source);
+extern "C" size_t ROCAL_API_CALL rocalPackedSourceLevel(RocalContext context, RocalTensor source);
 extern "C" void *ROCAL_API_CALL rocalTensorBuffer(RocalTensor tensor);
 // Binds an output tensor to device memory the caller owns (at least rocalTensorDataSize bytes, 16-byte aligned), before or
 // after rocalVerify and as often as wanted between runs: the node that produces the tensor writes there directly. Stands where

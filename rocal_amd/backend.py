@@ -20,6 +20,9 @@ _SIGS = {
     "rocalUpdateIntParameter": (_i, [_i, _vp]), "rocalUpdateFloatParameter": (_i, [_f, _vp]),
     "rocalGetIntValue": (_i, [_vp]), "rocalGetFloatValue": (_f, [_vp]),
     "rocalDeviceSource": (_vp, [_vp, _u, _u, _b]), "rocalDeviceSourceFeed": (_i, [_vp, _vp, _vp, _vp, _vp]),
+    "rocalPackedSource": (_vp, [_vp, _u, _u, _b, _u, C.c_size_t]),
+    "rocalPackedSourcePlaceImage": (_vp, [_vp, _vp, _u, _u, _u, C.POINTER(_u)]),
+    "rocalPackedSourcePush": (_i, [_vp, _vp]), "rocalPackedSourceWait": (_i, [_vp, _vp]), "rocalPackedSourceLevel": (C.c_size_t, [_vp, _vp]),
     "rocalTensorBuffer": (_vp, [_vp]), "rocalTensorRoi": (C.POINTER(_u), [_vp]), "rocalTensorDataSize": (C.c_size_t, [_vp]),
     "rocalTensorSetBuffer": (_i, [_vp, _vp, _vp]),
     "rocalToTensor": (_i, [_vp, _vp, _i, _i, _f, _f, _f, _f, _f, _f, _b, _i, _i, _i]),
@@ -156,6 +159,24 @@ class Backend:
         w = (C.c_uint * n)(*[int(x) for x in widths])
         h = (C.c_uint * n)(*[int(x) for x in heights])
         return host().rocalDeviceSourceFeed(handle, source, device_ptr, w, h)
+
+    def packedSource(self, handle, max_width, max_height, is_output, queue_depth, slot_bytes):
+        return host().rocalPackedSource(handle, max_width, max_height, is_output, queue_depth, slot_bytes)
+
+    def packedSourcePlaceImage(self, handle, source, index, width, height):
+        """Returns (address of the image's first row in pinned host memory, row stride in bytes); address 0 on error."""
+        stride = _u(0)
+        p = host().rocalPackedSourcePlaceImage(handle, source, index, width, height, C.byref(stride))
+        return (p or 0), int(stride.value)
+
+    def packedSourcePush(self, handle, source):
+        return host().rocalPackedSourcePush(handle, source)
+
+    def packedSourceWait(self, handle, source):
+        return host().rocalPackedSourceWait(handle, source)
+
+    def packedSourceLevel(self, handle, source):
+        return int(host().rocalPackedSourceLevel(handle, source))
 
     def tensorBuffer(self, t):
         return host().rocalTensorBuffer(t)

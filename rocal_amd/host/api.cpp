@@ -161,6 +161,74 @@ RocalStatus rocalDeviceSourceFeed(RocalContext p_context, RocalTensor p_source, 
     return ROCAL_OK;
 }
 
+/* ------------------------------------------------------------------ packed batches from a loader */
+
+RocalTensor rocalPackedSource(RocalContext p_context, unsigned max_width, unsigned max_height, bool is_output, unsigned queue_depth, size_t slot_bytes) {
+    if (!p_context) return nullptr;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        if (max_width == 0 || max_height == 0) THROW("source needs non-zero maximum dimensions")
+        const size_t n = context->master_graph->batch_size();
+        TensorInfo info({n, max_height, max_width, 3}, RocalTensorlayout::NHWC, RocalTensorDataType::UINT8);
+        // default capacity: every image at its maximum size (what the padded tensor of the reference takes)
+        if (slot_bytes == 0) slot_bytes = n * (size_t)max_height * (((size_t)max_width * 3 + 3) / 4 * 4);
+        return context->master_graph->create_packed_source(info, is_output, slot_bytes, queue_depth < 2 ? 2 : queue_depth);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return nullptr;
+    }
+}
+
+unsigned char *rocalPackedSourcePlaceImage(RocalContext p_context, RocalTensor p_source, unsigned index, unsigned width, unsigned height, unsigned *row_stride) {
+    if (!p_context) return nullptr;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        auto *t = static_cast<Tensor *>(p_source);
+        if (!t) THROW("null source")
+        const auto &shape = t->info().max_shape();
+        if (width > shape[0] || height > shape[1]) THROW("image of " + TOSTR(width) + " x " + TOSTR(height) + " exceeds the source's maximum of " + TOSTR(shape[0]) + " x " + TOSTR(shape[1]))
+        return context->master_graph->packed_buffer(t)->place_image(index, width, height, row_stride);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return nullptr;
+    }
+}
+
+RocalStatus rocalPackedSourcePush(RocalContext p_context, RocalTensor p_source) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->packed_buffer(static_cast<Tensor *>(p_source))->push();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+RocalStatus rocalPackedSourceWait(RocalContext p_context, RocalTensor p_source) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->packed_buffer(static_cast<Tensor *>(p_source))->block_if_empty();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+size_t rocalPackedSourceLevel(RocalContext p_context, RocalTensor p_source) {
+    if (!p_context) return 0;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        return context->master_graph->packed_buffer(static_cast<Tensor *>(p_source))->level();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return 0;
+    }
+}
+
 void rocalSetOutputs(RocalContext p_context, unsigned int num_of_outputs, std::vector<RocalTensor> &output_tensors) {
     if (!p_context) THROW("Invalid rocal context passed to rocalSetOutputs")
     auto *context = static_cast<Context *>(p_context);

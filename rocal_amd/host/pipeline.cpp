@@ -153,7 +153,21 @@ void Node::create(std::shared_ptr<Graph> graph) {
     create_node();  // a node that is fused away still sets up its parameters here, on the user thread
 }
 
-void Node::update_parameters() { update_node(); }
+void Node::update_parameters() {
+    // a packed source batch: its layout goes to the kernels before the node's own update (which clips the windows to each image)
+    if (_node && !_inputs.empty()) {
+        const PackedLayout *l = _inputs[0]->ragged();
+        if (l) {
+            check(rmx_op_set_ragged_source_strided(_node, l->offsets.data(), l->widths.data(), l->heights.data(), l->row_strides.data(), l->bytes),
+                  "rmx_op_set_ragged_source_strided");
+            _ragged_source = true;
+        } else if (_ragged_source) {
+            check(rmx_op_set_ragged_source(_node, nullptr, nullptr, nullptr, 0), "rmx_op_set_ragged_source");
+            _ragged_source = false;
+        }
+    }
+    update_node();
+}
 
 void Node::release() {
     if (_node) {
@@ -185,7 +199,7 @@ std::vector<uint32_t> Node::roi_as_array(const Roi2DCords *roi) const {
 
 /* ---------------------------------------------------------------- MasterGraph */
 
-MasterGraph::MasterGraph(size_t batch_size, int gpu_id, void *stream) : _batch_size(batch_size), _graph(std::make_shared<Graph>(gpu_id, stream)) {}
+MasterGraph::MasterGraph(size_t batch_size, int gpu_id, void *stream) : _batch_size(batch_size), _gpu_id(gpu_id), _graph(std::make_shared<Graph>(gpu_id, stream)) {}
 
 MasterGraph::~MasterGraph() {
     if (_to_tensor_op) rmx_op_destroy(_to_tensor_op);
@@ -255,8 +269,42 @@ void MasterGraph::bind_output(Tensor *t, void *device_ptr) {
     t->swap_handle(device_ptr);
 }
 
+Tensor *MasterGraph::create_packed_source(const TensorInfo &info, bool is_output, size_t slot_bytes, size_t depth) {
+    Tensor *t = create_tensor(info, is_output);
+    std::unique_ptr<PackedCircularBuffer> buf(new PackedCircularBuffer(_gpu_id, rmx_ctx_stream(_graph->get())));
+    buf->init(_batch_size, slot_bytes, depth);
+    _packed_sources.emplace_back(t, std::move(buf));
+    return t;
+}
+
+PackedCircularBuffer *MasterGraph::packed_buffer(Tensor *source) {
+    for (auto &p : _packed_sources)
+        if (p.first == source) return p.second.get();
+    THROW("the tensor is not a packed source")
+}
+
 void MasterGraph::run() {
     if (!_built) THROW("rocalVerify must be called before rocalRun")
+    // the oldest batch of every packed source: its device slot becomes the tensor's buffer (the graph's stream waits for
+    // the slot's copy), its layout and image sizes the tensor's (loader_module->load_next, master_graph.cpp:1134-1147)
+    for (auto &p : _packed_sources) {
+        if (p.second->level() == 0) THROW("rocalRun: a packed source has no batch (push one first)")
+        p.first->swap_handle(p.second->get_read_buffer_dev());
+        const PackedLayout &l = p.second->get_read_layout();
+        p.first->set_ragged(&l);
+        p.first->update_tensor_roi(l.widths, l.heights);
+    }
+    struct PopAtExit {  // the slots are given back when the launches are enqueued, also when a node throws
+        std::vector<std::pair<Tensor *, std::unique_ptr<PackedCircularBuffer>>> &v;
+        ~PopAtExit() {
+            for (auto &p : v) {
+                try {
+                    p.second->pop();
+                } catch (...) {
+                }
+            }
+        }
+    } pop_at_exit{_packed_sources};
     {
         StopWatch w(_time_us[0]);
         ParameterFactory::instance()->renew_parameters();

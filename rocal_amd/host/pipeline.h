@@ -24,6 +24,8 @@ union Roi2DCords {
     struct { unsigned x, y, w, h; } xywh;
 };
 
+#include "packed_buffer.h"
+
 class TensorInfo {
    public:
     TensorInfo() = default;
@@ -75,10 +77,15 @@ class Tensor {
     void update_tensor_roi(const std::vector<uint32_t> &width, const std::vector<uint32_t> &height);
     bool is_output = false;
     bool elided = false;  // virtual tensor inside a fused chain: never materialised
+    // A source whose batch lies packed in its buffer (PackedCircularBuffer): the layout of the current batch, or null for
+    // the dense [N, Hmax, Wmax, C] tensor. Nodes that read such a tensor hand the layout to their kernels before every update.
+    const PackedLayout *ragged() const { return _ragged; }
+    void set_ragged(const PackedLayout *l) { _ragged = l; }
 
    private:
     TensorInfo _info;
     void *_buffer = nullptr;
+    const PackedLayout *_ragged = nullptr;
 };
 
 class Node;
@@ -131,6 +138,7 @@ class Node {
     std::shared_ptr<Graph> _graph = nullptr;
     rmx_op *_node = nullptr;
     size_t _batch_size;
+    bool _ragged_source = false;  // the op currently reads a packed source
     void check(int status, const char *what);
     std::vector<uint32_t> roi_as_array(const Roi2DCords *roi) const;
 };
@@ -155,6 +163,10 @@ class MasterGraph {
     void build();
     void run();
     void set_output(Tensor *t);  // master_graph.cpp:337-349
+    // A source tensor fed through a ring of packed batches (stands where the loader module and its CircularBuffer stand,
+    // master_graph.cpp:1116-1160 / image_loader.cpp:115-170): run() takes the oldest batch of every such source.
+    Tensor *create_packed_source(const TensorInfo &info, bool is_output, size_t slot_bytes, size_t depth);
+    PackedCircularBuffer *packed_buffer(Tensor *source);
     // master_graph.cpp:514-856: converts the single u8 output tensor into a float tensor in caller memory
     void to_tensor(void *out_ptr, RocalTensorlayout format, float multiplier0, float multiplier1, float multiplier2, float offset0, float offset1,
                    float offset2, bool reverse_channels, RocalTensorDataType output_data_type, unsigned max_roi_height, unsigned max_roi_width);
@@ -180,6 +192,7 @@ class MasterGraph {
 
    private:
     size_t _batch_size;
+    int _gpu_id;
     std::shared_ptr<Graph> _graph;
     std::list<std::shared_ptr<Node>> _nodes;
     std::list<std::unique_ptr<Tensor>> _tensors;
@@ -188,6 +201,7 @@ class MasterGraph {
     std::shared_ptr<BoundingBoxGraph> _meta_graph;
     std::shared_ptr<MetaDataBatch> _input_meta, _output_meta;
     bool _built = false;
+    std::vector<std::pair<Tensor *, std::unique_ptr<PackedCircularBuffer>>> _packed_sources;
     double _time_us[3] = {0.0, 0.0, 0.0};
     // the conversion op of to_tensor(), rebuilt when the requested format changes
     rmx_op *_to_tensor_op = nullptr;

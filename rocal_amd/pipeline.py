@@ -97,6 +97,40 @@ class Pipeline:
         if status != types.OK:
             raise RuntimeError("feed failed: " + b.getErrorMessage(self._handle))
 
+    # ---- decoded images from a loader, batch by batch through a ring of packed pinned / device buffers
+    def packed_source(self, max_width, max_height, queue_depth=2, slot_bytes=0, is_output=False):
+        """A source fed image by image (place_image) and batch by batch (push): stands where the reference's loader copies every
+        decoded image into a padded batch. One asynchronous copy of the bytes written per batch; run() consumes the oldest batch."""
+        src = b.packedSource(self._handle, max_width, max_height, is_output, queue_depth, slot_bytes)
+        if not src:
+            raise RuntimeError("packed_source failed: " + b.getErrorMessage(self._handle))
+        return src
+
+    def place_image(self, source, index, image):
+        """image: numpy uint8 [h, w, 3], written into the pinned slot of the batch being assembled (rows at dword pitch)."""
+        import ctypes as C
+        import numpy as np
+        image = np.ascontiguousarray(image, dtype=np.uint8)
+        h, w, c = image.shape
+        assert c == 3
+        ptr, stride = b.packedSourcePlaceImage(self._handle, source, index, w, h)
+        if not ptr:
+            raise RuntimeError("place_image failed: " + b.getErrorMessage(self._handle))
+        dst = np.ctypeslib.as_array((C.c_ubyte * (stride * h)).from_address(ptr)).reshape(h, stride)
+        dst[:, :3 * w] = image.reshape(h, 3 * w)
+
+    def push(self, source):
+        if b.packedSourcePush(self._handle, source) != types.OK:
+            raise RuntimeError("push failed: " + b.getErrorMessage(self._handle))
+
+    def wait_for_batch(self, source):
+        """Blocks until the loader has pushed a batch (rocal_run on an empty ring raises instead of blocking)."""
+        if b.packedSourceWait(self._handle, source) != types.OK:
+            raise RuntimeError("wait_for_batch failed: " + b.getErrorMessage(self._handle))
+
+    def queued_batches(self, source):
+        return b.packedSourceLevel(self._handle, source)
+
     def bind_output(self, output, tensor):
         """The node that produces `output` writes straight into `tensor` (a torch CUDA tensor the caller owns): no copy afterwards."""
         assert tensor.is_cuda and tensor.is_contiguous() and tensor.numel() * tensor.element_size() >= b.tensorDataSize(output)
