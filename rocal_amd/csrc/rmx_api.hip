@@ -297,7 +297,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->fast_wpb = tune_env("RMX_TUNE_FAST_WPB", ctx->fast_wpb, 1, 4);
         ctx->upload_kernel = tune_env("RMX_TUNE_UPLOAD_KERNEL", ctx->upload_kernel, 0, 1);
         ctx->dma = tune_env("RMX_TUNE_DMA", ctx->dma, 0, 1);  // 0: the bilinear fast path always stages through registers
-        ctx->dma_lds = tune_env("RMX_TUNE_DMA_LDS", ctx->dma_lds, 2048, 10 * 1024) & ~15;  // LDS window of a wavefront
+        ctx->dma_lds = tune_env("RMX_TUNE_DMA_LDS", ctx->dma_lds, 2048, 32 * 1024) & ~15;  // LDS window of a wavefront
         ctx->dma_group = tune_env("RMX_TUNE_DMA_GROUP", ctx->dma_group, 0, 16);  // windows per wavefront, 0: chosen per batch
         ctx->tri_wpb = tune_env("RMX_TUNE_TRI_WPB", ctx->tri_wpb, 1, 4);
         ctx->warp_passes = tune_env("RMX_TUNE_WARP_PASSES", ctx->warp_passes, 1, 8);
@@ -961,7 +961,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         if (dfn) {
             // 10 KB measured best on MI355X: smaller caps cut more rows into two tiles, and the kernel's registers allow 16
             // wavefronts per CU, which 10 KB each still fit
-            const int bufcap = std::min(op->ctx->dma_lds, 10 * 1024);  // the kernel issues at most 10 loads of 1 KB per window
+            const int bufcap = op->ctx->dma_lds;
             int need_max = 64;
             for (int i = 0; i < op->n && dma; i++) {
                 RmxSample &s = t[i];

@@ -232,7 +232,10 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     // memory operations of a wavefront complete in issue order, so the wait for those loads, which allows the DEFERRED
     // youngest operations (the held-back stores) to be outstanding, never waits for a store to reach memory.
     constexpr bool DEFER = sizeof(T) <= 2;  // (an fp32 run is 24 registers: stored at once)
-    constexpr int DEFERRED = 3;             // store instructions of one packed group of 1- and 2-byte elements, both layouts
+    // The FEWEST store instructions a held-back group can become (more are harmless, fewer would let a load slip through the
+    // wait): three planes are three instructions; an interleaved run is contiguous and the compiler merges its stores up to
+    // 16 bytes each: 48 bytes of fp16 are three, 24 bytes of u8 two. tests/test_dma_waitcnt_cpu.py checks the generated code.
+    constexpr int DEFERRED = (LAYOUT == RMX_NHWC && sizeof(T) == 1) ? 2 : 3;
     int tile = 0, r0 = r_begin;
     DmaTile g = tile_geom(0);
     int a_v = issue(g, r0, min(r0 + wrows, r_end));
