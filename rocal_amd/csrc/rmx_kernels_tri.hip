@@ -15,6 +15,10 @@
 
 #include <type_traits>
 
+#ifndef RMX_TRI_DOWN_ATTR
+#define RMX_TRI_DOWN_ATTR
+#endif
+
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_tri[];
@@ -317,7 +321,7 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
 constexpr int TDM = 4;  // output rows in flight
 
 template <typename T, int LAYOUT, bool NORM, bool QUANT>
-__global__ void __launch_bounds__(256) rmx_resize_tri_down_kernel(RmxKArgs a) {
+__global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_kernel(RmxKArgs a) {
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const int wib = threadIdx.x / RMX_WAVE;
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
