@@ -14,19 +14,17 @@ struct SectorRow {
     float sg[3], nb0;  // sg of r,g,b ; nb of r
     float nb1, nb2, pad0, pad1;  // nb of g,b
 };
-RMX_DEV void sector_row(int hi, SectorRow &row) {
+constexpr SectorRow sector_row(int hi) {
     // codes: 0 = V, 1 = q, 2 = p, 3 = t
     const int rc[6] = {0, 1, 2, 2, 3, 0}, gc[6] = {3, 0, 0, 1, 2, 2}, bc[6] = {2, 2, 3, 0, 0, 1};
     const int h = hi == 6 ? 0 : (hi > 5 ? 5 : hi);  // row 6 repeats row 0 (see the hue reduction), row 7 is never read
     const int code[3] = {rc[h], gc[h], bc[h]};
-    float sg[3], nb[3];
-#pragma unroll
+    float sg[3] = {0.0f, 0.0f, 0.0f}, nb[3] = {0.0f, 0.0f, 0.0f};
     for (int c = 0; c < 3; c++) {
         sg[c] = code[c] == 1 ? -1.0f : (code[c] == 3 ? 1.0f : 0.0f);
         nb[c] = code[c] >= 2 ? -1.0f : 0.0f;
     }
-    row.sg[0] = sg[0]; row.sg[1] = sg[1]; row.sg[2] = sg[2]; row.nb0 = nb[0];
-    row.nb1 = nb[1]; row.nb2 = nb[2]; row.pad0 = 0.0f; row.pad1 = 0.0f;
+    return SectorRow{{sg[0], sg[1], sg[2]}, nb[0], nb[1], nb[2], 0.0f, 0.0f};
 }
 
 // Branch-free: lanes of a wavefront hold pixels of different hue sectors, so
@@ -61,21 +59,29 @@ RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const Sect
     b = __builtin_fmaf(bo, alpha, beta);
 }
 
-// The two tables of the twist in LDS: correctly rounded reciprocals of 0..255 (entry 0 is 0) and the sector coefficients.
+// The two tables of the twist: correctly rounded reciprocals of 0..255 (entry 0 is 0) and the sector coefficients. They are
+// made by the compiler (IEEE division in a constant expression gives the same bits as the division on the device) and lie in
+// device memory; a wavefront copies them into LDS, where the per-lane look-ups go.
 struct __attribute__((aligned(16))) ColorTables {
     float rcp[256];
     SectorRow sect[8];
 };
+constexpr ColorTables make_color_tables() {
+    ColorTables t{};
+    for (int v = 0; v < 256; v++) t.rcp[v] = (v == 0) ? 0.0f : 1.0f / (float)v;
+    for (int h = 0; h < 8; h++) t.sect[h] = sector_row(h);
+    return t;
+}
+static __device__ const ColorTables rmx_color_tables_rom = make_color_tables();
 
-// Fills the tables from one wavefront. Every wavefront of a workgroup writes the same values, so none has to wait for another:
-// each reads only what it has written itself.
+// Copies the tables into LDS from one wavefront: 80 pieces of 16 bytes, one per lane and 16 more. Every wavefront of a
+// workgroup writes the same values, so none has to wait for another: each reads only what it has written itself.
 RMX_DEV void color_tables_fill(ColorTables *t, int lane) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int v = lane + RMX_WAVE * i;
-        t->rcp[v] = (v == 0) ? 0.0f : 1.0f / (float)v;
-    }
-    if (lane < 8) sector_row(lane, t->sect[lane]);
+    static_assert(sizeof(ColorTables) == 80 * 16, "layout of the colour tables");
+    const uint4 *src = reinterpret_cast<const uint4 *>(&rmx_color_tables_rom);
+    uint4 *dst = reinterpret_cast<uint4 *>(t);
+    dst[lane] = src[lane];
+    if (lane < 16) dst[RMX_WAVE + lane] = src[RMX_WAVE + lane];
     wave_sync();
 }
 

@@ -16,12 +16,14 @@ enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
 
 template <typename T, int LAYOUT, int KIND, bool FAST>
 __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
-    __shared__ float rcp[256];
-    __shared__ __attribute__((aligned(16))) SectorRow sect[8];
+    __shared__ ColorTables tabs;
+    const float *rcp = tabs.rcp;
+    const SectorRow *sect = tabs.sect;
     if constexpr (KIND == COLOR_TWIST) {
-        int t = threadIdx.x;
-        if (t < 256) rcp[t] = (t == 0) ? 0.0f : 1.0f / (float)t;
-        if (t < 8) sector_row(t, sect[t]);
+        // the workgroup copies the two tables of the twist from device memory into LDS, 16 bytes per thread
+        const uint4 *rom = reinterpret_cast<const uint4 *>(&rmx_color_tables_rom);
+        uint4 *ram = reinterpret_cast<uint4 *>(&tabs);
+        for (unsigned i = threadIdx.x; i < sizeof(ColorTables) / 16; i += blockDim.x) ram[i] = rom[i];
         __syncthreads();
     }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
