@@ -61,3 +61,41 @@ def test_no_alloc_entry_point_refuses_a_batch_beyond_its_table(ctx):
     one = np.ones(n * 3, np.float32)
     with pytest.raises(RmxError, match="exceeds the 512 rows"):
         ops.resize_cmn_noalloc(ctx, sd, dd, src, dst, None, np.full(n, 8, np.uint32), np.full(n, 8, np.uint32), one, one)
+
+
+def test_no_alloc_entry_point_can_be_captured_in_a_graph():
+    """The whole call (its fill kernels carry the parameter rows as arguments) is recorded in a HIP graph and replayed on new
+    pixels, with eager work and synchronisation between the replays; every replay equals the eager call."""
+    import torch
+    s = torch.cuda.Stream()
+    c2 = ops.Context(0, stream=s.cuda_stream)
+    n, H, W, oh, ow = 9, 72, 96, 40, 48
+    img, roi, dw, dh, mirror, scale, bias = _case(5, n, H, W, oh, ow)
+    sd, dd = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, oh, ow, ops.NCHW, ops.FP16)
+    flags = ops.F_QUANTIZE_U8
+    with torch.cuda.stream(s):
+        src = torch.from_numpy(img).cuda()
+        out = torch.zeros((n, 3, oh, ow), dtype=torch.float16, device="cuda")
+        ops.resize_cmn_noalloc(c2, sd, dd, src, out, roi, dw, dh, scale, bias, mirror, flags=flags)  # warm-up before the capture
+        s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        ops.resize_cmn_noalloc(c2, sd, dd, src, out, roi, dw, dh, scale, bias, mirror, flags=flags)
+    rng = np.random.default_rng(8)
+    for rep in range(4):
+        pixels = rng.integers(0, 256, img.shape, dtype=np.uint8)
+        with torch.cuda.stream(s):
+            src.copy_(torch.from_numpy(pixels))
+            out.zero_()
+            g.replay()
+            s.synchronize()
+            got = out.cpu().numpy()
+            eager = torch.zeros_like(out)
+            ops.resize_cmn_noalloc(c2, sd, dd, src, eager, roi, dw, dh, scale, bias, mirror, flags=flags)
+            s.synchronize()
+        assert np.array_equal(got.view(np.uint16), eager.cpu().numpy().view(np.uint16)), "replay %d differs from the eager call" % rep
+        exp = orc.resize(pixels, roi, dw, dh, oh, ow, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                         flags=orc.F_QUANTIZE_U8)
+        for i in range(n):
+            assert np.array_equal(got[i, :, :dh[i], :dw[i]].view(np.uint16), exp[i, :, :dh[i], :dw[i]].view(np.uint16)), "replay %d, sample %d" % (rep, i)
+    c2.close()
