@@ -98,6 +98,9 @@ extern "C" RocalStatus ROCAL_API_CALL rocalTensorSetBuffer(RocalContext context,
 // x,y,w,h per sample
 extern "C" const unsigned *ROCAL_API_CALL rocalTensorRoi(RocalTensor tensor);
 extern "C" size_t ROCAL_API_CALL rocalTensorDataSize(RocalTensor tensor);
+// Padded dimensions in the order of the layout ({N,H,W,C} or {N,C,H,W}), layout and data type of a tensor
+// (rocalTensor::dims / layout / data_type, rocAL/include/api/rocal_api_tensor.h:60-90).
+extern "C" RocalStatus ROCAL_API_CALL rocalTensorInfo(RocalTensor tensor, size_t dims[4], int *layout, int *data_type);
 
 /* ---- tensors the caller wants to read after a run (rocal_api_data_transfer.h:75): called before rocalVerify, as the Python
    pipeline does for what define_graph returns; a tensor created with is_output = true is an output already. ---- */

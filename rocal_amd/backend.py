@@ -25,6 +25,7 @@ _SIGS = {
     "rocalPackedSourcePush": (_i, [_vp, _vp]), "rocalPackedSourceWait": (_i, [_vp, _vp]), "rocalPackedSourceLevel": (C.c_size_t, [_vp, _vp]),
     "rocalTensorBuffer": (_vp, [_vp]), "rocalTensorRoi": (C.POINTER(_u), [_vp]), "rocalTensorDataSize": (C.c_size_t, [_vp]),
     "rocalTensorSetBuffer": (_i, [_vp, _vp, _vp]),
+    "rocalTensorInfo": (_i, [_vp, C.POINTER(C.c_size_t), C.POINTER(_i), C.POINTER(_i)]),
     "rocalToTensor": (_i, [_vp, _vp, _i, _i, _f, _f, _f, _f, _f, _f, _b, _i, _i, _i]),
     "rocalCropResize": (_vp, [_vp, _vp, _u, _u, _b, _vp, _vp, _vp, _vp, _i, _i]),
     "rocalROIResize": (_vp, [_vp, _vp, _u, _u, _b, _u, _u, _f, _f, _i, _i, _i]),
@@ -186,6 +187,14 @@ class Backend:
 
     def tensorDataSize(self, t):
         return host().rocalTensorDataSize(t)
+
+    def tensorInfo(self, t):
+        """(dims in the order of the layout, layout, data type)"""
+        dims = (C.c_size_t * 4)()
+        layout, dtype = _i(0), _i(0)
+        if host().rocalTensorInfo(t, dims, C.byref(layout), C.byref(dtype)) != 0:
+            raise ValueError("not a tensor")
+        return [int(d) for d in dims], int(layout.value), int(dtype.value)
 
     def tensorRoi(self, t, n):
         p = host().rocalTensorRoi(t)

@@ -236,6 +236,15 @@ void rocalSetOutputs(RocalContext p_context, unsigned int num_of_outputs, std::v
     for (unsigned i = 0; i < num_of_outputs; i++) context->master_graph->set_output(static_cast<Tensor *>(output_tensors[i]));
 }
 
+RocalStatus rocalTensorInfo(RocalTensor p_tensor, size_t dims[4], int *layout, int *data_type) {
+    if (!p_tensor || !dims || !layout || !data_type) return ROCAL_INVALID_PARAMETER_TYPE;
+    const TensorInfo &info = static_cast<Tensor *>(p_tensor)->info();
+    for (size_t i = 0; i < 4; i++) dims[i] = i < info.dims().size() ? info.dims()[i] : 1;
+    *layout = (int)info.layout();
+    *data_type = (int)info.data_type();
+    return ROCAL_OK;
+}
+
 RocalStatus rocalTensorSetBuffer(RocalContext p_context, RocalTensor p_tensor, void *device_ptr) {
     if (!p_context) return ROCAL_CONTEXT_INVALID;
     auto *context = static_cast<Context *>(p_context);

@@ -139,6 +139,17 @@ class Pipeline:
         if b.tensorSetBuffer(self._handle, output, tensor.data_ptr()) != types.OK:
             raise RuntimeError("bind_output failed: " + b.getErrorMessage(self._handle))
 
+    def output_dlpack(self, output):
+        """A DLPack capsule of an output tensor: `torch.from_dlpack(pipe.output_dlpack(out))` aliases the buffer the last node
+        wrote (no copy); valid until the next run writes it again. With bind_output the direction is the other way round (the
+        node writes into the consumer's tensor)."""
+        from . import dlpack
+        dims, _, dtype = b.tensorInfo(output)
+        ptr = b.tensorBuffer(output)
+        if not ptr:
+            raise RuntimeError("the tensor has no buffer yet (build the pipeline first)")
+        return dlpack.to_dlpack(ptr, dims, dtype, self._device_id, keep_alive=self)
+
     def output_roi(self, output):
         return b.tensorRoi(output, self._batch_size)
 

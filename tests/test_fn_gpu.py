@@ -80,3 +80,32 @@ def test_warp_affine_and_flip_pipeline():
     assert np.array_equal(t_wa.cpu().numpy(), exp)
     assert np.array_equal(t_fl.cpu().numpy(), exp[:, :, ::-1])
     pipe.release()
+
+
+def test_output_through_dlpack():
+    """The output tensor handed to torch as a DLPack capsule: the torch tensor aliases the buffer the node wrote (same device
+    address, no copy) and holds the oracle's values."""
+    import torch
+    img = _image()
+    pipe = Pipeline(batch_size=N, device_id=0, seed=3)
+    with pipe:
+        src = pipe.device_source(W, H)
+        out = fn.crop_mirror_normalize(src, crop=(32, 40), mean=MEAN, std=STD, mirror=1, output_layout=types.NCHW, output_dtype=types.FLOAT)
+        pipe.set_outputs(out)
+    pipe.build()
+    dimg = torch.from_numpy(img).cuda()
+    pipe.feed(src, dimg, [w for w, _ in ROIS], [h for _, h in ROIS])
+    pipe.rocal_run()
+    t = torch.from_dlpack(pipe.output_dlpack(out))
+    assert t.is_cuda and t.dtype == torch.float32 and tuple(t.shape) == (N, 3, 32, 40)
+    from rocal_amd import backend
+    assert t.data_ptr() == backend.Backend().tensorBuffer(out)
+    crop = np.stack([orc.fixed_crop(w, h, 40, 32, anchor=(0.5, 0.5)) for w, h in ROIS])
+    scale, bias = orc.cmn_scale_bias(MEAN, STD, N)
+    exp = orc.crop_mirror_normalize(img, crop, scale, bias, np.ones(N, np.uint32), 32, 40, orc.NCHW, orc.FP32)
+    got = t.cpu().numpy()
+    for i in range(N):
+        cw, ch = int(crop[i, 2]), int(crop[i, 3])
+        assert np.array_equal(got[i, :, :ch, :cw], exp[i, :, :ch, :cw]), "sample %d" % i
+    del t
+    pipe.release()
