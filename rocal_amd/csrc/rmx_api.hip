@@ -122,12 +122,17 @@ struct rmx_op {
     int aux0 = 0, aux1 = 0;
     int fast_lds = 0, fast_strips = 1, fast_rows = 8, fast_wpb = 1;  // plan of fn_fast
     int fast_aux1 = 0;                                               // aux1 of fn_fast
+    // the streaming bilinear kernel in its any-width form: taken when fn_fast cannot be (a width that is not a multiple of 8,
+    // a destination base off 16-byte alignment), before the general kernel
+    rmx::KernelFn fn_mid = nullptr;
+    const char *mid_name = "";
+    int mid_lds = 0, mid_strips = 1, mid_rows = 4, mid_wpb = 1, mid_aux1 = 1;
     bool fast_needs_src16 = false;                                   // fn_fast also wants a 16-byte aligned source base
     uint64_t algo_bytes = 0;
     int stats_mode = 0, stats_per_channel = 1;  // Normalize: what is computed on the device (bit 0 mean, bit 1 standard deviation)
     float stats_scale = 1.0f, stats_shift = 0.0f;
-    rmx::KernelFn lds_fn[2] = {};  // kernels whose static LDS size has been asked of the runtime ([0] general, [1] fast)
-    int lds_static[2] = {};
+    rmx::KernelFn lds_fn[3] = {};  // kernels whose static LDS size has been asked of the runtime ([0] general, [1] fast, [2] mid)
+    int lds_static[3] = {};
 };
 
 namespace {
@@ -347,16 +352,19 @@ const char *rmx_op_plan(const rmx_op *op) {
     if (op->fn_fast)
         snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d waves_per_block=%d fast=1 group=%d",
                  (long long)op->n * op->fast_strips, op->fast_strips, op->fast_rows, op->fast_lds, op->fast_wpb, std::max(1, op->fast_aux1));
+    else if (op->fn_mid)
+        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d waves_per_block=%d fast=0 any_width=1 group=%d",
+                 (long long)op->n * op->mid_strips, op->mid_strips, op->mid_rows, op->mid_lds, op->mid_wpb, std::max(1, op->mid_aux1));
     else
         snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=0",
                  (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block);
     return buf;
 }
-const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : op->kernel_name) : ""; }
+const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : (op->fn_mid ? op->mid_name : op->kernel_name)) : ""; }
 
 // static LDS of a kernel (bytes), asked of the runtime once per op and kernel; -1 (with the error set) when the query fails
 static int static_lds_of(rmx_op *op, rmx::KernelFn fn) {
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 3; i++)
         if (op->lds_fn[i] == fn) return op->lds_static[i];
     hipFuncAttributes attr;
     hipError_t e = hipFuncGetAttributes(&attr, reinterpret_cast<const void *>(fn));
@@ -364,7 +372,7 @@ static int static_lds_of(rmx_op *op, rmx::KernelFn fn) {
         fail(RMX_ERR_HIP, "hipFuncGetAttributes failed: %d (%s)", (int)e, hipGetErrorString(e));
         return -1;
     }
-    const int slot = (fn == op->fn_fast) ? 1 : 0;
+    const int slot = (fn == op->fn_fast) ? 1 : (fn == op->fn_mid ? 2 : 0);
     op->lds_fn[slot] = fn;
     op->lds_static[slot] = (int)attr.sharedSizeBytes;
     return op->lds_static[slot];
@@ -406,6 +414,7 @@ static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *
     if ((op->kind == OP_WARP_AFFINE || op->kind == OP_ROTATE) && (((uintptr_t)dst) & 15u)) a.aux1 &= ~1;  // packed stores need an aligned base
     // the fast specialisation wants 16-byte aligned batch bases (rows of both sides are then aligned too)
     const bool fast = op->fn_fast && (((uintptr_t)dst) & 15u) == 0 && (!op->fast_needs_src16 || (((uintptr_t)src) & 15u) == 0);
+    const bool mid = !fast && op->fn_mid;
     int wpb = op->waves_per_block;
     if (fast) {
         a.strips = op->fast_strips;
@@ -413,9 +422,15 @@ static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *
         a.aux0 = op->fast_rows;
         a.aux1 = op->fast_aux1;
         wpb = op->fast_wpb;
+    } else if (mid) {
+        a.strips = op->mid_strips;
+        a.lds_bytes = op->mid_lds;
+        a.aux0 = op->mid_rows;
+        a.aux1 = op->mid_aux1;
+        wpb = op->mid_wpb;
     }
     HIP_TRY(hipSetDevice(op->ctx->device));
-    rmx::KernelFn fn = fast ? op->fn_fast : op->fn;
+    rmx::KernelFn fn = fast ? op->fn_fast : (mid ? op->fn_mid : op->fn);
     // a workgroup's LDS = the wavefronts' dynamic slices + what the kernel declares statically (coalescing slabs, colour
     // tables): fewer wavefronts per workgroup when the sum would not fit
     const int static_lds = static_lds_of(op, fn);
@@ -902,9 +917,13 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
     // the whole source window of a strip of `rows` destination rows at once; the x-tile of a sample is
     // narrowed until that window fits the LDS budget of one wavefront.
     op->fn_fast = nullptr;
-    if (op->interp == RMX_INTERP_LINEAR && op->dst.w % 8 == 0) {
-        // (the kernel multiplies row indices and the row stride with 24-bit multiplies)
-        bool ok = op->src.w * 3u < (1u << 23) && op->src.h < (1u << 23);
+    op->fn_mid = nullptr;
+    if (op->interp == RMX_INTERP_LINEAR) {
+        // (the kernels multiply row indices and the row stride with 24-bit multiplies)
+        const bool base_ok = op->src.w * 3u < (1u << 23) && op->src.h < (1u << 23);
+        bool widths8 = op->dst.w % 8 == 0;
+        for (int i = 0; i < op->n && widths8; i++) widths8 = t[i].dst_w % 8 == 0;
+        bool ok = base_ok && widths8;
         // 4 rows and a 10 KB slice measured best on MI355X (more, shorter-lived wavefronts per CU)
         const int rows = op->ctx->fast_rows, cap = op->ctx->fast_lds;
         int need_max = 64;
@@ -948,17 +967,16 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             op->fast_aux1 = 0;
             if (op->fast_lds > op->ctx->max_lds_per_block - kStaticLdsMax) op->fn_fast = nullptr;
         }
-        // Streaming variant (source rows straight into LDS): needs every source row to start at
-        // the same byte phase (row stride a multiple of 4) and a destination format it is built for.
-        bool dma = ok && op->fn_fast && op->ctx->dma;
+        // Streaming kernel (source rows straight into LDS): needs every source row to start at the same byte phase (row stride
+        // a multiple of 4). Its any-width form serves every destination; the form for whole groups and aligned rows replaces
+        // the staged kernel above where that applies.
+        bool dma = base_ok && op->ctx->dma;
         if (dma) {
             if (op->layout.empty()) dma = (op->src.w * 3u) % 4u == 0;
             else
                 for (int i = 0; i < op->n && dma; i++) dma = op->layout[i].row_stride % 4u == 0;
         }
-        const char *dname = nullptr;
-        rmx::KernelFn dfn = dma ? rmx::select_resize_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &dname) : nullptr;
-        if (dfn) {
+        if (dma) {
             // 10 KB measured best on MI355X: smaller caps cut more rows into two tiles, and the kernel's registers allow 16
             // wavefronts per CU, which 10 KB each still fit
             const int bufcap = op->ctx->dma_lds;
@@ -986,17 +1004,31 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 }
             }
             if (dma && need_max <= op->ctx->max_lds_per_block - kStaticLdsMax) {
-                op->fn_fast = dfn;
-                op->fast_name = dname;
-                op->fast_lds = (need_max + 15) / 16 * 16;
-                op->fast_rows = rows;
                 // A wavefront works through `group` windows (of `rows` destination rows) below each other per x-tile, so that the
-                // tile's x taps are computed once for all of them; as many as still leave about four wavefronts per SIMD.
+                // tile's x taps are computed once for all of them (1 measured best: more leave too few wavefronts to fill the chip evenly).
                 const long windows = (long)op->n * ((max_dh + rows - 1) / rows);
                 const int group = op->ctx->dma_group ? op->ctx->dma_group : (int)std::max<long>(1, std::min<long>(8, windows / 4096));
-                op->fast_strips = std::max(1, (max_dh + rows * group - 1) / (rows * group));
-                op->fast_wpb = std::max(1, std::min(op->ctx->fast_wpb, (op->ctx->max_lds_per_block - kStaticLdsMax) / std::max(1, op->fast_lds)));
-                op->fast_aux1 = group;
+                const int lds = (need_max + 15) / 16 * 16;
+                const int strips = std::max(1, (max_dh + rows * group - 1) / (rows * group));
+                const int wpb = std::max(1, std::min(op->ctx->fast_wpb, (op->ctx->max_lds_per_block - kStaticLdsMax) / std::max(1, lds)));
+                op->fn_mid = rmx::select_resize_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, false, &op->mid_name);
+                op->mid_lds = lds;
+                op->mid_rows = rows;
+                op->mid_strips = strips;
+                op->mid_wpb = wpb;
+                op->mid_aux1 = group;
+                const char *dname = nullptr;
+                rmx::KernelFn dfn = widths8 ? rmx::select_resize_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, true, &dname) : nullptr;
+                if (dfn) {
+                    op->fn_fast = dfn;
+                    op->fast_name = dname;
+                    op->fast_lds = lds;
+                    op->fast_rows = rows;
+                    op->fast_strips = strips;
+                    op->fast_wpb = wpb;
+                    op->fast_aux1 = group;
+                    op->fast_needs_src16 = false;
+                }
             }
         }
     }

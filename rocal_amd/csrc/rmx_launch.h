@@ -9,7 +9,7 @@ typedef void (*KernelFn)(RmxKArgs);
 KernelFn select_cmn_kernel(int dtype, int layout, bool norm, bool fast, const char **name);
 KernelFn select_resize_linear_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name);
 KernelFn select_resize_fast_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name);
-KernelFn select_resize_dma_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name);
+KernelFn select_resize_dma_kernel(int dtype, int layout, bool norm, bool quant, int chain, bool aligned, const char **name);
 KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, const char **name);

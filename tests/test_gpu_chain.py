@@ -51,7 +51,7 @@ def _expected(img, roi, rw, rh, crop, scale, bias, mirror, oh, ow, layout, dtype
 
 @pytest.mark.parametrize("aligned", [True, False])
 @pytest.mark.parametrize("kind", ["brightness", "contrast", "twist", "hue", "saturation"])
-def test_resize_colour_cmn_chain(ctx, kind, aligned):
+def test_resize_colour_cmn_chain(ctx, ctx_staged, kind, aligned):
     import torch
     rng = np.random.default_rng(sum(map(ord, kind)) * 2 + int(aligned))
     n, H, W = 5, 90, 120
@@ -72,18 +72,27 @@ def test_resize_colour_cmn_chain(ctx, kind, aligned):
     mirror = rng.integers(0, 2, n).astype(np.uint32)
     scale, bias = _scale_bias(n)
     flag, arrays, colour_fn = _colour_params(kind, rng, n)
-    for layout, dtype in ((ops.NCHW, ops.FP16), (ops.NHWC, ops.FP32)):
-        op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, oh, ow, layout, dtype), ops.LINEAR,
-                        flags=ops.F_QUANTIZE_U8 | flag)
-        op.update_color_cmn(roi, rw, rh, scale, bias, arrays, mirror, crop)
-        # aligned: the streaming kernel (planar fp16; the source rows are 360 bytes) or the staged one (interleaved fp32)
-        assert op.kernel_name == (("rmx_resize_dma_kernel" if dtype == ops.FP16 else "rmx_resize_fast_kernel") if aligned else "rmx_resize_kernel")
-        out = op.alloc_output()
-        op.launch(torch.from_numpy(img).cuda(), out)
-        ctx.sync()
-        got = out.cpu().numpy()
-        exp = _expected(img, roi, rw, rh, crop, scale, bias, mirror, oh, ow, layout, dtype, colour_fn)
-        assert np.array_equal(_bits(got), _bits(exp)), "%s aligned=%s (%s, %s): %d values differ" % (kind, aligned, op.kernel_name, op.plan, int((got != exp).sum()))
+    # aligned: the streaming kernel (planar fp16; the source rows are 360 bytes) or the staged one (interleaved fp32).
+    # Any other width: the streaming kernel's any-width form, and the general kernel on a context without streaming.
+    streaming = {True: lambda dtype: "rmx_resize_dma_kernel" if dtype == ops.FP16 else "rmx_resize_fast_kernel",
+                 False: lambda dtype: "rmx_resize_dma_kernel"}[aligned]
+    cases = [(ctx, streaming)] + ([] if aligned else [(ctx_staged, lambda dtype: "rmx_resize_kernel")])
+    exp = {}
+    for c, name_of in cases:
+        for layout, dtype in ((ops.NCHW, ops.FP16), (ops.NHWC, ops.FP32)):
+            op = ops.Resize(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, oh, ow, layout, dtype), ops.LINEAR,
+                            flags=ops.F_QUANTIZE_U8 | flag)
+            op.update_color_cmn(roi, rw, rh, scale, bias, arrays, mirror, crop)
+            assert op.kernel_name == name_of(dtype), op.plan
+            out = op.alloc_output()
+            op.launch(torch.from_numpy(img).cuda(), out)
+            c.sync()
+            got = out.cpu().numpy()
+            if (layout, dtype) not in exp:
+                exp[layout, dtype] = _expected(img, roi, rw, rh, crop, scale, bias, mirror, oh, ow, layout, dtype, colour_fn)
+            e = exp[layout, dtype]
+            assert np.array_equal(_bits(got), _bits(e)), "%s aligned=%s (%s, %s): %d values differ" % (
+                kind, aligned, op.kernel_name, op.plan, int((got != e).sum()))
 
 
 def test_random_resized_crop_colour_twist_cmn_full_size(ctx):

@@ -73,6 +73,67 @@ def test_streaming_and_staged_kernels_agree_with_the_oracle(ctx, ctx_staged, ctx
     assert names == ["rmx_resize_dma_kernel", "rmx_resize_fast_kernel", "rmx_resize_dma_kernel"]
 
 
+@pytest.mark.parametrize("layout,dtype", [(ops.NCHW, ops.FP16), (ops.NCHW, ops.FP32), (ops.NCHW, ops.UINT8), (ops.NHWC, ops.FP16),
+                                          (ops.NHWC, ops.FP32), (ops.NHWC, ops.UINT8)])
+def test_streaming_kernel_any_width_and_any_destination_base(ctx, ctx_dma_small, layout, dtype):
+    """Destination widths that are not multiples of 8 (225, 37, 1 ...) and a destination whose first byte is not 16-byte
+    aligned: the streaming kernel's any-width form stores element by element. Every format, interleaved fp32 included; short
+    last groups of every length 1..7; mirrored and unmirrored; tiles cut by the small LDS setting; the padding around each
+    written window must keep the fill value."""
+    import torch
+    rng = np.random.default_rng(5100 + 7 * layout + dtype)
+    n, H, W = 12, 150, 200
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.empty((n, 4), np.uint32)
+    for i in range(n):
+        w, h = int(rng.integers(1, W + 1)), int(rng.integers(1, H + 1))
+        roi[i] = (int(rng.integers(0, W - w + 1)), int(rng.integers(0, H - h + 1)), w, h)
+    roi[0] = (0, 0, W, H)
+    roi[1] = (W - 9, H - 5, 9, 5)
+    roi[n - 1] = (W - 40, H - 30, 40, 30)  # ends on the last byte of the batch buffer
+    roi[2] = (3, 5, 1, 1)
+    OH, OW = 100, 229
+    dw = np.array([int(rng.integers(max(1, -(-int(roi[i, 2]) // 3)), OW + 1)) for i in range(n)], np.uint32)
+    dh = np.array([int(rng.integers(max(1, -(-int(roi[i, 3]) // 3)), OH + 1)) for i in range(n)], np.uint32)
+    dw[0], dh[0] = 225, 97
+    dw[2] = 1
+    dw[3:10] = 8 * (dw[3:10] // 8) + np.arange(1, 8)  # every length of the short last group
+    dw = np.minimum(dw, OW).astype(np.uint32)
+    mirror = rng.integers(0, 2, n).astype(np.uint32)
+    mirror[0] = 1
+    scale, bias = _scale_bias(n)
+    norm = dtype != ops.UINT8
+    flags = ops.F_QUANTIZE_U8 if norm else 0
+    exp = orc.resize(img, roi, dw, dh, OH, OW, interp=orc.LINEAR, mirror=mirror, scale=scale if norm else None, bias=bias if norm else None,
+                     layout=layout, dtype=dtype, flags=orc.F_QUANTIZE_U8 if norm else 0)
+    sd, dd = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, layout, dtype)
+    dimg = _gpu(img)
+    esz = exp.dtype.itemsize
+    for c in (ctx, ctx_dma_small):
+        op = ops.Resize(c, sd, dd, ops.LINEAR, flags=flags)
+        if norm:
+            op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        else:
+            op.update(roi, dw, dh, mirror)
+        assert op.kernel_name == "rmx_resize_dma_kernel" and "any_width=1" in op.plan, op.plan
+        for shift in (0, 1, 3):  # elements between a 256-byte boundary and the destination's first byte
+            raw = torch.full((exp.size * esz + 256,), 0x5A, dtype=torch.uint8, device="cuda")
+            out = raw[shift * esz: shift * esz + exp.size * esz].view(ops.torch_dtype(dtype)).view(exp.shape)
+            op.launch(dimg, out)
+            c.sync()
+            got = out.cpu().numpy()
+            fill = np.frombuffer(bytes([0x5A]) * esz, exp.dtype)[0]
+            want = np.full_like(exp, fill)
+            for i in range(n):
+                if layout == ops.NCHW:
+                    want[i, :, :dh[i], :dw[i]] = exp[i, :, :dh[i], :dw[i]]
+                else:
+                    want[i, :dh[i], :dw[i]] = exp[i, :dh[i], :dw[i]]
+            assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), "shift %d (%s)" % (shift, op.plan)
+            r = raw.cpu().numpy()
+            assert (r[:shift * esz] == 0x5A).all() and (r[shift * esz + exp.size * esz:] == 0x5A).all()
+
+
 @pytest.mark.parametrize("rows", [1, 3, 4, 8])
 def test_strip_heights(rows):
     """Strips of one to eight rows, with destination heights that leave a short last strip."""
