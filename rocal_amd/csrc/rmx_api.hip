@@ -81,7 +81,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -308,6 +308,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->warp_passes = tune_env("RMX_TUNE_WARP_PASSES", ctx->warp_passes, 1, 8);
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
         ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
+        ctx->tri_tpx = tune_env("RMX_TUNE_TRI_TPX", ctx->tri_tpx, 1, 2);     // output columns per lane of the downscaling kernel
     }
     *out = ctx;
     return RMX_OK;
@@ -759,7 +760,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         op->fn = rmx::select_resize_tri_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
         if (!op->fn) return fail(RMX_ERR_UNSUPPORTED, "triangular resize kernel not available");
         // 128 output columns per wave (two per lane); ring of horizontally filtered rows per wave
-        const int tile_w = 128;
+        int tile_w = 128;
         float max_ry = 1.0f, max_rx = 1.0f;
         for (int i = 0; i < op->n; i++) {
             if (t[i].dst_w <= 0 || t[i].dst_h <= 0) continue;
@@ -818,7 +819,8 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         }
         int rows = op->ctx->tri_rows > 0 ? op->ctx->tri_rows : 12;
         if (down) {
-            op->fn = rmx::select_resize_tri_down_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
+            tile_w = 64 * op->ctx->tri_tpx;
+            op->fn = rmx::select_resize_tri_down_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, op->ctx->tri_tpx, &op->kernel_name);
             // LDS slice: the rows of one staging round (four 16-byte loads per lane = 4, 2 or 1 rows, by row length)
             size_t lds = 0;
             for (int i = 0; i < op->n; i++) {
@@ -832,7 +834,8 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 const int need = std::max(pitch, std::max(2 * std::min(pitch, 512 + pads), 4 * std::min(pitch, 256 + pads)));
                 lds = std::max(lds, (size_t)need * 4);
             }
-            op->lds_per_wave = (int)((std::max<size_t>(lds, 64) + 15) / 16 * 16);  // the staged source rows only
+            // the staged source rows and the table of vertical coefficients (64 source rows x 4 output rows in flight)
+            op->lds_per_wave = (int)((std::max<size_t>(lds, 64) + 15) / 16 * 16) + 64 * 4 * 4;
             if (op->lds_per_wave > op->ctx->max_lds_per_block)
                 return fail(RMX_ERR_UNSUPPORTED, "triangular resize needs %d bytes of LDS per wave", op->lds_per_wave);
             // Rows per strip: a strip of R rows filters R*ratio + taps source rows, and the device runs the strips in

@@ -15,8 +15,10 @@
 
 #include <type_traits>
 
-#ifndef RMX_TRI_DOWN_ATTR
-#define RMX_TRI_DOWN_ATTR
+// Wavefronts per SIMD the register budget of the downscaling kernel is set for, by columns per lane (a workgroup of 256
+// threads is one wavefront per SIMD): 128 registers with two columns, 96 with one.
+#ifndef RMX_TRI_DOWN_WAVES
+#define RMX_TRI_DOWN_WAVES(npx) ((npx) == 1 ? 5 : 4)
 #endif
 
 namespace rmx {
@@ -320,8 +322,10 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
 // neighbouring lanes read source pixels `ratio` dwords apart, half the bank stride of adjacent column pairs.
 constexpr int TDM = 4;  // output rows in flight
 
-template <typename T, int LAYOUT, bool NORM, bool QUANT>
-__global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_kernel(RmxKArgs a) {
+template <typename T, int LAYOUT, bool NORM, bool QUANT, int NPX>
+__global__ void __launch_bounds__(256, RMX_TRI_DOWN_WAVES(NPX)) rmx_resize_tri_down_kernel(RmxKArgs a) {
+    constexpr int TPX = NPX;            // columns per lane: lane, lane + 64, ...
+    constexpr int TTW = RMX_WAVE * NPX;  // output columns per wave tile
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const int wib = threadIdx.x / RMX_WAVE;
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
@@ -365,6 +369,74 @@ __global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_ker
         bi[c] = P.bias[c];
     }
 
+    // tile-wide staged source column range (wave-uniform)
+    int l_first, l_last;
+    {
+        float w0;
+        tri_loc(ax, pcx + xt, (float)xlo, l_first, w0);
+        tri_loc(ax, pcx + xt + tw - 1, (float)xlo, l_last, w0);
+    }
+    const int cs = max(min(l_first, xhi), xlo);
+    const int ce = max(min(l_last + kx - 1, xhi), xlo);
+    const int items = (ce - cs + 4) >> 2;
+    // staged row: [lpad: copies of the first column][items*4 pixels from column cs][copies of the last column].
+    // With the border columns repeated in LDS no tap index needs clamping in the horizontal pass.
+    const int nrep_l = max(cs - l_first, 0), nrep_r = max(l_last + kx - 1 - ce, 0);
+    const int lpad = (nrep_l + 3) & ~3;
+    const int spitch = lpad + items * 4 + ((nrep_r + 3) & ~3);  // dwords per staged row
+
+    // ---- output rows of the strip, one per lane (a strip has at most 64 rows): first tap row and its weight offset;
+    // wave-uniform code fetches a row's entry with v_readlane
+    int oloc_v;
+    float ow0_v;
+    tri_loc(ay, pcy + min(r0 + lane, r1 - 1), (float)ylo, oloc_v, ow0_v);
+    auto row_loc = [&](int r) { return __builtin_amdgcn_readlane(oloc_v, r - r0); };
+    auto row_w0 = [&](int r) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, ow0_v), r - r0)); };
+    auto last_tap_row = [&](int r) { return max(min(row_loc(r) + ky - 1, yhi), ylo); };
+    const int y_first = max(min(row_loc(r0), yhi), ylo);
+    const int y_last = last_tap_row(r1 - 1);
+
+    // ---- staging plan of the tile. A row is `items` four-pixel items; a round is four 16-byte loads per lane:
+    // 4 rows of one slot, 2 rows of two slots or 1 row of up to four slots (a row has at most 3 x 64 items at up
+    // to 8 taps; spare slots repeat the last one). Everything that does not depend on the row is computed here:
+    // the dword-aligned byte offset of the slot's item inside a row, the byte phase (the same for all items of a
+    // lane, they are 12 bytes apart) and the item's place in the staged row.
+    const int spr = (items + RMX_WAVE - 1) / RMX_WAVE;
+    const int sh = spr == 1 ? 0 : (spr == 2 ? 1 : 2);  // log2(slots per row)
+    // every wide load of this wavefront stays inside the batch buffer (last row, last item, carry and load width)
+    // (rows longer than the three slots of a round take the row-by-row path as well)
+    const bool safe = items <= 3 * RMX_WAVE && simg + ((size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16) <= buf_end;
+    // rows per round, never more than the slice holds (then the spare slots repeat a row); the bounds-checked path
+    // stages one row at a time. (The tail of the slice holds the table of vertical coefficients.)
+    const int rpr = safe ? min(4 >> sh, max(1, ((a.lds_bytes >> 2) - TDM * RMX_WAVE) / spitch)) : 1;
+    // (the item's byte offset in memory follows from its place in the staged row: 3 bytes per dword, which is recomputed per
+    // load rather than kept in four more registers)
+    uint32_t sl_lds[4];
+    bool sl_on[4];
+    const uint32_t low = ((uint32_t)cs * 3u) & 3u;  // (items are 12 bytes apart: one phase for the whole row)
+    const uint32_t al_base = (((uint32_t)cs * 3u) & ~3u) - 3u * (uint32_t)lpad;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int k = min(i & ((1 << sh) - 1), spr - 1);
+        const int j = min(lane + RMX_WAVE * k, items - 1);
+        sl_lds[i] = (uint32_t)(lpad + 4 * j);
+        sl_on[i] = lane + RMX_WAVE * k < items;
+    }
+
+    // A round of loads. (Issuing the first round here, ahead of the set-up of the coefficients below, was measured: the 16
+    // registers it keeps busy make the compiler spill inside the filter loop, 86 us instead of 73.)
+    u32x4_a4 t[4];
+    auto issue = [&](int yb, int nr) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int q = min(i >> sh, nr - 1);
+            const uint32_t ro = (uint32_t)(yb + q) * row_stride + skew;  // wave-uniform: row start from base4
+            const uint32_t r = ro & 3u;
+            uint32_t place = sl_lds[i];
+            asm volatile("" : "+v"(place));  // (keeps the product below inside the loop)
+            t[i] = *reinterpret_cast<const u32x4_a4 *>(base4 + (((ro - r) + al_base + ((low + r) & 4u)) + 3u * place));
+        }
+    };
     // ---- per-lane columns: taps, coefficients (registers), column sums, destination column (mirrored if asked)
     int locx[TPX];
     bool col_on[TPX];
@@ -384,78 +456,55 @@ __global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_ker
 #pragma unroll
         for (int k = 0; k < 8; k++) creg[i][k] = (k < kx) ? tri_coeff(w0, ax.radius, k, ax.fscale) : 0.0f;
     }
-    // tile-wide staged source column range (wave-uniform)
-    int l_first, l_last;
-    {
-        float w0;
-        tri_loc(ax, pcx + xt, (float)xlo, l_first, w0);
-        tri_loc(ax, pcx + xt + tw - 1, (float)xlo, l_last, w0);
-    }
-    const int cs = max(min(l_first, xhi), xlo);
-    const int ce = max(min(l_last + kx - 1, xhi), xlo);
-    const int items = (ce - cs + 4) >> 2;
-    // staged row: [lpad: copies of the first column][items*4 pixels from column cs][copies of the last column].
-    // With the border columns repeated in LDS no tap index needs clamping in the horizontal pass.
-    const int nrep_l = max(cs - l_first, 0), nrep_r = max(l_last + kx - 1 - ce, 0);
-    const int lpad = (nrep_l + 3) & ~3;
-    const int spitch = lpad + items * 4 + ((nrep_r + 3) & ~3);  // dwords per staged row
+    // byte offsets of a lane's first taps inside a staged row
+    uint32_t tap_ofs[TPX];
+#pragma unroll
+    for (int i = 0; i < TPX; i++) tap_ofs[i] = (uint32_t)(lpad + locx[i] - cs) * 4u;
 
-    // ---- output rows in flight: rq .. rq+TDM-1 (wave-uniform state), slot 0 is the oldest
-    int rq = r0;
-    int qloc[TDM];
-    float qw0[TDM];
+    // sum of the vertical coefficients of output row r0 + lane, taps ascending; the row that completes fetches its sum from
+    // the lane that holds it
+    float rsum_v = 0.0f;
+    for (int j = 0; j < ky; j++) rsum_v += tri_coeff(ow0_v, ay.radius, j, ay.fscale);
+    rsum_v = (rsum_v == 0.0f) ? 1.0f : rsum_v;
+
+    // ---- output rows in flight: row r accumulates in slot (r - r0) & 3 until its last tap row has been added. rq is the
+    // oldest row in flight, qlast its last tap row (wave-uniform state).
     float acc[TDM][3][TPX];
 #pragma unroll
-    for (int m = 0; m < TDM; m++) {
-        tri_loc(ay, pcy + min(rq + m, r1 - 1), (float)ylo, qloc[m], qw0[m]);
+    for (int m = 0; m < TDM; m++)
 #pragma unroll
         for (int c = 0; c < 3; c++)
 #pragma unroll
             for (int i = 0; i < TPX; i++) acc[m][c][i] = 0.0f;
-    }
-    int y_last;
-    {
-        int loc;
-        float w0;
-        tri_loc(ay, pcy + r1 - 1, (float)ylo, loc, w0);
-        y_last = max(min(loc + ky - 1, yhi), ylo);
-    }
-    const int y_first = max(min(qloc[0], yhi), ylo);
-    // sum of the vertical coefficients of output row r0 + lane (a strip has at most 64 rows), taps ascending;
-    // the row that completes fetches its sum from the lane that holds it
-    float rsum_v = 0.0f;
-    {
-        int loc;
-        float w0;
-        tri_loc(ay, pcy + min(r0 + lane, r1 - 1), (float)ylo, loc, w0);
-        for (int j = 0; j < ky; j++) rsum_v += tri_coeff(w0, ay.radius, j, ay.fscale);
-        rsum_v = (rsum_v == 0.0f) ? 1.0f : rsum_v;
-    }
+    int rq = r0;
+    int qlast = last_tap_row(r0);
 
-    // ---- staging plan of the tile. A row is `items` four-pixel items; a round is four 16-byte loads per lane:
-    // 4 rows of one slot, 2 rows of two slots or 1 row of up to four slots (a row has at most 3 x 64 items at up
-    // to 8 taps; spare slots repeat the last one). Everything that does not depend on the row is computed here:
-    // the dword-aligned byte offset of the slot's item inside a row, the byte phase (the same for all items of a
-    // lane, they are 12 bytes apart) and the item's place in the staged row.
-    const int spr = (items + RMX_WAVE - 1) / RMX_WAVE;
-    const int sh = spr == 1 ? 0 : (spr == 2 ? 1 : 2);  // log2(slots per row)
-    // rows per round, never more than the slice holds (then the spare slots repeat a row)
-    const int rpr = min(4 >> sh, max(1, (a.lds_bytes >> 2) / spitch));
-    uint32_t sl_al[4], sl_lds[4];
-    bool sl_on[4];
-    const uint32_t low = ((uint32_t)(cs + 4 * min(lane, items - 1)) * 3u) & 3u;
+    // ---- vertical coefficients by source row, a table of 64 rows x 4 slots in the tail of the LDS slice: entry (l, k) is
+    // the coefficient with which source row ytab + l enters the output row of slot k (0: none; fma(h, 0, acc) == acc for
+    // the finite h a filtered row is, so all four slots take every row and no branch is needed). Lane l writes row l; the
+    // filter loop reads a row's entry with one broadcast read. Rebuilt every 64 source rows. The first and the last row
+    // of the window serve several taps of a row each (clamped tap indices) and take their own path below.
+    float *cftab = reinterpret_cast<float *>(srcrow + ((a.lds_bytes >> 2) - TDM * RMX_WAVE));
+    int ytab = y_first;
+    auto build_table = [&]() {
+        const int y = ytab + lane;
+        float cf[TDM];
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int k = min(i & ((1 << sh) - 1), spr - 1);
-        const int j = min(lane + RMX_WAVE * k, items - 1);
-        sl_al[i] = ((uint32_t)(cs + 4 * j) * 3u) & ~3u;
-        sl_lds[i] = (uint32_t)(lpad + 4 * j);
-        sl_on[i] = lane + RMX_WAVE * k < items;
-    }
-    // every wide load of this wavefront stays inside the batch buffer (last row, last item, carry and load width)
-    // (rows longer than the three slots of a round take the row-by-row path as well)
-    const bool safe = items <= 3 * RMX_WAVE && simg + ((size_t)y_last * row_stride + (size_t)(cs + 4 * (items - 1)) * 3 + 3 + 4 + 16) <= buf_end;
-
+        for (int k = 0; k < TDM; k++) cf[k] = 0.0f;
+        for (int rb = r0; rb < r1; rb += TDM) {
+#pragma unroll
+            for (int k = 0; k < TDM; k++) {
+                const int r = rb + k;
+                if (r < r1) {
+                    const int j = y - row_loc(r);
+                    const float c = tri_coeff(row_w0(r), ay.radius, j, ay.fscale);
+                    if ((uint32_t)j < (uint32_t)ky) cf[k] = c;
+                }
+            }
+        }
+        *reinterpret_cast<float4 *>(cftab + TDM * lane) = make_float4(cf[0], cf[1], cf[2], cf[3]);
+        wave_sync();
+    };
     // clamp-to-edge columns of the nr staged rows
     auto replicate = [&](int nr) {
         if (nrep_l + nrep_r > 0) {
@@ -470,16 +519,42 @@ __global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_ker
         }
     };
 
+    // An output row whose last tap row has been added: normalise, epilogue, store; its slot starts again at zero.
+    auto emit = [&](auto slot) {
+        constexpr int M = decltype(slot)::value;
+        const float rsum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rq - r0));
+#pragma unroll
+        for (int i = 0; i < TPX; i++) {
+            const float inv = 1 / (rsum * colsum[i]);
+#pragma unroll
+            for (int ch = 0; ch < 3; ch++) {
+                float t = acc[M][ch][i] * inv;
+                acc[M][ch][i] = 0.0f;
+                if constexpr (QUANT) t = round_u8(t);
+                if constexpr (NORM) t = __builtin_fmaf(t, sc[ch], bi[ch]);
+                // wave-uniform row pointer + the lane's column offset
+                if constexpr (LAYOUT == RMX_NCHW) {
+                    T *rowp = dimg + ((size_t)ch * a.dst_h + rq) * a.dst_w;
+                    if (col_on[i]) rowp[xcol[i]] = OutCvt<T>::cvt(t);
+                } else {
+                    T *rowp = dimg + (size_t)rq * a.dst_w * 3 + ch;
+                    if (col_on[i]) rowp[xcol[i] * 3u] = OutCvt<T>::cvt(t);
+                }
+            }
+        }
+    };
+
     // staged row q is source row yy: filter it and add it to the output rows in flight. NT = taps of the unrolled
     // horizontal pass (4, 6 or 8 >= kx): taps beyond kx carry coefficient 0 (fma(p, 0, a) == a for the finite p
     // an unpacked byte always is), so no bound test is needed inside; all LDS reads go out before the arithmetic.
     auto process_row = [&](auto nt, int q, int yy) {
         constexpr int NT = decltype(nt)::value;
-        const uint32_t *srow = srcrow + q * spitch + lpad;
+        const uint8_t *srow = reinterpret_cast<const uint8_t *>(srcrow) + (uint32_t)(q * spitch) * 4u;
         uint32_t px[TPX][NT];
+        const float4 cv4 = *reinterpret_cast<const float4 *>(cftab + TDM * (yy - ytab));
 #pragma unroll
         for (int i = 0; i < TPX; i++) {
-            const uint32_t *p0 = srow + (locx[i] - cs);
+            const uint32_t *p0 = reinterpret_cast<const uint32_t *>(srow + tap_ofs[i]);
 #pragma unroll
             for (int k = 0; k < NT; k++) px[i][k] = p0[k];
         }
@@ -497,67 +572,77 @@ __global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_ker
             h[1][i] = a1;
             h[2][i] = a2;
         }
-        // ---- vertical pass: the taps of the rows in flight that read source row yy (a tap index that
-        // leaves the window reads its first / last row, so the border rows can serve several taps)
+        // ---- vertical pass
+        if (yy != ylo && yy != yhi) {
+            // a row inside the window is one tap of every output row that reads it
+            const float cv[TDM] = {cv4.x, cv4.y, cv4.z, cv4.w};
 #pragma unroll
-        for (int m = 0; m < TDM; m++) {
-            if (rq + m < r1) {
-                int jlo = (yy == ylo) ? 0 : yy - qloc[m];
-                int jhi = (yy == yhi) ? ky - 1 : yy - qloc[m];
-                jlo = max(jlo, 0);
-                jhi = min(jhi, ky - 1);
-                for (int j = jlo; j <= jhi; j++) {
-                    const float c = tri_coeff(qw0[m], ay.radius, j, ay.fscale);
-#pragma unroll
-                    for (int ch = 0; ch < 3; ch++)
-#pragma unroll
-                        for (int i = 0; i < TPX; i++) acc[m][ch][i] = __builtin_fmaf(h[ch][i], c, acc[m][ch][i]);
-                }
-            }
-        }
-        // ---- rows whose last tap was this source row: normalise, epilogue, store, shift the queue
-        while (rq < r1 && max(min(qloc[0] + ky - 1, yhi), ylo) <= yy) {
-            const float rsum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rq - r0));
-#pragma unroll
-            for (int i = 0; i < TPX; i++) {
-                const float inv = 1 / (rsum * colsum[i]);
-#pragma unroll
-                for (int ch = 0; ch < 3; ch++) {
-                    float t = acc[0][ch][i] * inv;
-                    if constexpr (QUANT) t = round_u8(t);
-                    if constexpr (NORM) t = __builtin_fmaf(t, sc[ch], bi[ch]);
-                    // wave-uniform row pointer + the lane's column offset
-                    if constexpr (LAYOUT == RMX_NCHW) {
-                        T *rowp = dimg + ((size_t)ch * a.dst_h + rq) * a.dst_w;
-                        if (col_on[i]) rowp[xcol[i]] = OutCvt<T>::cvt(t);
-                    } else {
-                        T *rowp = dimg + (size_t)rq * a.dst_w * 3 + ch;
-                        if (col_on[i]) rowp[xcol[i] * 3u] = OutCvt<T>::cvt(t);
-                    }
-                }
-            }
-#pragma unroll
-            for (int m = 0; m + 1 < TDM; m++) {
-                qloc[m] = qloc[m + 1];
-                qw0[m] = qw0[m + 1];
+            for (int m = 0; m < TDM; m++)
 #pragma unroll
                 for (int ch = 0; ch < 3; ch++)
 #pragma unroll
-                    for (int i = 0; i < TPX; i++) acc[m][ch][i] = acc[m + 1][ch][i];
+                    for (int i = 0; i < TPX; i++) acc[m][ch][i] = __builtin_fmaf(h[ch][i], cv[m], acc[m][ch][i]);
+        } else {
+            // the first / last row of the window: every tap index that leaves the window reads it too, in tap order
+#pragma unroll
+            for (int m = 0; m < TDM; m++) {
+                const int r = rq + ((m - (rq - r0)) & (TDM - 1));  // the row in flight that lives in slot m
+                if (r < r1) {
+                    const int loc = row_loc(r);
+                    const float w0 = row_w0(r);
+                    int jlo = (yy == ylo) ? 0 : yy - loc;
+                    int jhi = (yy == yhi) ? ky - 1 : yy - loc;
+                    jlo = max(jlo, 0);
+                    jhi = min(jhi, ky - 1);
+                    for (int j = jlo; j <= jhi; j++) {
+                        const float c = tri_coeff(w0, ay.radius, j, ay.fscale);
+#pragma unroll
+                        for (int ch = 0; ch < 3; ch++)
+#pragma unroll
+                            for (int i = 0; i < TPX; i++) acc[m][ch][i] = __builtin_fmaf(h[ch][i], c, acc[m][ch][i]);
+                    }
+                }
+            }
+        }
+        // ---- rows whose last tap was this source row
+        while (qlast <= yy && rq < r1) {
+            switch ((rq - r0) & (TDM - 1)) {
+                case 0: emit(std::integral_constant<int, 0>{}); break;
+                case 1: emit(std::integral_constant<int, 1>{}); break;
+                case 2: emit(std::integral_constant<int, 2>{}); break;
+                default: emit(std::integral_constant<int, 3>{}); break;
             }
             rq++;
-            tri_loc(ay, pcy + min(rq + TDM - 1, r1 - 1), (float)ylo, qloc[TDM - 1], qw0[TDM - 1]);
-#pragma unroll
-            for (int ch = 0; ch < 3; ch++)
-#pragma unroll
-                for (int i = 0; i < TPX; i++) acc[TDM - 1][ch][i] = 0.0f;
+            qlast = last_tap_row(min(rq, r1 - 1));
         }
     };
 
     auto run = [&](auto nt) {
-        if (!safe) {
-            // the wavefront's rows touch the last bytes of the batch buffer: row by row, bounds-checked loads
-            for (int y = y_first; y <= y_last; y++) {
+        // Software pipeline over the rounds: the loads of the next round are issued before the rows of the current
+        // one are filtered and wait in registers, so a round trip to memory runs under the arithmetic of the
+        // previous round. The four loads are straight-line and unconditional (rows beyond the last repeat it).
+        if (safe) issue(y_first, min(rpr, y_last - y_first + 1));
+        build_table();  // (under the round trip of the first loads)
+        for (int y = y_first; y <= y_last;) {
+            const int nr = min(rpr, y_last - y + 1);
+            if (y + nr - ytab > RMX_WAVE) {
+                ytab = y;
+                build_table();
+            }
+            if (safe) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int q = min(i >> sh, nr - 1);
+                    const uint32_t r = ((uint32_t)(y + q) * row_stride + skew) & 3u;
+                    const uint32_t d[4] = {t[i].x, t[i].y, t[i].z, t[i].w};
+                    const uint4 px = expand4(d, (low + r) & 3u);
+                    if (sl_on[i]) *reinterpret_cast<uint4 *>(srcrow + (uint32_t)(q * spitch) + sl_lds[i]) = px;
+                }
+                wave_sync();
+                const int yn = y + nr;
+                issue(min(yn, y_last), max(1, min(rpr, y_last - yn + 1)));
+            } else {
+                // the wavefront's rows touch the last bytes of the batch buffer: row by row, bounds-checked loads
                 for (int j = lane; j < items; j += RMX_WAVE) {
                     const uint8_t *pp = simg + (size_t)y * row_stride + (size_t)(cs + 4 * j) * 3;
                     uint32_t w[3];
@@ -570,43 +655,11 @@ __global__ void __launch_bounds__(256) RMX_TRI_DOWN_ATTR rmx_resize_tri_down_ker
                     *reinterpret_cast<uint4 *>(srcrow + lpad + 4 * j) = px;
                 }
                 wave_sync();
-                replicate(1);
-                process_row(nt, 0, y);
-                wave_sync();  // the next row overwrites the staged one
             }
-            return;
-        }
-        // Software pipeline over the rounds: the loads of the next round are issued before the rows of the current
-        // one are filtered and wait in registers, so a round trip to memory runs under the arithmetic of the
-        // previous round. The four loads are straight-line and unconditional (rows beyond the last repeat it).
-        u32x4_a4 t[4];
-        auto issue = [&](int yb, int nr) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int q = min(i >> sh, nr - 1);
-                const uint32_t ro = (uint32_t)(yb + q) * row_stride + skew;  // wave-uniform: row start from base4
-                const uint32_t r = ro & 3u;
-                t[i] = *reinterpret_cast<const u32x4_a4 *>(base4 + ((ro - r) + sl_al[i] + ((low + r) & 4u)));
-            }
-        };
-        issue(y_first, min(rpr, y_last - y_first + 1));
-        for (int y = y_first; y <= y_last;) {
-            const int nr = min(rpr, y_last - y + 1);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int q = min(i >> sh, nr - 1);
-                const uint32_t r = ((uint32_t)(y + q) * row_stride + skew) & 3u;
-                const uint32_t d[4] = {t[i].x, t[i].y, t[i].z, t[i].w};
-                const uint4 px = expand4(d, (low + r) & 3u);
-                if (sl_on[i]) *reinterpret_cast<uint4 *>(srcrow + (uint32_t)(q * spitch) + sl_lds[i]) = px;
-            }
-            wave_sync();
-            const int yn = y + nr;
-            issue(min(yn, y_last), max(1, min(rpr, y_last - yn + 1)));
             replicate(nr);
             for (int q = 0; q < nr; q++) process_row(nt, q, y + q);
             wave_sync();  // the next round overwrites the staged rows
-            y = yn;
+            y += nr;
         }
     };
     if (kx <= 4) run(std::integral_constant<int, 4>{});
@@ -637,27 +690,33 @@ KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, 
     }
 }
 
-template <typename T, int LAYOUT>
+template <typename T, int LAYOUT, int NPX>
 static KernelFn pick3_down(bool norm, bool quant) {
-    if (norm && quant) return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, true, true>;
-    if (norm) return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, true, false>;
-    return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, false, false>;
+    if (norm && quant) return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, true, true, NPX>;
+    if (norm) return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, true, false, NPX>;
+    return (KernelFn)rmx_resize_tri_down_kernel<T, LAYOUT, false, false, NPX>;
 }
 
-KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
-    *name = "rmx_resize_tri_down_kernel";
+template <int NPX>
+static KernelFn pick_down(int dtype, int layout, bool norm, bool quant) {
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return pick3_down<float, RMX_NCHW>(norm, quant);
-            case RMX_FP16: return pick3_down<__half, RMX_NCHW>(norm, quant);
-            default: return pick3_down<uint8_t, RMX_NCHW>(norm, quant);
+            case RMX_FP32: return pick3_down<float, RMX_NCHW, NPX>(norm, quant);
+            case RMX_FP16: return pick3_down<__half, RMX_NCHW, NPX>(norm, quant);
+            default: return pick3_down<uint8_t, RMX_NCHW, NPX>(norm, quant);
         }
     }
     switch (dtype) {
-        case RMX_FP32: return pick3_down<float, RMX_NHWC>(norm, quant);
-        case RMX_FP16: return pick3_down<__half, RMX_NHWC>(norm, quant);
-        default: return pick3_down<uint8_t, RMX_NHWC>(norm, quant);
+        case RMX_FP32: return pick3_down<float, RMX_NHWC, NPX>(norm, quant);
+        case RMX_FP16: return pick3_down<__half, RMX_NHWC, NPX>(norm, quant);
+        default: return pick3_down<uint8_t, RMX_NHWC, NPX>(norm, quant);
     }
+}
+
+// columns_per_lane: 1 (tiles of 64 output columns) or 2 (tiles of 128)
+KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, int columns_per_lane, const char **name) {
+    *name = "rmx_resize_tri_down_kernel";
+    return columns_per_lane == 1 ? pick_down<1>(dtype, layout, norm, quant) : pick_down<2>(dtype, layout, norm, quant);
 }
 
 }  // namespace rmx
