@@ -818,7 +818,33 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             }
         }
         int rows = op->ctx->tri_rows > 0 ? op->ctx->tri_rows : 12;
-        if (down) {
+        // Streaming form of the downscaling variant (source rows straight into LDS as raw bytes): every source row must start
+        // at the same byte phase (row stride a multiple of 4), and four LDS rows of the widest tile plus the table of vertical
+        // coefficients must leave room for ten wavefronts per CU at least.
+        bool tdma = down && op->ctx->dma && op->ctx->tri_tpx == 2 && ky <= 64;
+        if (tdma) {
+            if (op->layout.empty()) tdma = (op->src.w * 3u) % 4u == 0;
+            else
+                for (int i = 0; i < op->n && tdma; i++) tdma = op->layout[i].row_stride % 4u == 0;
+        }
+        if (tdma) {
+            size_t pitch_max = 64;
+            for (int i = 0; i < op->n; i++) {
+                const RmxSample &s = t[i];
+                if (s.dst_w <= 0 || s.dst_h <= 0) continue;
+                const int kxi = (int)std::ceil(2.0f * std::max(s.rx, 1.0f));
+                const int cols = std::min<int>((int)op->src.w, (int)std::ceil(128 * (double)std::max(s.rx, 1.0f))) + kxi + 4;
+                // margin (two pieces at most) + phase + data + right replicas + the reach of an 8-tap read, in whole pieces
+                pitch_max = std::max(pitch_max, (size_t)32 + (size_t)((3 + 3 * (cols + 8) + 8 + 15) / 16 * 16));
+            }
+            const size_t lds = 4 * pitch_max + (64 + 64) * 4 * 4;  // + vertical coefficients: 64 source rows and 64 passes x 4 slots
+            if (pitch_max > 128 * 16 || lds > 16 * 1024) tdma = false;
+            else {
+                op->fn = rmx::select_resize_tri_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
+                op->lds_per_wave = (int)lds;
+            }
+        }
+        if (down && !tdma) {
             tile_w = 64 * op->ctx->tri_tpx;
             op->fn = rmx::select_resize_tri_down_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, op->ctx->tri_tpx, &op->kernel_name);
             // LDS slice: the rows of one staging round (four 16-byte loads per lane = 4, 2 or 1 rows, by row length)
@@ -838,12 +864,15 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             op->lds_per_wave = (int)((std::max<size_t>(lds, 64) + 15) / 16 * 16) + 64 * 4 * 4;
             if (op->lds_per_wave > op->ctx->max_lds_per_block)
                 return fail(RMX_ERR_UNSUPPORTED, "triangular resize needs %d bytes of LDS per wave", op->lds_per_wave);
+        }
+        if (down) {
             // Rows per strip: a strip of R rows filters R*ratio + taps source rows, and the device runs the strips in
             // rounds of (wavefront slots) at a time; pick the R with the least rounds x rows-per-strip. Measured on
             // MI355X: a batch of equal strips that march in step runs 10-20 % slower than one whose last strip of each
             // image is a short one, so an R that leaves a remainder of at most R/2 rows is preferred.
             if (op->ctx->tri_rows == 0) {
-                const int per_cu = std::max(1, std::min(16, (160 * 1024) / op->lds_per_wave));
+                // (wavefronts per CU: 16 by the registers of the kernel that stages through registers, 20 by those of the streaming one)
+                const int per_cu = std::max(1, std::min(tdma ? 20 : 16, (160 * 1024) / op->lds_per_wave));
                 const long slots = (long)op->ctx->num_cus * per_cu;
                 double best_cost = 0.0;
                 for (int r = 4; r <= 64; r++) {

@@ -35,6 +35,23 @@ RMX_DEV const uint8_t *sample_base(const RmxKArgs &a, int s, uint32_t &row_strid
     return a.src + (size_t)s * a.src_h * row_stride;
 }
 
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
+typedef const __attribute__((address_space(1))) void *glb_ptr_t;
+typedef __attribute__((address_space(3))) uint8_t lds_u8;    // explicit LDS pointers: every access below is a DS instruction,
+typedef __attribute__((address_space(3))) uint32_t lds_u32;  // never a FLAT one (which would also count as vector memory)
+
+// A wave-uniform value that the vector unit produced (float arithmetic has no scalar form), moved into a scalar register
+// by an instruction the optimiser cannot look through: everything derived from it stays scalar arithmetic. (The
+// readfirstlane builtin is folded away for values known to be uniform, and the dependants then run on the vector unit.)
+// The compiler does not see inside the statement, so the wait states this chip wants around the instruction are spelled
+// out: one between a vector instruction that writes the source register and the read of it, five before a vector memory
+// instruction may read the scalar result (two before a vector ALU instruction may).
+RMX_DEV int to_sgpr(int v) {
+    int r;
+    asm("s_nop 0\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(r) : "v"(v));
+    return r;
+}
+
 // Order LDS traffic between the lanes of one wavefront. A wave's DS instructions execute in
 // issue order, so no hardware barrier is needed: this only stops the compiler from moving
 // LDS reads above the writes they depend on.

@@ -41,11 +41,6 @@ namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_dma[];
 
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-typedef const __attribute__((address_space(1))) void *glb_ptr_t;
-typedef __attribute__((address_space(3))) uint8_t lds_u8;    // explicit LDS pointers: every access below is a DS instruction,
-typedef __attribute__((address_space(3))) uint32_t lds_u32;  // never a FLAT one (which would also count as vector memory)
-
 RMX_DEV float src_coord_d(int u, float ratio, float off, float lo) {
     float s = (float)u * ratio;
     s = s + off;
@@ -53,18 +48,6 @@ RMX_DEV float src_coord_d(int u, float ratio, float off, float lo) {
     return s;
 }
 
-
-// A wave-uniform value that the vector unit produced (float arithmetic has no scalar form), moved into a scalar register
-// by an instruction the optimiser cannot look through: everything derived from it stays scalar arithmetic. (The
-// readfirstlane builtin is folded away for values known to be uniform, and the dependants then run on the vector unit.)
-// The compiler does not see inside the statement, so the wait states this chip wants around the instruction are spelled
-// out: one between a vector instruction that writes the source register and the read of it, five before a vector memory
-// instruction may read the scalar result (two before a vector ALU instruction may).
-RMX_DEV int to_sgpr(int v) {
-    int r;
-    asm("s_nop 0\n\tv_readfirstlane_b32 %0, %1\n\ts_nop 4" : "=s"(r) : "v"(v));
-    return r;
-}
 
 // One x-tile of a wavefront's rows: destination columns [xt, xt + tw) and the source columns they read. Wave-uniform.
 struct DmaTile {

@@ -12,6 +12,7 @@
 // Source rows enter the ring exactly once per strip; the intermediate never touches HBM.
 #include "rmx_device.h"
 #include "rmx_launch.h"
+#include "rmx_tri_math.h"
 
 #include <type_traits>
 
@@ -28,34 +29,6 @@ extern __shared__ uint32_t rmx_lds_tri[];
 constexpr int TTW = 128;  // output columns per wave tile
 constexpr int TPX = 2;    // columns per lane
 constexpr int TRB = 3;    // source rows staged per batch (one memory round trip per batch, not per row)
-
-struct TriAxis {
-    float ratio, radius, fscale, offset;
-    int ksize;
-};
-
-RMX_DEV TriAxis tri_axis(float ratio, float fscale) {
-    TriAxis t;
-    t.ratio = ratio;
-    t.radius = ratio > 1.0f ? ratio : 1.0f;
-    t.fscale = fscale;
-    t.offset = (ratio - 1) * 0.5f - t.radius;
-    t.ksize = (int)ceilf(t.radius * 2);
-    return t;
-}
-
-RMX_DEV void tri_loc(const TriAxis &t, int d, float lo, int &loc, float &w0) {
-    float raw = (float)d * t.ratio;
-    raw = raw + t.offset;
-    raw = raw + lo;
-    loc = (int)ceilf(raw);
-    w0 = (float)loc - raw;
-}
-
-RMX_DEV float tri_coeff(float w0, float radius, int k, float fscale) {
-    float c = 1 - fabsf((w0 - radius + (float)k) * fscale);
-    return c < 0 ? 0 : c;
-}
 
 template <typename T, int LAYOUT, bool NORM, bool QUANT>
 __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {

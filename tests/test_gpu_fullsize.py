@@ -126,15 +126,20 @@ def test_degenerate_samples(ctx):
     assert np.array_equal(got[0, :8, :8], exp[0, :8, :8]) and np.array_equal(got[2, :8, :16], exp[2, :8, :16])
 
 
+@pytest.mark.parametrize("streaming", [False, True])
 @pytest.mark.parametrize("rx,ry", [(1.3, 1.0), (1.9, 2.4), (3.0, 3.0), (3.7, 3.7), (2.5, 1.2)])
-def test_triangular_downscale_tap_and_row_length_classes(ctx, rx, ry):
-    """The downscaling triangular kernel: 4/6/8-tap specialisations, 1/2/3 load slots per source row, partial
-    last tile, per-sample windows, mirror, and an exact-size source whose last rows take the bounds-checked
-    loader. (rx, ry) are the ratios of the first sample; the others shrink a little more or less."""
+def test_triangular_downscale_tap_and_row_length_classes(ctx, rx, ry, streaming):
+    """The downscaling triangular kernels: 4/6/8-tap specialisations, 1/2/3 load slots per source row, partial
+    last tile, per-sample windows (edge replicas on both sides, windows away from the origin at every byte phase), mirror,
+    and an exact-size source whose last rows take the bounds-checked loader. (rx, ry) are the ratios of the first sample;
+    the others shrink a little more or less. streaming: a source width that is a multiple of 4 (every row starts at the
+    same byte phase), which the kernel that loads rows straight into LDS takes; otherwise the one that stages through
+    registers."""
     import torch
     rng = np.random.default_rng(int(rx * 100 + ry * 10))
     n, dw0, dh0 = 3, 200, 37
     W, H = int(round(dw0 * rx)) + 9, int(round(dh0 * ry)) + 5
+    W = (W + 3) // 4 * 4 if streaming else W | 1
     img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
     roi = np.array([[0, 0, W - 9, H - 5], [4, 3, W - 4, H - 3], [9, 5, W - 9, H - 5]], np.uint32)  # the last two end at (W-1, H-1)
     dw = np.array([dw0, dw0 - 8, dw0 - 7], np.uint32)
@@ -151,7 +156,7 @@ def test_triangular_downscale_tap_and_row_length_classes(ctx, rx, ry):
         else:
             op.update_cmn(roi, dw, dh, scale, bias, mirror)
             exp = orc.resize(img, roi, dw, dh, dh0, dw0, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=layout, dtype=dtype)
-        assert op.kernel_name == "rmx_resize_tri_down_kernel"
+        assert op.kernel_name == ("rmx_resize_tri_dma_kernel" if streaming else "rmx_resize_tri_down_kernel")
         out = op.alloc_output()
         op.launch(src.view(n, H, W, 3), out)
         ctx.sync()
@@ -160,7 +165,8 @@ def test_triangular_downscale_tap_and_row_length_classes(ctx, rx, ry):
 
 
 def test_triangular_ring_and_downscale_kernels_agree(ctx, monkeypatch):
-    """The same downscaling batch through the ring kernel (forced) and through the register kernel."""
+    """The same downscaling batch through the ring kernel (forced), the kernel that stages rows through registers (forced)
+    and the one that loads them straight into LDS."""
     import torch
     rng = np.random.default_rng(77)
     n, H, W = 2, 150, 260
@@ -168,17 +174,18 @@ def test_triangular_ring_and_downscale_kernels_agree(ctx, monkeypatch):
     roi = np.array([[0, 0, W, H], [10, 6, 240, 140]], np.uint32)
     dw, dh = np.array([96, 88], np.uint32), np.array([64, 50], np.uint32)
     outs = []
-    for ring in ("0", "1"):
+    for ring, dma, name in (("1", "1", "rmx_resize_tri_kernel"), ("0", "0", "rmx_resize_tri_down_kernel"), ("0", "1", "rmx_resize_tri_dma_kernel")):
         monkeypatch.setenv("RMX_TUNE_TRI_RING", ring)
+        monkeypatch.setenv("RMX_TUNE_DMA", dma)
         c2 = ops.Context()
         op = ops.Resize(c2, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 64, 96, ops.NCHW, ops.FP32), ops.TRIANGULAR)
         op.update(roi, dw, dh)
-        assert op.kernel_name == ("rmx_resize_tri_kernel" if ring == "1" else "rmx_resize_tri_down_kernel")
+        assert op.kernel_name == name
         out = op.alloc_output()
         op.launch(torch.from_numpy(img).cuda(), out)
         c2.sync()
         outs.append(out.cpu().numpy())
-    assert np.array_equal(_bits(outs[0]), _bits(outs[1]))
+    assert np.array_equal(_bits(outs[0]), _bits(outs[1])) and np.array_equal(_bits(outs[0]), _bits(outs[2]))
 
 
 @pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST])
