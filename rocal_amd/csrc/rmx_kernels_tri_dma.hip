@@ -19,6 +19,13 @@
 
 #include <type_traits>
 
+// " nt": streaming stores (the output is written once and read by another kernel much later)
+#ifdef RMX_TDMA_NT_ON
+#define RMX_TDMA_NT " nt"
+#else
+#define RMX_TDMA_NT ""
+#endif
+
 namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_tdma[];
@@ -60,9 +67,9 @@ RMX_DEV void tri_taps(const uint32_t (&e)[NE], const float (&c)[8], float &a0, f
 // instructions issued behind them, so their number must not be left to the compiler): `bits` to row + voff + OFF bytes.
 template <typename T, int OFF>
 RMX_DEV void store_elem(const T *row, uint32_t voff, uint32_t bits) {
-    if constexpr (sizeof(T) == 4) asm volatile("global_store_dword %0, %1, %2 offset:%3" ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
-    else if constexpr (sizeof(T) == 2) asm volatile("global_store_short %0, %1, %2 offset:%3" ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
-    else asm volatile("global_store_byte %0, %1, %2 offset:%3" ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
+    if constexpr (sizeof(T) == 4) asm volatile("global_store_dword %0, %1, %2 offset:%3" RMX_TDMA_NT ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
+    else if constexpr (sizeof(T) == 2) asm volatile("global_store_short %0, %1, %2 offset:%3" RMX_TDMA_NT ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
+    else asm volatile("global_store_byte %0, %1, %2 offset:%3" RMX_TDMA_NT ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
 }
 
 // acc += h * c and acc = 0 on the accumulator's own register. (Written as plain expressions, the accumulators of the rows
@@ -179,16 +186,25 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
         lane_off[k] = 16u * (uint32_t)max(min(c - (lm >> 4), nd - 1), 0);
         piece_on[k] = c < ppr;
     }
-    // Starts the transfer of source rows y0, y0 + 1 (rows behind the last repeat it) into the two slots of one half of the
-    // ring. Returns whether a row was stored by the lanes: one whose last piece would leave the batch buffer, which only the
-    // last row of the last sample can be.
-    auto issue = [&](int y0, int half) {
+    // Rows from y_lanes on are stored by the lanes, with bounds-checked loads: those whose last piece would leave the batch
+    // buffer, which only the last row of the last sample of the buffer can be (a row's pieces end less than 16 bytes behind
+    // the row); should even the row before it not fit, every row goes that way.
+    const uint32_t tail = col4 + 16u * (uint32_t)nd;
+    int y_lanes = y_last + 1;
+    if ((uint64_t)((uint32_t)y_last * row_stride) + tail > (uint64_t)lim)
+        y_lanes = (y_last > y_first && (uint64_t)((uint32_t)(y_last - 1) * row_stride) + tail <= (uint64_t)lim) ? y_last : y_first;
+
+    // Starts the transfer of the next two source rows (rows behind the last repeat it) into the two slots of one half of the
+    // ring; y_next / roff_next walk down the rows. Returns whether a row was stored by the lanes.
+    int y_next = y_first;
+    uint32_t roff_next = (uint32_t)y_first * row_stride + col4;
+    auto issue = [&](lds_u8 *half_base) {
         bool by_lanes = false;
 #pragma unroll
         for (int q = 0; q < TS_RPS; q++) {
-            const uint32_t roff = (uint32_t)min(y0 + q, y_last) * row_stride + col4;
-            lds_u8 *slot = bufb + (half * TS_RPS + q) * pitch;
-            if ((uint64_t)roff + 16ull * (uint64_t)nd <= (uint64_t)lim) {
+            const uint32_t roff = roff_next;
+            lds_u8 *slot = half_base + q * pitch;
+            if (y_next < y_lanes) {
                 const uint8_t *rowp = base4 + roff;
 #pragma unroll
                 for (int k = 0; k < TS_NCH; k++) {
@@ -197,7 +213,6 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
                     }
                 }
             } else {
-                // the row touches the last bytes of the batch buffer: bounds-checked byte loads, stored by the lanes
                 by_lanes = true;
                 for (int c = lane; c < ppr; c += RMX_WAVE) {
                     const uint32_t off = roff + 16u * (uint32_t)max(min(c - (lm >> 4), nd - 1), 0);
@@ -213,6 +228,10 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
                         dst4[i] = v;
                     }
                 }
+            }
+            if (y_next < y_last) {
+                y_next++;
+                roff_next += row_stride;
             }
         }
         return by_lanes;
@@ -258,11 +277,11 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
         rep_src = (uint32_t)(lm + ph + (is_l ? 0 : 3 * (ce - cs)) + c);
         rep_dst = (uint32_t)(lm + ph + (is_l ? -3 * (j + 1) : 3 * (ce - cs + 1 + j)) + c);
     }
-    auto replicate = [&](int half, int nr) {
+    auto replicate = [&](lds_u8 *half_base, int nr) {
         if (nrep_b > 0) {
             if (lane < nrep_b) {
                 for (int q = 0; q < nr; q++) {
-                    lds_u8 *slot = bufb + (half * TS_RPS + q) * pitch;
+                    lds_u8 *slot = half_base + q * pitch;
                     slot[rep_dst] = slot[rep_src];
                 }
             }
@@ -289,6 +308,7 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
     // filter loop reads a row's entry with one broadcast read. Rebuilt every 64 source rows. The first and the last row
     // of the window serve several taps of a row each (clamped tap indices) and take their own path below.
     lds_f32 *cftab = (lds_f32 *)(bufb + tab_off);
+    const lds_f32x4 *cv_next = (const lds_f32x4 *)cftab;  // the table entry of the next source row
     int ytab = y_first;
     auto build_table = [&]() {
         const int y = ytab + lane;
@@ -310,10 +330,15 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
         wave_sync();
     };
 
-    // An output row whose last tap row has been added: normalise, epilogue, store; its slot starts again at zero.
+    // An output row whose last tap row has been added: normalise, epilogue, store; its slot starts again at zero. orow walks
+    // down the output rows (planar: the row of channel 0; the other planes lie `plane` elements on).
+    T *orow = dimg + (size_t)r0 * a.dst_w * (LAYOUT == RMX_NCHW ? 1 : 3);
+    const size_t plane = (size_t)a.dst_h * a.dst_w;
+    const int orow_step = a.dst_w * (LAYOUT == RMX_NCHW ? 1 : 3);
+    int rsum_idx = 0;
     auto emit = [&](auto slot) {
         constexpr int M = decltype(slot)::value;
-        const float rsum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rq - r0));
+        const float rsum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rsum_idx));
 #pragma unroll
         for (int i = 0; i < TPX; i++) {
             const float inv = 1 / (rsum * colsum[i]);
@@ -324,10 +349,10 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
                 if constexpr (QUANT) t = round_u8(t);
                 if constexpr (NORM) t = __builtin_fmaf(t, sc[ch], bi[ch]);
                 // wave-uniform row pointer + the lane's column offset
-                if constexpr (LAYOUT == RMX_NCHW) store_elem<T, 0>(dimg + ((size_t)ch * a.dst_h + rq) * a.dst_w, xoff[i], elem_bits<T>(t));
-                else if (ch == 0) store_elem<T, 0>(dimg + (size_t)rq * a.dst_w * 3, xoff[i], elem_bits<T>(t));
-                else if (ch == 1) store_elem<T, (int)sizeof(T)>(dimg + (size_t)rq * a.dst_w * 3, xoff[i], elem_bits<T>(t));
-                else store_elem<T, 2 * (int)sizeof(T)>(dimg + (size_t)rq * a.dst_w * 3, xoff[i], elem_bits<T>(t));
+                if constexpr (LAYOUT == RMX_NCHW) store_elem<T, 0>(orow + ch * plane, xoff[i], elem_bits<T>(t));
+                else if (ch == 0) store_elem<T, 0>(orow, xoff[i], elem_bits<T>(t));
+                else if (ch == 1) store_elem<T, (int)sizeof(T)>(orow, xoff[i], elem_bits<T>(t));
+                else store_elem<T, 2 * (int)sizeof(T)>(orow, xoff[i], elem_bits<T>(t));
             }
         }
     };
@@ -336,16 +361,15 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
     // unrolled horizontal pass (4, 6 or 8 >= kx): taps beyond kx carry coefficient 0 (fma(p, 0, a) == a for the finite p an
     // unpacked byte always is), so no bound test is needed inside. A column's 3 NT bytes start at byte tap_ph of dword
     // tap_w: NE + 1 dwords are read and realigned into NE.
-    auto process_row = [&](auto nt, int slot, int yy) {
+    auto process_row = [&](auto nt, const lds_u8 *srow, int yy) {
         constexpr int NT = decltype(nt)::value;
         constexpr int NE = (3 * NT + 3) / 4;
-        const lds_u8 *srow = bufb + slot * pitch;
         // A row inside the window is one tap of every output row that reads it: one pass, coefficients from the table. The
         // first / last row of the window is also read by every tap index that leaves the window: one pass per such tap, in
         // tap order, coefficients computed here by lane p for pass p (rare: twice per image column of strips at most).
-        const lds_f32x4 *cvp = (const lds_f32x4 *)(cftab + TS_SLOTS * (yy - ytab));
+        const lds_f32x4 *cvp = cv_next++;
         int npass = 1;
-        if (yy == ylo || yy == yhi) {
+        if ((uint32_t)(yy - ylo - 1) >= (uint32_t)(yhi - ylo - 1)) {  // yy == ylo or yy == yhi (rows lie inside the window)
             float ec[TS_SLOTS];
             npass = 0;
 #pragma unroll
@@ -400,16 +424,18 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
             cv4 = cvp[p];
         }
         // ---- rows whose last tap was this source row
-        while (qlast <= yy && rq < r1) {
-            switch ((rq - r0) & (TS_SLOTS - 1)) {
+        while (qlast <= yy) {
+            switch (rsum_idx & (TS_SLOTS - 1)) {
                 case 0: emit(std::integral_constant<int, 0>{}); break;
                 case 1: emit(std::integral_constant<int, 1>{}); break;
                 case 2: emit(std::integral_constant<int, 2>{}); break;
                 default: emit(std::integral_constant<int, 3>{}); break;
             }
             rq++;
+            rsum_idx++;
+            orow += orow_step;
             emitted++;
-            qlast = last_tap_row(min(rq, r1 - 1));
+            qlast = rq < r1 ? last_tap_row(rq) : 0x7fffffff;  // (behind the last row: no source row completes anything)
         }
     };
 
@@ -420,13 +446,14 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
     // started right behind the wait (the slots they fill were read for the last time in the step before).
     constexpr int NS = 3 * TPX;  // store instructions per output row
     auto run = [&](auto nt) {
-        bool by_lanes = issue(y_first, 0);
+        lds_u8 *half_cur = bufb, *half_nxt = bufb + TS_RPS * pitch;
+        bool by_lanes = issue(half_cur);
         build_table();  // (under the round trip of the first loads)
-        int half = 0;
-        for (int y = y_first; y <= y_last; y += TS_RPS, half ^= 1) {
+        for (int y = y_first; y <= y_last; y += TS_RPS) {
             const int nr = min(TS_RPS, y_last - y + 1);
             if (y + nr - ytab > RMX_WAVE) {
                 ytab = y;
+                cv_next = (const lds_f32x4 *)cftab;
                 build_table();
             }
             if (by_lanes || emitted > 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the lanes' own loads, or many rows)
@@ -435,10 +462,13 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
             else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NS) : "memory");
             wave_sync();
             emitted = 0;
-            by_lanes = (y + TS_RPS <= y_last) ? issue(y + TS_RPS, half ^ 1) : false;
-            replicate(half, nr);
-            for (int q = 0; q < nr; q++) process_row(nt, half * TS_RPS + q, y + q);
+            by_lanes = (y + TS_RPS <= y_last) ? issue(half_nxt) : false;
+            replicate(half_cur, nr);
+            for (int q = 0; q < nr; q++) process_row(nt, half_cur + q * pitch, y + q);
             wave_sync();  // the slots are reused two steps on
+            lds_u8 *t = half_cur;
+            half_cur = half_nxt;
+            half_nxt = t;
         }
     };
     if (kx <= 4) run(std::integral_constant<int, 4>{});
