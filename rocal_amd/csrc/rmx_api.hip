@@ -81,7 +81,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_per_cu = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -309,6 +309,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
         ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
         ctx->tri_tpx = tune_env("RMX_TUNE_TRI_TPX", ctx->tri_tpx, 1, 2);     // output columns per lane of the downscaling kernel
+        ctx->tri_per_cu = tune_env("RMX_TUNE_TRI_PER_CU", ctx->tri_per_cu, 0, 32);  // wavefronts per CU the strip planner counts on (0: by registers and LDS)
     }
     *out = ctx;
     return RMX_OK;
@@ -821,25 +822,47 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         // Streaming form of the downscaling variant (source rows straight into LDS as raw bytes): every source row must start
         // at the same byte phase (row stride a multiple of 4), and four LDS rows of the widest tile plus the table of vertical
         // coefficients must leave room for ten wavefronts per CU at least.
-        bool tdma = down && op->ctx->dma && op->ctx->tri_tpx == 2 && ky <= 64;
+        bool tdma = down && op->ctx->dma && op->ctx->tri_tpx == 2 && ky <= 16;
         if (tdma) {
             if (op->layout.empty()) tdma = (op->src.w * 3u) % 4u == 0;
             else
                 for (int i = 0; i < op->n && tdma; i++) tdma = op->layout[i].row_stride % 4u == 0;
         }
         if (tdma) {
+            // The widest LDS row over all tiles, by the kernel's own fp32 law for a tile's first and last tap (its byte phase
+            // inside a dword is taken at its worst, 3).
             size_t pitch_max = 64;
-            for (int i = 0; i < op->n; i++) {
+            for (int i = 0; i < op->n && tdma; i++) {
                 const RmxSample &s = t[i];
                 if (s.dst_w <= 0 || s.dst_h <= 0) continue;
-                const int kxi = (int)std::ceil(2.0f * std::max(s.rx, 1.0f));
-                const int cols = std::min<int>((int)op->src.w, (int)std::ceil(128 * (double)std::max(s.rx, 1.0f))) + kxi + 4;
-                // margin (two pieces at most) + phase + data + right replicas + the reach of an 8-tap read, in whole pieces
-                pitch_max = std::max(pitch_max, (size_t)32 + (size_t)((3 + 3 * (cols + 8) + 8 + 15) / 16 * 16));
+                const float radius = s.rx > 1.0f ? s.rx : 1.0f;
+                const float offset = (s.rx - 1) * 0.5f - radius;
+                const int kxi = (int)std::ceil(radius * 2);
+                const int xlo = s.src_x, xhi = s.src_x + s.src_w - 1;
+                auto loc_of = [&](int d) {
+                    float raw = (float)d * s.rx;
+                    raw = raw + offset;
+                    raw = raw + (float)xlo;
+                    return (int)std::ceil(raw);
+                };
+                for (int xt = 0; xt < (int)s.dst_w; xt += 128) {
+                    const int tw = std::min(128, (int)s.dst_w - xt);
+                    const int lf = loc_of(s.pc_x + xt), ll = loc_of(s.pc_x + xt + tw - 1);
+                    const int cs = std::max(std::min(lf, xhi), xlo), ce = std::max(std::min(ll + kxi - 1, xhi), xlo);
+                    const int nrep_l = std::max(cs - lf, 0), nrep_r = std::max(ll + kxi - 1 - ce, 0);
+                    const int nd = (3 + 3 * (ce - cs + 1) + 15) >> 4;
+                    const int lm = ((3 * nrep_l + 15) >> 4) << 4;
+                    const int body = std::max(3 + 3 * (ll + 8 - cs) + 8, 16 * nd);
+                    const int pitch = lm + (((body + 15) >> 4) << 4);
+                    if (pitch > 128 * 16 || 3 * (nrep_l + nrep_r) > 64) tdma = false;
+                    pitch_max = std::max(pitch_max, (size_t)pitch);
+                }
             }
-            const size_t lds = 4 * pitch_max + (64 + 64) * 4 * 4;  // + vertical coefficients: 64 source rows and 64 passes x 4 slots
-            if (pitch_max > 128 * 16 || lds > 16 * 1024) tdma = false;
-            else {
+            // ring of four source rows (six were measured: 18 instead of 20 wavefronts per CU, a fifth slower) + vertical
+            // coefficients: 64 source rows and 16 passes x 4 slots
+            const size_t lds = 4 * pitch_max + (64 + 16) * 4 * 4;
+            if (lds > 16 * 1024) tdma = false;
+            if (tdma) {
                 op->fn = rmx::select_resize_tri_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
                 op->lds_per_wave = (int)lds;
             }
@@ -872,7 +895,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             // image is a short one, so an R that leaves a remainder of at most R/2 rows is preferred.
             if (op->ctx->tri_rows == 0) {
                 // (wavefronts per CU: 16 by the registers of the kernel that stages through registers, 20 by those of the streaming one)
-                const int per_cu = std::max(1, std::min(tdma ? 20 : 16, (160 * 1024) / op->lds_per_wave));
+                const int per_cu = op->ctx->tri_per_cu > 0 ? op->ctx->tri_per_cu : std::max(1, std::min(tdma ? 20 : 16, (160 * 1024) / op->lds_per_wave));
                 const long slots = (long)op->ctx->num_cus * per_cu;
                 double best_cost = 0.0;
                 for (int r = 4; r <= 64; r++) {

@@ -19,11 +19,10 @@
 
 #include <type_traits>
 
-// " nt": streaming stores (the output is written once and read by another kernel much later)
-#ifdef RMX_TDMA_NT_ON
-#define RMX_TDMA_NT " nt"
-#else
-#define RMX_TDMA_NT ""
+// Wavefronts per SIMD the register budget is set for (a workgroup of 256 threads is one wavefront per SIMD): 96 registers,
+// met without spills. Measured on 1080p -> 640 x 360: a budget for six gains nothing, for four loses a fifth.
+#ifndef RMX_TDMA_WAVES
+#define RMX_TDMA_WAVES 5
 #endif
 
 namespace rmx {
@@ -37,6 +36,8 @@ typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
 constexpr int TS_SLOTS = 4;  // output rows in flight
 constexpr int TS_RPS = 2;    // source rows per step; the ring holds two steps
 constexpr int TS_NCH = 2;    // load instructions per row at most (64 pieces of 16 bytes each)
+constexpr int TS_TAB = 64;   // source rows of the table of vertical coefficients
+constexpr int TS_EDGE = 16;  // passes of an edge row at most (= vertical taps the host admits)
 
 template <int B>
 RMX_DEV float ubyte_at(uint32_t v) {
@@ -67,9 +68,9 @@ RMX_DEV void tri_taps(const uint32_t (&e)[NE], const float (&c)[8], float &a0, f
 // instructions issued behind them, so their number must not be left to the compiler): `bits` to row + voff + OFF bytes.
 template <typename T, int OFF>
 RMX_DEV void store_elem(const T *row, uint32_t voff, uint32_t bits) {
-    if constexpr (sizeof(T) == 4) asm volatile("global_store_dword %0, %1, %2 offset:%3" RMX_TDMA_NT ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
-    else if constexpr (sizeof(T) == 2) asm volatile("global_store_short %0, %1, %2 offset:%3" RMX_TDMA_NT ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
-    else asm volatile("global_store_byte %0, %1, %2 offset:%3" RMX_TDMA_NT ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
+    if constexpr (sizeof(T) == 4) asm volatile("global_store_dword %0, %1, %2 offset:%3" ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
+    else if constexpr (sizeof(T) == 2) asm volatile("global_store_short %0, %1, %2 offset:%3" ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
+    else asm volatile("global_store_byte %0, %1, %2 offset:%3" ::"v"(voff), "v"(bits), "s"(row), "n"(OFF) : "memory");
 }
 
 // acc += h * c and acc = 0 on the accumulator's own register. (Written as plain expressions, the accumulators of the rows
@@ -86,7 +87,7 @@ RMX_DEV uint32_t elem_bits(float v) {
 }
 
 template <typename T, int LAYOUT, bool NORM, bool QUANT>
-__global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) {
+__global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel(RmxKArgs a) {
     constexpr int TPX = 2;               // columns per lane: lane and lane + 64
     constexpr int TTW = RMX_WAVE * TPX;  // output columns per wave tile
     const int lane = threadIdx.x & (RMX_WAVE - 1);
@@ -160,7 +161,7 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
     const int body = max(ph + 3 * (l_last + 8 - cs) + 8, 16 * nd);
     const int pitch = lm + (((body + 15) >> 4) << 4);
     const int ppr = pitch >> 4;  // pieces per row
-    const int tab_off = a.lds_bytes - TS_SLOTS * (RMX_WAVE + RMX_WAVE) * 4;  // coefficient table: 64 rows, and up to 64 passes of an edge row
+    const int tab_off = a.lds_bytes - TS_SLOTS * (TS_TAB + TS_EDGE) * 4;  // the tables of vertical coefficients
     // (the host sizes the slice for four rows of the widest tile; a tile that does not fit is left alone)
     if (2 * TS_RPS * pitch > tab_off || ppr > TS_NCH * RMX_WAVE || 3 * (nrep_l + nrep_r) > RMX_WAVE) return;
 
@@ -386,8 +387,8 @@ __global__ void __launch_bounds__(256, 4) rmx_resize_tri_dma_kernel(RmxKArgs a) 
                     if (j <= jhi) ec[m] = c;
                 }
             }
-            lds_f32 *etab = cftab + TS_SLOTS * RMX_WAVE;
-            *(lds_f32x4 *)(etab + TS_SLOTS * lane) = f32x4{ec[0], ec[1], ec[2], ec[3]};  // (the host admits 64 vertical taps at most)
+            lds_f32 *etab = cftab + TS_SLOTS * TS_TAB;
+            if (lane < TS_EDGE) *(lds_f32x4 *)(etab + TS_SLOTS * lane) = f32x4{ec[0], ec[1], ec[2], ec[3]};
             wave_sync();
             cvp = (const lds_f32x4 *)etab;
             npass = max(npass, 1);

@@ -38,3 +38,34 @@ def test_held_back_stores_cover_the_wait_count():
         assert stores_behind >= n, "%s: waits with vmcnt(%d) but only %d stores follow the loads" % (m.group(1), n, stores_behind)
         checked += 1
     assert checked >= 20  # every instance of the kernel
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="needs hipcc")
+def test_streaming_triangular_kernel_counts_its_stores():
+    """The streaming triangular kernel waits for its loads into LDS with s_waitcnt vmcnt(6 x output rows stored since): every
+    output row must be exactly six store instructions (written as inline assembly, one per element and lane), no store may
+    come from the compiler, nothing may spill to scratch memory (scratch traffic counts as vector memory too), and the only
+    waits with a number are the two the source names."""
+    from rocal_amd import build as rbuild
+    src = os.path.join(ROOT, "rocal_amd", "csrc", "rmx_kernels_tri_dma.hip")
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "tdma.s")
+        subprocess.run([HIPCC] + list(rbuild.FLAGS) + ["-I" + os.path.join(ROOT, "rocal_amd", "csrc"), "-I" + os.path.join(ROOT, "include"),
+                        "--cuda-device-only", "-S", src, "-o", out], check=True, capture_output=True, timeout=600)
+        text = open(out).read()
+    funcs = re.split(r"\n(?=_ZN3rmx25rmx_resize_tri_dma_kernel[^\n]*:\s)", text)
+    checked = 0
+    for f in funcs:
+        m = re.match(r"(_ZN3rmx25rmx_resize_tri_dma_kernel\S*):", f)
+        if not m:
+            continue
+        body = f.split("s_endpgm")[0]
+        stores = re.findall(r"^\s*(global_store_\w+|flat_store_\w+|buffer_store_\w+|scratch_\w+)", body, re.M)
+        # three tap-count variants of the row loop x four accumulator slots x (two columns x three channels)
+        assert len(stores) == 3 * 4 * 6, "%s: %d store instructions" % (m.group(1), len(stores))
+        assert len(set(stores)) == 1 and stores[0].startswith("global_store_"), "%s: %s" % (m.group(1), sorted(set(stores)))
+        waits = sorted(set(int(x) for x in re.findall(r"s_waitcnt vmcnt\((\d+)\)", body)))
+        assert set(waits) <= {0, 6, 12}, "%s: waits %s" % (m.group(1), waits)
+        assert "global_load_lds_dwordx4" in body
+        checked += 1
+    assert checked == 18  # every instance of the kernel

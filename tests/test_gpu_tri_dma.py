@@ -1,0 +1,148 @@
+"""The streaming triangular kernel (source rows straight into LDS as packed bytes) against the oracle, bit for bit, on what is
+specific to it: windows that start at every byte phase of a dword, edge replicas on both sides, every output format, strips
+whose source rows outnumber the table of vertical coefficients, many vertical taps, mirror, packed (ragged) sources whose
+rows start at multiples of 4 bytes, and the kernel that stages through registers on the same batches."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from rocal_amd import ops, workloads as wl
+
+pytestmark = pytest.mark.gpu
+
+
+def _gpu(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _bits(a):
+    return np.ascontiguousarray(a).view(np.uint8)
+
+
+def _scale_bias(n):
+    return orc.cmn_scale_bias(wl.MEAN, wl.STD, n)
+
+
+def _check_windows(got, exp, dw, dh, layout, fill, what):
+    n = got.shape[0]
+    want = np.full_like(exp, fill)
+    for i in range(n):
+        if layout == ops.NCHW:
+            want[i, :, :dh[i], :dw[i]] = exp[i, :, :dh[i], :dw[i]]
+        else:
+            want[i, :dh[i], :dw[i]] = exp[i, :dh[i], :dw[i]]
+    assert np.array_equal(_bits(got), _bits(want)), "%s: %d values differ" % (what, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("layout,dtype", [(ops.NCHW, ops.FP16), (ops.NCHW, ops.FP32), (ops.NCHW, ops.UINT8), (ops.NHWC, ops.FP16),
+                                          (ops.NHWC, ops.FP32), (ops.NHWC, ops.UINT8)])
+def test_formats_phases_and_edges(ctx, ctx_staged, layout, dtype):
+    """Eight samples over a 256-pixel-wide source (768-byte rows): the whole image (replicas left and right), windows whose
+    first column is 1, 2, 3 ... pixels in (every byte phase), windows that end at the last column / row, a narrow and a
+    short one; destinations narrower than the tensor (the padding keeps the fill value); both kernels."""
+    rng = np.random.default_rng(900 + 7 * layout + dtype)
+    n, H, W = 8, 200, 256
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.array([[0, 0, W, H], [1, 0, 200, 150], [2, 7, 222, 180], [3, 1, 253, 199], [5, 9, 251, 191], [40, 30, 60, 90], [100, 150, 156, 50],
+                    [0, 0, W, H]], np.uint32)
+    dw = np.array([100, 77, 129, 64, 130, 31, 57, 200], np.uint32)
+    dh = np.array([61, 50, 47, 30, 61, 40, 11, 61], np.uint32)
+    OH, OW = 61, 200
+    mirror = np.array([0, 1, 0, 1, 1, 0, 1, 0], np.uint32)
+    scale, bias = _scale_bias(n)
+    norm = dtype != ops.UINT8
+    exp = orc.resize(img, roi, dw, dh, OH, OW, interp=orc.TRIANGULAR, mirror=mirror, scale=scale if norm else None, bias=bias if norm else None,
+                     layout=layout, dtype=dtype)
+    for c, name in ((ctx, "rmx_resize_tri_dma_kernel"), (ctx_staged, "rmx_resize_tri_down_kernel")):
+        op = ops.Resize(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, layout, dtype), ops.TRIANGULAR)
+        if norm:
+            op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        else:
+            op.update(roi, dw, dh, mirror)
+        assert op.kernel_name == name, op.plan
+        out = op.alloc_output(fill=7)
+        op.launch(_gpu(img), out)
+        c.sync()
+        _check_windows(out.cpu().numpy(), exp, dw, dh, layout, 7, name)
+
+
+@pytest.mark.parametrize("ry,rows", [(7.4, 0), (5.1, 20), (2.0, 64), (1.0, 7)])
+def test_many_vertical_taps_and_long_strips(ctx, ry, rows):
+    """Vertical ratios up to 7.4 (15 taps: rows at the window's ends are read by up to 8 clamped taps each), strips whose
+    source rows outnumber the 64 rows of the coefficient table (it is rebuilt on the way), strips of 64 output rows, ratio 1."""
+    from conftest import _ctx_with_env
+    c = _ctx_with_env(RMX_TUNE_TRI_ROWS=rows) if rows else ctx
+    rng = np.random.default_rng(int(ry * 10) + rows)
+    n, dh0, dw0 = 3, 70, 150
+    H, W = int(round(dh0 * ry)) + 6, 340
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    roi = np.array([[0, 0, W, H], [4, 3, 300, H - 6], [17, 0, 323, H - 1]], np.uint32)
+    dw = np.array([dw0, 131, 150], np.uint32)
+    dh = np.array([dh0, dh0 - 3, dh0], np.uint32)
+    mirror = np.array([1, 0, 1], np.uint32)
+    scale, bias = _scale_bias(n)
+    exp = orc.resize(img, roi, dw, dh, dh0, dw0, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+    op = ops.Resize(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, dh0, dw0, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert op.kernel_name == "rmx_resize_tri_dma_kernel", op.plan
+    out = op.alloc_output(fill=3)
+    op.launch(_gpu(img), out)
+    c.sync()
+    _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 3, "ry=%g rows=%d (%s)" % (ry, rows, op.plan))
+    if rows:
+        c.close()
+
+
+def test_more_than_sixteen_vertical_taps_take_the_other_kernel(ctx):
+    rng = np.random.default_rng(3)
+    n, H, W = 1, 400, 64
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    roi = np.array([[0, 0, W, H]], np.uint32)
+    dw, dh = np.array([32], np.uint32), np.array([40], np.uint32)  # ratio 10: 20 taps
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, 40, 32, ops.NHWC, ops.UINT8), ops.TRIANGULAR)
+    op.update(roi, dw, dh)
+    assert op.kernel_name == "rmx_resize_tri_down_kernel"
+    out = op.alloc_output()
+    op.launch(_gpu(img), out)
+    ctx.sync()
+    exp = orc.resize(img, roi, dw, dh, 40, 32, interp=orc.TRIANGULAR, layout=ops.NHWC, dtype=ops.UINT8)
+    assert np.array_equal(out.cpu().numpy(), exp)
+
+
+def test_packed_source_with_rows_at_multiples_of_four(ctx):
+    """Packed images (a byte offset and a row stride per image, strides multiples of 4) in an exact-size buffer: the last rows
+    of the last image end on the last bytes of the buffer and are staged by the lanes with bounds-checked loads."""
+    rng = np.random.default_rng(8)
+    n = 4
+    widths = np.array([300, 257, 128, 400], np.uint32)
+    heights = np.array([120, 90, 77, 150], np.uint32)
+    strides = (3 * widths + 3) // 4 * 4
+    offsets, parts, pos = [], [], 0
+    padded = np.zeros((n, 150, 400, 3), np.uint8)
+    for i in range(n):
+        h, w, st = int(heights[i]), int(widths[i]), int(strides[i])
+        im = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+        padded[i, :h, :w] = im
+        rows = np.zeros((h, st), np.uint8)
+        rows[:, :3 * w] = im.reshape(h, 3 * w)
+        offsets.append(pos)
+        parts.append(rows.reshape(-1))
+        pos += rows.size
+    packed = np.concatenate(parts)
+    packed = packed[:offsets[-1] + (int(heights[-1]) - 1) * int(strides[-1]) + 3 * int(widths[-1])]  # nothing behind the last pixel
+    roi = np.array([[0, 0, widths[i], heights[i]] for i in range(n)], np.uint32)
+    roi[1] = (3, 2, 250, 85)
+    dw = np.array([140, 100, 64, 180], np.uint32)
+    dh = np.array([50, 40, 31, 60], np.uint32)
+    mirror = np.array([0, 1, 1, 0], np.uint32)
+    scale, bias = _scale_bias(n)
+    exp = orc.resize(padded, roi, dw, dh, 60, 180, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+    op = ops.Resize(ctx, ops.desc(n, 150, 400, ops.NHWC, ops.UINT8), ops.desc(n, 60, 180, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+    op.set_ragged_source(np.array(offsets, np.uint64), widths, heights, packed.size, row_strides=strides)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert op.kernel_name == "rmx_resize_tri_dma_kernel", op.plan
+    out = op.alloc_output(fill=1)
+    op.launch(_gpu(packed), out)
+    ctx.sync()
+    _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 1, "packed source")
