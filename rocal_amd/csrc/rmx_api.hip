@@ -1419,7 +1419,7 @@ static int create_warp(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const
     int rc = make_op(ctx, kind, src, dst, roi_type, out);
     if (rc) return rc;
     (*out)->interp = interpolation;
-    (*out)->fn = rmx::select_warp_kernel(interpolation, dst->dtype, dst->layout, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_warp_kernel(interpolation, dst->dtype, dst->layout, false, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -1430,6 +1430,15 @@ static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, con
     uint64_t bytes = 0;
     int max_dw = 1, max_dh = 1;
     double worst_box = 0;
+    // The form that loads the source box straight into LDS as packed bytes needs every source row to start at the same byte
+    // phase (row stride a multiple of 4).
+    bool raw = op->ctx->dma != 0;
+    if (raw) {
+        if (op->layout.empty()) raw = (op->src.w * 3u) % 4u == 0;
+        else
+            for (int i = 0; i < op->n && raw; i++) raw = op->layout[i].row_stride % 4u == 0;
+    }
+    op->fn = rmx::select_warp_kernel(op->interp, op->dst.dtype, op->dst.layout, raw, &op->kernel_name);
     for (int i = 0; i < op->n; i++) {
         RmxSample &s = t[i];
         int rc = read_roi(op, roi, i, &s.src_x, &s.src_y, &s.src_w, &s.src_h);
@@ -1460,14 +1469,21 @@ static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, con
         if (std::isfinite(bw) && std::isfinite(bh)) {
             bw = std::min(bw, (double)s.src_w + 1);
             bh = std::min(bh, (double)s.src_h + 1);
-            // (boxes of up to 60 dwords per row are staged at a pitch of 60, see the kernel)
-            const double pitch = std::ceil(bw / 4) * 4 + 4;
-            worst_box = std::max(worst_box, (pitch <= 60.0 ? 60.0 : pitch) * bh);
+            if (raw) {
+                // (packed bytes: rows of whole 16-byte pieces from the dword that holds the box's first pixel; boxes of up to
+                // kWarpRawPieces pieces per row are staged at that pitch; in dwords, like the other form)
+                const double pieces = std::ceil((3.0 + 3.0 * (bw + 1.0)) / 16.0);
+                worst_box = std::max(worst_box, (pieces <= rmx::kWarpRawPieces ? (double)rmx::kWarpRawPieces : pieces) * 4.0 * bh);
+            } else {
+                // (boxes of up to 60 dwords per row are staged at a pitch of 60, see the kernel)
+                const double pitch = std::ceil(bw / 4) * 4 + 4;
+                worst_box = std::max(worst_box, (pitch <= 60.0 ? 60.0 : pitch) * bh);
+            }
         }
     }
     op->algo_bytes = bytes;
     const int cap = 16 * 1024;  // per wave (16 loads per lane); bigger boxes fall back to global gathers inside the kernel
-    int need = (int)std::min<double>(worst_box * 4, (double)cap);
+    int need = (int)std::min<double>(worst_box * 4 + (raw ? 16 : 0), (double)cap);
     op->lds_per_wave = std::max(256, (need + 15) / 16 * 16);
     op->waves_per_block = std::max(1, std::min(op->ctx->warp_wpb, op->ctx->max_lds_per_block / op->lds_per_wave));
     const int passes = op->ctx->warp_passes;

@@ -10,6 +10,12 @@
 // taps of pixels that fall outside the ROI are read from wherever their (meaningless) address points inside
 // the slice and the result is replaced by 0. When the box does not fit the slice (strong minification) the
 // wavefront gathers from global memory instead.
+//
+// RAW (every source row starts at the same byte phase: row strides multiples of 4): the box travels from global memory
+// straight into LDS as packed bytes (global_load_lds_dwordx4, 16 bytes per lane: no vector register, no unpacking, no LDS
+// store; piece i of the box, rows one after the other, is loaded by lane i & 63 of load instruction i >> 6), three bytes
+// per pixel instead of four, and a tap pair (two packed pixels, 6 bytes at any byte phase) is read as three aligned dwords
+// and realigned with two v_alignbyte. Values and operations from there on are the same.
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
@@ -26,6 +32,7 @@ typedef __attribute__((address_space(3))) uint32_t lds_u32;  // explicit LDS poi
 
 constexpr int WTW = 32, WTH = 16;  // destination tile: 4 lanes x 8 px wide, 16 rows per pass
 constexpr int WFP = 60;            // fixed LDS pitch (dwords) of boxes that fit it
+constexpr int WRP = kWarpRawPieces;  // RAW: fixed LDS pitch in 16-byte pieces (an odd number spreads the rows over the LDS banks)
 
 RMX_DEV uint32_t load_px_global(const uint8_t *p) {
     return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16);
@@ -38,7 +45,7 @@ RMX_DEV int floor_i32(float x) {
     return r;
 }
 
-template <typename T, int LAYOUT, bool NEAREST>
+template <typename T, int LAYOUT, bool NEAREST, bool RAW>
 __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     const int wib = threadIdx.x / RMX_WAVE;
@@ -104,10 +111,17 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     // Boxes of at most WFP - 1 columns (every tile of a map that does not minify) are staged at ONE pitch, known to the
     // compiler: the address of a tap is two instructions (a 24-bit multiply-add and a shift-add) and the row below is an
     // offset inside the read instruction. 15 items: an odd number of 16-byte items spreads the rows over the LDS banks.
-    const bool fixed = items * 4 <= WFP;
-    const int pitch = fixed ? WFP : items * 4;
-    const int total = (bh + 1) * items;
-    const bool use_lds = !empty && total <= 16 * RMX_WAVE && (size_t)(bh + 1) * pitch * 4 <= (size_t)a.lds_bytes;
+    // RAW: a row is ppr 16-byte pieces from the dword that holds pixel bx0 (byte phase ph inside it)
+    const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
+    const uint32_t colb = (uint32_t)max(bx0, 0) * 3u + skew;
+    const int ph = (int)(colb & 3u);
+    const int ppr_box = (ph + 3 * (max(bw, 0) + 1) + 15) >> 4;
+    const bool fixed = RAW ? ppr_box <= WRP : items * 4 <= WFP;
+    const int ppr = fixed ? WRP : ppr_box;
+    const int pitch = RAW ? ppr * 4 : (fixed ? WFP : items * 4);  // dwords
+    const int total = (bh + 1) * (RAW ? ppr : items);            // 16-byte pieces (RAW) or four-pixel items of the box
+    // (RAW: the three dwords read for the last tap of the last row may reach 8 bytes behind the box)
+    const bool use_lds = !empty && total <= 16 * RMX_WAVE && (size_t)(bh + 1) * pitch * 4 + (RAW ? 16 : 0) <= (size_t)a.lds_bytes;
 
     const int lr = lane >> 2, g = lane & 3;
     const int x0 = X0 + g * PX;
@@ -174,10 +188,60 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
         return;
     }
 
+    if constexpr (RAW) {
+        // ---- the box straight into LDS: piece idx = (row, piece of the row) in row order lands at byte 16 idx of the slice
+        const uint8_t *base4 = simg - skew;
+        const uint32_t col4 = colb & ~3u;
+        lds_u8 *ldsb = (lds_u8 *)(lds_ptr_t)rmx_lds_warp + (uint32_t)to_sgpr((int)((uint32_t)wib * (uint32_t)a.lds_bytes));
+        // every piece of the box lies inside the batch buffer (the last rows of the last sample may not)
+        const bool safe = simg + ((size_t)min(by1 + 1, yhi) * row_stride + (size_t)bx0 * 3 + 16 * (size_t)ppr) <= buf_end;
+        const float inv_ppr = 1.0f / (float)ppr;
+        if (safe) {
+            for (int j0 = 0; j0 < total; j0 += RMX_WAVE) {
+                const int idx = j0 + lane;
+                // idx / ppr: (idx + 0.5) / ppr is at least 0.5/ppr away from an integer, so the truncation is exact
+                const int r = fixed ? idx / WRP : (int)(((float)idx + 0.5f) * inv_ppr);
+                const int c = idx - __mul24(r, ppr);
+                const uint32_t off = (uint32_t)min(by0 + r, yhi) * row_stride + col4 + 16u * (uint32_t)c;
+                if (idx < total) __builtin_amdgcn_global_load_lds((glb_ptr_t)(base4 + off), (lds_ptr_t)(ldsb + 16 * j0), 16, 0, 0);
+            }
+            // the compiler does not order LDS reads behind loads into LDS: await them explicitly
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        } else {
+            // the box touches the last bytes of the batch buffer: bounds-checked byte loads, stored by the lanes
+            const uint64_t left = (uint64_t)(buf_end - base4);
+            const uint32_t lim = left > 0xffffffffull ? 0xffffffffu : (uint32_t)left;
+            for (int idx = lane; idx < total; idx += RMX_WAVE) {
+                const int r = idx / ppr, c = idx - r * ppr;
+                const uint32_t off = (uint32_t)min(by0 + r, yhi) * row_stride + col4 + 16u * (uint32_t)c;
+                lds_u32 *dst4 = (lds_u32 *)(ldsb + 16 * idx);
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    uint32_t v = 0;
+#pragma unroll
+                    for (int b = 0; b < 4; b++) {
+                        const uint32_t ob = off + 4u * i + b;
+                        v |= (ob < lim ? (uint32_t)base4[ob] : 0u) << (8 * b);
+                    }
+                    dst4[i] = v;
+                }
+            }
+        }
+        wave_sync();
+        // the column behind the box repeats its last column where that is the ROI's last column (only then is it read)
+        if (bx1 == xhi) {
+            for (int r = lane; r <= bh; r += RMX_WAVE) {
+                lds_u8 *px = ldsb + r * (pitch * 4) + ph + 3 * (bw - 1);
+                px[3] = px[0];
+                px[4] = px[1];
+                px[5] = px[2];
+            }
+            wave_sync();
+        }
+    } else
     // ---- stage the box: (row, 4-pixel item) pairs form one flat index space dealt to the lanes; rows beyond
     // the box repeat the ROI's last row (the clamp does it); all loads go out before the first is consumed
     {
-        const uint32_t skew = (uint32_t)((uintptr_t)simg & 3u);
         const uint8_t *base4 = simg - skew;
         const uint32_t col0 = (uint32_t)bx0 * 3u + skew;
         const float inv_items = 1.0f / (float)items;
@@ -233,7 +297,9 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
 
     // ---- gather and blend, branch-free
     // LDS byte address of source pixel (0, 0): the slice's base minus the box origin (may lie below the slice)
-    const int lbase0 = (int)(uint32_t)(uintptr_t)(lds_u32 *)lds - 4 * (by0 * pitch + bx0);
+    // (RAW: byte address of the first byte of source pixel (0, 0), three bytes per pixel)
+    const int lbase0 = RAW ? (int)(uint32_t)(uintptr_t)(lds_u32 *)lds + ph - (4 * by0 * pitch + 3 * bx0)
+                           : (int)(uint32_t)(uintptr_t)(lds_u32 *)lds - 4 * (by0 * pitch + bx0);
     // pixels whose floor lies inside the ROI: xlo <= s < xhi + 1 (and not NaN), tested on the clamped coordinate
     // (upper bounds: the float just below xhi + 1, a positive number, so one step down in its bit pattern)
     const float cx_lo = (float)xlo, cx_hi = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, (float)(xhi + 1)) - 1u);
@@ -271,7 +337,16 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
                 }
                 const int ix0 = floor_i32(sx), iy0 = floor_i32(sy);
                 const lds_u32 *t0p, *t1p;
-                if constexpr (FIXED) {
+                uint32_t tph = 0;  // RAW: byte phase of the tap pair inside its first dword
+                if constexpr (RAW) {
+                    uint32_t rowb, adr;
+                    if constexpr (FIXED) asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(rowb) : "v"(iy0), "s"(WRP * 16), "v"(lbase_v));
+                    else rowb = (uint32_t)(__mul24(iy0, pitch * 4) + lbase0);
+                    asm("v_mad_i32_i24 %0, %1, 3, %2" : "=v"(adr) : "v"(ix0), "v"(rowb));
+                    tph = adr & 3u;
+                    t0p = (const lds_u32 *)(adr & ~3u);
+                    t1p = FIXED ? t0p + WRP * 4 : t0p + pitch;
+                } else if constexpr (FIXED) {
                     // byte address: a 24-bit multiply-add of the row onto the (scalar) slice base, a shift-add of the column
                     // (spelled out: left to itself the compiler makes a shift, a multiply and a three-way add of it)
                     uint32_t rowb, adr;
@@ -285,11 +360,24 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
                 }
                 float o0, o1, o2;
                 if constexpr (NEAREST) {
-                    const uint32_t tl = t0p[0];
+                    uint32_t tl = t0p[0];
+                    if constexpr (RAW) tl = __builtin_amdgcn_alignbyte(t0p[1], tl, tph);
                     o0 = ubyte0(tl); o1 = ubyte1(tl); o2 = ubyte2(tl);
                 } else {
-                    const uint32_t tl = t0p[0], tr = t0p[1];
-                    const uint32_t bl = t1p[0], br = t1p[1];
+                    uint32_t tl = t0p[0], tr = t0p[1];
+                    uint32_t bl = t1p[0], br = t1p[1];
+                    if constexpr (RAW) {
+                        // six bytes from byte tph on: TL in bytes 0..2 of the first realigned dword, TR from its byte 3 on
+                        const uint32_t t2 = t0p[2], b2 = t1p[2];
+                        const uint32_t tlo = __builtin_amdgcn_alignbyte(tr, tl, tph), thi = __builtin_amdgcn_alignbyte(t2, tr, tph);
+                        const uint32_t blo = __builtin_amdgcn_alignbyte(br, bl, tph), bhi = __builtin_amdgcn_alignbyte(b2, br, tph);
+                        const float wx = __builtin_amdgcn_fractf(sx), wy = __builtin_amdgcn_fractf(sy);
+                        const float omx = 1.0f - wx, omy = 1.0f - wy;
+                        const float w00 = omy * omx, w01 = omy * wx, w10 = wy * omx;
+                        o0 = __builtin_fmaf(ubyte0(tlo), w00, __builtin_fmaf(ubyte3(tlo), w01, __builtin_fmaf(ubyte0(blo), w10, ubyte3(blo) * wy * wx)));
+                        o1 = __builtin_fmaf(ubyte1(tlo), w00, __builtin_fmaf(ubyte0(thi), w01, __builtin_fmaf(ubyte1(blo), w10, ubyte0(bhi) * wy * wx)));
+                        o2 = __builtin_fmaf(ubyte2(tlo), w00, __builtin_fmaf(ubyte1(thi), w01, __builtin_fmaf(ubyte2(blo), w10, ubyte1(bhi) * wy * wx)));
+                    } else {
                     // s - floor(s): exact for the non-negative coordinates of pixels inside the ROI
                     const float wx = __builtin_amdgcn_fractf(sx), wy = __builtin_amdgcn_fractf(sy);
                     const float omx = 1.0f - wx, omy = 1.0f - wy;
@@ -297,6 +385,7 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
                     o0 = __builtin_fmaf(ubyte0(tl), w00, __builtin_fmaf(ubyte0(tr), w01, __builtin_fmaf(ubyte0(bl), w10, ubyte0(br) * wy * wx)));
                     o1 = __builtin_fmaf(ubyte1(tl), w00, __builtin_fmaf(ubyte1(tr), w01, __builtin_fmaf(ubyte1(bl), w10, ubyte1(br) * wy * wx)));
                     o2 = __builtin_fmaf(ubyte2(tl), w00, __builtin_fmaf(ubyte2(tr), w01, __builtin_fmaf(ubyte2(bl), w10, ubyte2(br) * wy * wx)));
+                    }
                 }
                 v[0][k] = inb ? o0 : 0.0f;
                 v[1][k] = inb ? o1 : 0.0f;
@@ -322,25 +411,27 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     }
 }
 
-template <bool NEAREST>
+template <bool NEAREST, bool RAW>
 static KernelFn pick(int dtype, int layout) {
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return (KernelFn)rmx_warp_kernel<float, RMX_NCHW, NEAREST>;
-            case RMX_FP16: return (KernelFn)rmx_warp_kernel<__half, RMX_NCHW, NEAREST>;
-            default: return (KernelFn)rmx_warp_kernel<uint8_t, RMX_NCHW, NEAREST>;
+            case RMX_FP32: return (KernelFn)rmx_warp_kernel<float, RMX_NCHW, NEAREST, RAW>;
+            case RMX_FP16: return (KernelFn)rmx_warp_kernel<__half, RMX_NCHW, NEAREST, RAW>;
+            default: return (KernelFn)rmx_warp_kernel<uint8_t, RMX_NCHW, NEAREST, RAW>;
         }
     }
     switch (dtype) {
-        case RMX_FP32: return (KernelFn)rmx_warp_kernel<float, RMX_NHWC, NEAREST>;
-        case RMX_FP16: return (KernelFn)rmx_warp_kernel<__half, RMX_NHWC, NEAREST>;
-        default: return (KernelFn)rmx_warp_kernel<uint8_t, RMX_NHWC, NEAREST>;
+        case RMX_FP32: return (KernelFn)rmx_warp_kernel<float, RMX_NHWC, NEAREST, RAW>;
+        case RMX_FP16: return (KernelFn)rmx_warp_kernel<__half, RMX_NHWC, NEAREST, RAW>;
+        default: return (KernelFn)rmx_warp_kernel<uint8_t, RMX_NHWC, NEAREST, RAW>;
     }
 }
 
-KernelFn select_warp_kernel(int interp, int dtype, int layout, const char **name) {
-    *name = "rmx_warp_kernel";
-    return interp == RMX_INTERP_NEAREST ? pick<true>(dtype, layout) : pick<false>(dtype, layout);
+// raw: the box as packed bytes, loaded straight into LDS (every source row must start at the same byte phase)
+KernelFn select_warp_kernel(int interp, int dtype, int layout, bool raw, const char **name) {
+    *name = raw ? "rmx_warp_kernel(raw)" : "rmx_warp_kernel";
+    if (raw) return interp == RMX_INTERP_NEAREST ? pick<true, true>(dtype, layout) : pick<false, true>(dtype, layout);
+    return interp == RMX_INTERP_NEAREST ? pick<true, false>(dtype, layout) : pick<false, false>(dtype, layout);
 }
 
 }  // namespace rmx

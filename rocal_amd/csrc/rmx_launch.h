@@ -17,7 +17,12 @@ KernelFn select_resize_tri_dma_kernel(int dtype, int layout, bool norm, bool qua
 KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name);
 KernelFn select_point_kernel(int kind, int dtype, int layout, bool fast, const char **name);
 KernelFn select_transpose_kernel(int dtype, int layout, const char **name);
-KernelFn select_warp_kernel(int interp, int dtype, int layout, const char **name);
+KernelFn select_warp_kernel(int interp, int dtype, int layout, bool raw, const char **name);
+// LDS pitch, in 16-byte pieces, at which the raw form of the warp kernel stages every box that fits it
+#ifndef RMX_WARP_RAW_PIECES
+#define RMX_WARP_RAW_PIECES 11
+#endif
+constexpr int kWarpRawPieces = RMX_WARP_RAW_PIECES;
 // Normalize: (reduce: zero + per-sample integer moments,) then the FMA constants into the rows of `table` (device memory)
 void launch_stats(hipStream_t stream, const RmxKArgs &a, unsigned long long *counters, RmxSample *table, const float *given, int mode, int per_channel,
                   float scale, float shift, bool reduce);
