@@ -188,16 +188,19 @@ def test_triangular_ring_and_downscale_kernels_agree(ctx, monkeypatch):
     assert np.array_equal(_bits(outs[0]), _bits(outs[1])) and np.array_equal(_bits(outs[0]), _bits(outs[2]))
 
 
+@pytest.mark.parametrize("W", [83, 84])
 @pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST])
-def test_warp_on_an_exact_size_source_and_tiny_windows(ctx, interp):
+def test_warp_on_an_exact_size_source_and_tiny_windows(ctx, interp, W):
     """Boxes that reach the last bytes of the batch buffer (bounds-checked staging), a 1x1 and a 2x3 ROI, ROIs away
-    from the origin (repeated edge column / row), destinations that are not multiples of 8 or of the tile."""
+    from the origin (repeated edge column / row), destinations that are not multiples of 8 or of the tile. Width 84: rows
+    start at multiples of 4 bytes, the form of the kernel that loads boxes straight into LDS; 83: the one that stages them
+    through registers."""
     import torch
     rng = np.random.default_rng(21)
-    n, H, W = 5, 67, 83
+    n, H = 5, 67
     img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
     roi = np.array([[0, 0, W, H], [40, 30, 1, 1], [20, 10, 2, 3], [11, 7, 72, 60], [0, 0, W, H]], np.uint32)
-    dw = np.array([83, 40, 33, 77, 83], np.uint32)
+    dw = np.array([W, 40, 33, 77, W], np.uint32)
     dh = np.array([67, 20, 41, 50, 67], np.uint32)
     affine = np.array([[1.0, 0.0, 0.0, 1.0, 0.0, 0.0],          # identity: reads up to the last pixel
                        [0.1, 0.0, 0.0, 0.1, 0.0, 0.0],
@@ -209,6 +212,7 @@ def test_warp_on_an_exact_size_source_and_tiny_windows(ctx, interp):
     sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
     op = ops.WarpAffine(ctx, sd, sd, interp)
     op.update(roi, affine, dw, dh)
+    assert op.kernel_name == ("rmx_warp_kernel(raw)" if W % 4 == 0 else "rmx_warp_kernel")
     out = op.alloc_output()
     src = torch.from_numpy(img.reshape(-1).copy()).cuda()
     op.launch(src.view(n, H, W, 3), out)

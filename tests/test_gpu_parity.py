@@ -316,7 +316,8 @@ def test_color_twist_all_rgb_values(ctx):
 # ------------------------------------------------------------------ K4: warp / rotate
 
 @pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST])
-def test_warp_affine_config3_small(ctx, interp):
+def test_warp_affine_config3_small(ctx, ctx_staged, interp):
+    """(both forms of the kernel: boxes straight into LDS as packed bytes, and staged through registers)"""
     n = 6
     c = wl.config3(n=n, size=160)
     dw = np.full(n, 160, np.uint32)
@@ -324,20 +325,23 @@ def test_warp_affine_config3_small(ctx, interp):
     m = np.stack([orc.affine_from_rocal(a) for a in c["affine"]])
     exp = orc.warp_affine(c["img"], c["roi"], m, dw, dh, 160, 160, interp=interp)
     sd = ops.desc(n, 160, 160, ops.NHWC, ops.UINT8)
-    op = ops.WarpAffine(ctx, sd, sd, interp)
-    op.update(c["roi"], c["affine"], dw, dh)
-    out = op.alloc_output()
-    op.launch(_gpu(c["img"]), out)
-    _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="warp")
+    for cx, name in ((ctx, "rmx_warp_kernel(raw)"), (ctx_staged, "rmx_warp_kernel")):
+        op = ops.WarpAffine(cx, sd, sd, interp)
+        op.update(c["roi"], c["affine"], dw, dh)
+        assert op.kernel_name == name
+        out = op.alloc_output()
+        op.launch(_gpu(c["img"]), out)
+        _check(_cpu(out, cx), exp, ops.UINT8, exact=True, what=name)
 
 
-def test_rotate_and_odd_shapes(ctx):
+@pytest.mark.parametrize("W", [101, 104])
+def test_rotate_and_odd_shapes(ctx, W):
     rng = np.random.default_rng(13)
-    n, H, W = 5, 75, 101
+    n, H = 5, 75
     img = wl.smooth_noise(rng, n, H, W, sigma=1.5)
-    roi = np.array([[0, 0, 101, 75], [3, 2, 90, 70], [0, 0, 50, 75], [0, 0, 101, 75], [7, 7, 64, 64]], np.uint32)
+    roi = np.array([[0, 0, W, 75], [3, 2, 90, 70], [0, 0, 50, 75], [1, 0, W - 1, 75], [7, 7, 64, 64]], np.uint32)
     angle = np.array([45.0, -30.0, 90.0, 0.0, 179.0], np.float32)
-    dw = np.array([101, 90, 80, 101, 64], np.uint32)
+    dw = np.array([W, 90, 80, W - 1, 64], np.uint32)
     dh = np.array([75, 70, 75, 75, 64], np.uint32)
     m = np.stack([orc.rotate_matrix(a) for a in angle])
     exp = orc.warp_affine(img, roi, m, dw, dh, H, W, interp=orc.LINEAR)
@@ -349,13 +353,15 @@ def test_rotate_and_odd_shapes(ctx):
     _check(_cpu(out, ctx), exp, ops.UINT8, exact=True, what="rotate")
 
 
-def test_warp_minification_falls_back_to_global_gather(ctx):
-    """Scale 6x: the source box of a tile exceeds the LDS slice, the kernel gathers from global memory."""
+@pytest.mark.parametrize("W", [400, 401])
+def test_warp_minification_falls_back_to_global_gather(ctx, W):
+    """Scale 6x: the source box of a tile exceeds the LDS slice, the kernel gathers from global memory; scale 2: boxes wider
+    than the fixed LDS pitch (rows at the box's own pitch)."""
     rng = np.random.default_rng(14)
-    n, H, W = 2, 400, 400
+    n, H = 3, 400
     img = wl.smooth_noise(rng, n, H, W, sigma=1.5)
     roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
-    affine = np.array([[6.0, 0.3, -0.2, 5.5, 3.0, -2.0], [0.2, 7.0, -6.5, 0.1, 0.0, 0.0]], np.float32)
+    affine = np.array([[6.0, 0.3, -0.2, 5.5, 3.0, -2.0], [0.2, 7.0, -6.5, 0.1, 0.0, 0.0], [2.1, 0.4, -0.3, 1.9, 1.5, 0.5]], np.float32)
     dw = np.full(n, 64, np.uint32)
     dh = np.full(n, 64, np.uint32)
     m = np.stack([orc.affine_from_rocal(a) for a in affine])

@@ -175,11 +175,16 @@ def test_random_colour(ctx, seed):
     assert np.array_equal(got, exp), "seed %d kind %d (%s): %d values differ" % (seed, kind, op.plan, int((got != exp).sum()))
 
 
+@pytest.mark.parametrize("w4", [False, True])
 @pytest.mark.parametrize("seed", range(24))
-def test_random_warp(ctx, seed):
+def test_random_warp(ctx, seed, w4):
+    """w4: a source width that is a multiple of 4 (rows start at one byte phase), which takes the form of the kernel that
+    loads the source boxes straight into LDS as packed bytes."""
     rng = np.random.default_rng(5000 + seed)
     n = int(rng.integers(1, 5))
     H, W = int(rng.integers(4, 140)), int(rng.integers(4, 180))
+    if w4:
+        W = (W + 3) // 4 * 4
     img, src = _src(rng, n, H, W)
     roi = _rand_roi(rng, n, H, W)
     dw = np.minimum(rng.integers(1, 200, n), W).astype(np.uint32)
