@@ -337,12 +337,24 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     const size_t plane = (size_t)a.dst_h * a.dst_w;
     const int orow_step = a.dst_w * (LAYOUT == RMX_NCHW ? 1 : 3);
     int rsum_idx = 0;
+    // 1 / (row sum x column sum) is kept from one output row to the next: rows of an integer ratio all have the same sum,
+    // and the division is a dozen instructions per column
+    int rsum_bits_prev = 0;  // (no row sum is +0: a zero sum is replaced by 1)
+    float inv_c[TPX];
+#pragma unroll
+    for (int i = 0; i < TPX; i++) inv_c[i] = 0.0f;
     auto emit = [&](auto slot) {
         constexpr int M = decltype(slot)::value;
-        const float rsum = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rsum_idx));
+        const int rsum_bits = __builtin_amdgcn_readlane(__builtin_bit_cast(int, rsum_v), rsum_idx);
+        if (rsum_bits != rsum_bits_prev) {
+            rsum_bits_prev = rsum_bits;
+            const float rsum = __builtin_bit_cast(float, rsum_bits);
+#pragma unroll
+            for (int i = 0; i < TPX; i++) inv_c[i] = 1 / (rsum * colsum[i]);
+        }
 #pragma unroll
         for (int i = 0; i < TPX; i++) {
-            const float inv = 1 / (rsum * colsum[i]);
+            const float inv = inv_c[i];
 #pragma unroll
             for (int ch = 0; ch < 3; ch++) {
                 float t = acc[M][ch][i] * inv;
