@@ -20,7 +20,8 @@
 #include <type_traits>
 
 // Wavefronts per SIMD the register budget is set for (a workgroup of 256 threads is one wavefront per SIMD): 96 registers,
-// met without spills. Measured on 1080p -> 640 x 360: a budget for six gains nothing, for four loses a fifth.
+// met without spills. Measured on 1080p -> 640 x 360: a budget for six gains nothing, for four loses a fifth. (Also measured:
+// touching the rows of the step after next ahead of the loads, to have them in L2: 65.8 against 60.6 us.)
 #ifndef RMX_TDMA_WAVES
 #define RMX_TDMA_WAVES 5
 #endif
