@@ -1,7 +1,8 @@
 """The streaming triangular kernel (source rows straight into LDS as packed bytes) against the oracle, bit for bit, on what is
 specific to it: windows that start at every byte phase of a dword, edge replicas on both sides, every output format, strips
 whose source rows outnumber the table of vertical coefficients, many vertical taps, mirror, packed (ragged) sources whose
-rows start at multiples of 4 bytes, and the kernel that stages through registers on the same batches."""
+rows start at multiples of 4 bytes (image bases at every byte phase), and the kernel that stages through registers on the same
+batches; the same packed sources through the raw form of the warp kernel."""
 import numpy as np
 import pytest
 
@@ -110,27 +111,39 @@ def test_more_than_sixteen_vertical_taps_take_the_other_kernel(ctx):
     assert np.array_equal(out.cpu().numpy(), exp)
 
 
-def test_packed_source_with_rows_at_multiples_of_four(ctx):
-    """Packed images (a byte offset and a row stride per image, strides multiples of 4) in an exact-size buffer: the last rows
-    of the last image end on the last bytes of the buffer and are staged by the lanes with bounds-checked loads."""
-    rng = np.random.default_rng(8)
-    n = 4
-    widths = np.array([300, 257, 128, 400], np.uint32)
-    heights = np.array([120, 90, 77, 150], np.uint32)
+def _packed(rng, widths, heights, gaps):
+    """Images packed into one buffer, rows padded to multiples of 4 bytes, `gaps[i]` bytes in front of image i (so that image
+    bases fall on every byte phase); returns (buffer, offsets, strides, the same images in a padded tensor)."""
+    n = len(widths)
     strides = (3 * widths + 3) // 4 * 4
     offsets, parts, pos = [], [], 0
-    padded = np.zeros((n, 150, 400, 3), np.uint8)
+    padded = np.zeros((n, int(heights.max()), int(widths.max()), 3), np.uint8)
     for i in range(n):
         h, w, st = int(heights[i]), int(widths[i]), int(strides[i])
         im = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
         padded[i, :h, :w] = im
         rows = np.zeros((h, st), np.uint8)
         rows[:, :3 * w] = im.reshape(h, 3 * w)
+        parts.append(np.full(int(gaps[i]), 0xEE, np.uint8))
+        pos += int(gaps[i])
         offsets.append(pos)
         parts.append(rows.reshape(-1))
         pos += rows.size
     packed = np.concatenate(parts)
     packed = packed[:offsets[-1] + (int(heights[-1]) - 1) * int(strides[-1]) + 3 * int(widths[-1])]  # nothing behind the last pixel
+    return packed, np.array(offsets, np.uint64), strides.astype(np.uint32), padded
+
+
+def test_packed_source_with_rows_at_multiples_of_four(ctx):
+    """Packed images (a byte offset and a row stride per image, strides multiples of 4, bases at byte phases 0, 1, 2, 3) in an
+    exact-size buffer: the last rows of the last image end on the last bytes of the buffer and are staged by the lanes with
+    bounds-checked loads."""
+    rng = np.random.default_rng(8)
+    n = 4
+    widths = np.array([300, 257, 128, 400], np.uint32)
+    heights = np.array([120, 90, 77, 150], np.uint32)
+    packed, offsets, strides, padded = _packed(rng, widths, heights, [0, 1, 2, 3])
+    assert sorted(int(o) % 4 for o in offsets) == [0, 1, 2, 3] or len(set(int(o) % 4 for o in offsets)) >= 3
     roi = np.array([[0, 0, widths[i], heights[i]] for i in range(n)], np.uint32)
     roi[1] = (3, 2, 250, 85)
     dw = np.array([140, 100, 64, 180], np.uint32)
@@ -139,10 +152,41 @@ def test_packed_source_with_rows_at_multiples_of_four(ctx):
     scale, bias = _scale_bias(n)
     exp = orc.resize(padded, roi, dw, dh, 60, 180, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
     op = ops.Resize(ctx, ops.desc(n, 150, 400, ops.NHWC, ops.UINT8), ops.desc(n, 60, 180, ops.NCHW, ops.FP16), ops.TRIANGULAR)
-    op.set_ragged_source(np.array(offsets, np.uint64), widths, heights, packed.size, row_strides=strides)
+    op.set_ragged_source(offsets, widths, heights, packed.size, row_strides=strides)
     op.update_cmn(roi, dw, dh, scale, bias, mirror)
     assert op.kernel_name == "rmx_resize_tri_dma_kernel", op.plan
+    # (torch places the buffer at a 256-byte boundary; the kernels require a 4-byte aligned buffer, not aligned images)
     out = op.alloc_output(fill=1)
     op.launch(_gpu(packed), out)
     ctx.sync()
     _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 1, "packed source")
+
+
+@pytest.mark.parametrize("interp", [ops.LINEAR, ops.NEAREST])
+def test_warp_on_a_packed_source_with_rows_at_multiples_of_four(ctx, interp):
+    """The same kind of source through WarpAffine: its form that loads source boxes straight into LDS, with image bases at
+    every byte phase and boxes that end on the last bytes of the buffer."""
+    rng = np.random.default_rng(9)
+    n = 4
+    widths = np.array([120, 97, 64, 150], np.uint32)
+    heights = np.array([90, 70, 33, 110], np.uint32)
+    packed, offsets, strides, padded = _packed(rng, widths, heights, [0, 3, 2, 1])
+    H, W = padded.shape[1], padded.shape[2]
+    roi = np.array([[0, 0, widths[i], heights[i]] for i in range(n)], np.uint32)
+    roi[1] = (5, 4, 80, 60)
+    affine = np.array([[1.0, 0.0, 0.0, 1.0, 0.0, 0.0], [0.9, 0.25, -0.2, 1.1, 3.5, -2.25], [0.7, -0.6, 0.6, 0.7, 1.0, 2.0], [1.0, 0.0, 0.0, 1.0, 0.4, 0.6]], np.float32)
+    dw = np.array([120, 80, 64, 150], np.uint32)
+    dh = np.array([90, 60, 33, 110], np.uint32)
+    m = np.stack([orc.affine_from_rocal(a) for a in affine])
+    exp = orc.warp_affine(padded, roi, m, dw, dh, H, W, interp=interp)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    op = ops.WarpAffine(ctx, sd, sd, interp)
+    op.set_ragged_source(offsets, widths, heights, packed.size, row_strides=strides)
+    op.update(roi, affine, dw, dh)
+    assert op.kernel_name == "rmx_warp_kernel(raw)", op.plan
+    out = op.alloc_output()
+    op.launch(_gpu(packed), out)
+    ctx.sync()
+    got = out.cpu().numpy()
+    for i in range(n):
+        assert np.array_equal(got[i, :dh[i], :dw[i]], exp[i, :dh[i], :dw[i]]), "sample %d: %d values differ" % (i, int((got[i, :dh[i], :dw[i]] != exp[i, :dh[i], :dw[i]]).sum()))
