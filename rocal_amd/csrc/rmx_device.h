@@ -35,6 +35,13 @@ RMX_DEV const uint8_t *sample_base(const RmxKArgs &a, int s, uint32_t &row_strid
     return a.src + (size_t)s * a.src_h * row_stride;
 }
 
+// Cache policy of the loads that go straight into LDS (0: default; 2: non-temporal). Non-temporal source loads were
+// measured: a batch that is still in the last-level cache is then read from HBM all the same (the bilinear and triangular
+// kernels run at their out-of-cache speed always, no faster out of cache), and the warp kernel, whose tiles share box rows,
+// loses 7 %.
+#ifndef RMX_LDS_LOAD_AUX
+#define RMX_LDS_LOAD_AUX 0
+#endif
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
 typedef const __attribute__((address_space(1))) void *glb_ptr_t;
 typedef __attribute__((address_space(3))) uint8_t lds_u8;    // explicit LDS pointers: every access below is a DS instruction,

@@ -163,7 +163,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     for (int r = 0; r < nrows; r++) {
                         const int ysrc = max(min(a_v + r, yhi), ylo);
                         const uint8_t *rowp = base4 + ((uint32_t)ysrc * row_stride + g.col4);
-                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(bufb + (r * g.ppr + c0) * 16), 16, 0, 0);
+                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(bufb + (r * g.ppr + c0) * 16), 16, 0, RMX_LDS_LOAD_AUX);
                     }
                 }
             }

@@ -211,7 +211,7 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
 #pragma unroll
                 for (int k = 0; k < TS_NCH; k++) {
                     if (k * RMX_WAVE < ppr) {
-                        if (piece_on[k]) __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off[k]), (lds_ptr_t)(slot + k * RMX_WAVE * 16), 16, 0, 0);
+                        if (piece_on[k]) __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off[k]), (lds_ptr_t)(slot + k * RMX_WAVE * 16), 16, 0, RMX_LDS_LOAD_AUX);
                     }
                 }
             } else {

@@ -203,7 +203,7 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
                 const int r = fixed ? idx / WRP : (int)(((float)idx + 0.5f) * inv_ppr);
                 const int c = idx - __mul24(r, ppr);
                 const uint32_t off = (uint32_t)min(by0 + r, yhi) * row_stride + col4 + 16u * (uint32_t)c;
-                if (idx < total) __builtin_amdgcn_global_load_lds((glb_ptr_t)(base4 + off), (lds_ptr_t)(ldsb + 16 * j0), 16, 0, 0);
+                if (idx < total) __builtin_amdgcn_global_load_lds((glb_ptr_t)(base4 + off), (lds_ptr_t)(ldsb + 16 * j0), 16, 0, RMX_LDS_LOAD_AUX);
             }
             // the compiler does not order LDS reads behind loads into LDS: await them explicitly
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
