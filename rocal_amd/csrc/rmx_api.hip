@@ -81,7 +81,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_per_cu = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_per_cu = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -309,6 +309,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
         ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
         ctx->tri_tpx = tune_env("RMX_TUNE_TRI_TPX", ctx->tri_tpx, 1, 2);     // output columns per lane of the downscaling kernel
+        ctx->deal_xcd = tune_env("RMX_TUNE_DEAL_XCD", ctx->deal_xcd, 0, 1);  // samples dealt round-robin to the XCDs (0: eight runs in batch order)
         ctx->tri_per_cu = tune_env("RMX_TUNE_TRI_PER_CU", ctx->tri_per_cu, 0, 32);  // wavefronts per CU the strip planner counts on (0: by registers and LDS)
     }
     *out = ctx;
@@ -446,6 +447,16 @@ static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *
     if (blocks == 0 || blocks > 0x7fffffffull) return fail(RMX_ERR_INVALID, "grid of %llu workgroups is out of range", (unsigned long long)blocks);
     a.wpb = wpb;
     a.nblocks = (uint32_t)blocks;
+    // reciprocals for wave_to_sample (rounded up; exact while dividend x divisor < 2^32, else the kernel divides / keeps batch order)
+    auto recip = [](uint64_t d) { return (uint32_t)(((1ull << 32) + d - 1) / d); };
+    a.inv_strips = (a.strips > 1 && waves * (uint64_t)a.strips < (1ull << 32)) ? recip((uint64_t)a.strips) : 0u;
+    a.per_xcd = 0;
+    a.inv_per_xcd = 0;
+    if (op->ctx->deal_xcd && op->n >= 16 && (uint64_t)op->n * (uint64_t)(op->n / 8) < (1ull << 32)) {
+        a.per_xcd = (uint32_t)(op->n / 8);
+        a.inv_per_xcd = a.per_xcd > 1 ? recip(a.per_xcd) : 0u;
+        if (a.per_xcd == 1) a.per_xcd = 0;  // (8..15 samples: nothing to deal)
+    }
     if (op->kind == OP_NORMALIZE) {
         // moments of every sample's window (when asked for), then the FMA constants into the rows the streaming pass reads;
         // the side table of the slot holds the given statistics (6 floats per sample) and, behind them, the 64-bit counters

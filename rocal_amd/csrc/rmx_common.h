@@ -59,6 +59,9 @@ struct RmxKArgs {
     const RmxSrcLayout *layout;  // per-sample source placement, or null: sample s starts at s*src_h*src_w*3
     const uint8_t *src2;         // second source batch of the same shape (Blend), else null
     const uint8_t *extra;        // per-sample side table behind the layout entries (Gamma: 256 bytes per sample), else null
+    // wavefront -> (sample, strip) without a division, and samples dealt round-robin to the XCDs (see wave_to_sample)
+    uint32_t inv_strips;         // ceil(2^32 / strips), or 0: divide
+    uint32_t per_xcd, inv_per_xcd;  // samples per XCD (n / 8) and ceil(2^32 / per_xcd); per_xcd 0: samples in batch order
 };
 
 #define RMX_WAVE 64

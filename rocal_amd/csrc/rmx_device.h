@@ -79,6 +79,24 @@ RMX_DEV uint32_t xcd_swizzle(uint32_t b, uint32_t nblocks) {
     return (b % XCDS) * per + (b / XCDS);
 }
 
+// Which sample and which of its strips a wavefront works on. The launch numbers its wavefronts so that consecutive ones
+// share an XCD (xcd_swizzle): XCD k gets the k-th eighth of them. Were the samples taken in batch order, a batch whose cost
+// grows or falls along its length (images sorted by size) would give one XCD all the heavy samples (measured: 38 instead of
+// 31 us on the RandomResizedCrop batch sorted by window area). So the samples are dealt round-robin: the i-th sample of XCD k
+// is sample 8 i + k; all strips of a sample still share an XCD and its L2. The two divisions are multiplications by
+// reciprocals that the host rounds up, exact for the ranges the host admits (dividend x divisor < 2^32).
+RMX_DEV void wave_to_sample(const RmxKArgs &a, uint32_t wave, int &sample, int &strip) {
+    const uint32_t strips = (uint32_t)a.strips;
+    const uint32_t slot = a.inv_strips ? __umulhi(wave, a.inv_strips) : (strips == 1 ? wave : wave / strips);
+    strip = (int)(wave - slot * strips);
+    uint32_t s = slot;
+    if (slot < a.per_xcd * 8u) {
+        const uint32_t k = __umulhi(slot, a.inv_per_xcd);  // slot / per_xcd: the XCD
+        s = (slot - k * a.per_xcd) * 8u + k;
+    }
+    sample = (int)s;
+}
+
 // ---------------------------------------------------------------- source loads
 
 // Load `ND` consecutive dwords starting at the 4-byte-aligned address that contains byte

@@ -33,8 +33,8 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + (threadIdx.x / RMX_WAVE);
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int strip = (int)(wave % (uint32_t)a.strips);
+    int s, strip;
+    wave_to_sample(a, wave, s, strip);
     // whole table row in one round trip (the empty statement keeps the fetch above the early exit)
     const RmxSample P = a.table[s];
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.flags), "s"(P.scale[0]), "s"(P.bias[2]));

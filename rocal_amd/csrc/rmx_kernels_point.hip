@@ -34,8 +34,8 @@ __global__ void __launch_bounds__(256) rmx_point_kernel(RmxKArgs a) {
     uint32_t wave = blockIdx.x * (uint32_t)a.wpb + (uint32_t)wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int strip = (int)(wave % (uint32_t)a.strips);
+    int s, strip;
+    wave_to_sample(a, wave, s, strip);
     const RmxSample P = a.table[s];
     const int w = P.dst_w, h = P.dst_h;
     const int srows = a.aux0;

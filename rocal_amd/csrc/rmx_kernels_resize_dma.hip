@@ -75,8 +75,8 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int grp = (int)(wave % (uint32_t)a.strips);
+    int s, grp;
+    wave_to_sample(a, wave, s, grp);
     const RmxSample P = a.table[s];
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.plan[1]));
 

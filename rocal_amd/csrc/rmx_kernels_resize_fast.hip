@@ -57,8 +57,8 @@ __global__ void __launch_bounds__(256) rmx_resize_fast_kernel(RmxKArgs a) {
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int strip = (int)(wave % (uint32_t)a.strips);
+    int s, strip;
+    wave_to_sample(a, wave, s, strip);
     // the whole 128-byte row at once: one memory round trip before the first use, not one per field group
     // (the empty statement "uses" fields from every part of the row, which keeps the compiler from sinking
     // part of the fetch below the early exit)

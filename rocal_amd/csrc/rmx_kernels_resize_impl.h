@@ -112,8 +112,8 @@ __global__ void __launch_bounds__(256) rmx_resize_kernel(RmxKArgs a) {
     uint32_t wave = xcd_swizzle(blockIdx.x, gridDim.x) * (blockDim.x / RMX_WAVE) + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int strip = (int)(wave % (uint32_t)a.strips);
+    int s, strip;
+    wave_to_sample(a, wave, s, strip);
     const RmxSample &P = a.table[s];
 
     const int dw = P.dst_w, dh = P.dst_h;

@@ -22,8 +22,8 @@ __global__ void __launch_bounds__(256) rmx_stats_reduce_kernel(RmxKArgs a, unsig
     uint32_t wave = blockIdx.x * (blockDim.x / RMX_WAVE) + threadIdx.x / RMX_WAVE;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int strip = (int)(wave % (uint32_t)a.strips);
+    int s, strip;
+    wave_to_sample(a, wave, s, strip);
     const RmxSample &P = a.table[s];
     const int w = P.dst_w, h = P.dst_h, x1 = P.src_x, y1 = P.src_y;
     const int r0 = strip * a.aux0;

@@ -22,8 +22,8 @@ __global__ void __launch_bounds__(256) rmx_transpose_kernel(RmxKArgs a) {
     uint32_t wave = blockIdx.x * (blockDim.x / RMX_WAVE) + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int tile = (int)(wave % (uint32_t)a.strips);
+    int s, tile;
+    wave_to_sample(a, wave, s, tile);
     const RmxSample &P = a.table[s];
     const int w = P.src_w, h = P.src_h;  // the window; the output is h columns wide and w rows high
     const int ty = tile / a.aux0, tx = tile - ty * a.aux0;

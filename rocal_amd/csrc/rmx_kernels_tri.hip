@@ -38,8 +38,8 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
     uint32_t wave = xcd_swizzle(blockIdx.x, gridDim.x) * (blockDim.x / RMX_WAVE) + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int part = (int)(wave % (uint32_t)a.strips);
+    int s, part;
+    wave_to_sample(a, wave, s, part);
     const int tiles_x = a.aux1;
     const int strip = part / tiles_x, tx = part - strip * tiles_x;
     const RmxSample &P = a.table[s];
@@ -305,8 +305,8 @@ __global__ void __launch_bounds__(256, RMX_TRI_DOWN_WAVES(NPX)) rmx_resize_tri_d
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int part = (int)(wave % (uint32_t)a.strips);
+    int s, part;
+    wave_to_sample(a, wave, s, part);
     const int tiles_x = a.aux1;
     const int strip = part / tiles_x, tx = part - strip * tiles_x;
     // the whole table row in one round trip

@@ -97,8 +97,8 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int part = (int)(wave % (uint32_t)a.strips);
+    int s, part;
+    wave_to_sample(a, wave, s, part);
     const int tiles_x = a.aux1;
     const int strip = part / tiles_x, tx = part - strip * tiles_x;
     // the whole table row in one round trip

@@ -53,8 +53,8 @@ __global__ void __launch_bounds__(256) rmx_warp_kernel(RmxKArgs a) {
     uint32_t wave = xcd_swizzle(blockIdx.x, a.nblocks) * (uint32_t)a.wpb + wib;
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
-    const int s = (int)(wave / (uint32_t)a.strips);
-    const int tile = (int)(wave % (uint32_t)a.strips);
+    int s, tile;
+    wave_to_sample(a, wave, s, tile);
     const int tiles_x = a.aux0;
     const int passes = a.aux1 >> 8;
     const bool packed_ok = (a.aux1 & 1) != 0;
