@@ -85,12 +85,15 @@ RMX_DEV uint32_t xcd_swizzle(uint32_t b, uint32_t nblocks) {
 // 31 us on the RandomResizedCrop batch sorted by window area). So the samples are dealt round-robin: the i-th sample of XCD k
 // is sample 8 i + k; all strips of a sample still share an XCD and its L2. The two divisions are multiplications by
 // reciprocals that the host rounds up, exact for the ranges the host admits (dividend x divisor < 2^32).
-RMX_DEV void wave_to_sample(const RmxKArgs &a, uint32_t wave, int &sample, int &strip) {
+// With the deal the eight XCDs also work on eight neighbouring samples at a time, one moving window of addresses instead
+// of eight (measured: 2-8 % faster on uniform batches too). `deal` is false in the kernels that do not renumber their
+// workgroups (xcd_swizzle): there the device already walks the batch as one stream, and a deal would only scatter it.
+RMX_DEV void wave_to_sample(const RmxKArgs &a, uint32_t wave, int &sample, int &strip, bool deal = true) {
     const uint32_t strips = (uint32_t)a.strips;
     const uint32_t slot = a.inv_strips ? __umulhi(wave, a.inv_strips) : (strips == 1 ? wave : wave / strips);
     strip = (int)(wave - slot * strips);
     uint32_t s = slot;
-    if (slot < a.per_xcd * 8u) {
+    if (deal && slot < a.per_xcd * 8u) {
         const uint32_t k = __umulhi(slot, a.inv_per_xcd);  // slot / per_xcd: the XCD
         s = (slot - k * a.per_xcd) * 8u + k;
     }

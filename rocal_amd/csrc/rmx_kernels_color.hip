@@ -39,7 +39,9 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
     int s, strip;
-    wave_to_sample(a, wave, s, strip);
+    // workgroups in launch order (no XCD renumbering): the whole device walks the batch as one contiguous address stream,
+    // and dealing the samples would only break that stream up (measured: 11-16 % slower)
+    wave_to_sample(a, wave, s, strip, false);
     // whole table row in one round trip (the empty statement keeps the fetch above the early exit)
     const RmxSample P = a.table[s];
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.flags), "s"(P.color[0]), "s"(P.color[3]));

@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(256) rmx_stats_reduce_kernel(RmxKArgs a, unsig
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
     int s, strip;
-    wave_to_sample(a, wave, s, strip);
+    wave_to_sample(a, wave, s, strip, false);  // no XCD renumbering in this kernel: batch order keeps the address stream contiguous
     const RmxSample &P = a.table[s];
     const int w = P.dst_w, h = P.dst_h, x1 = P.src_x, y1 = P.src_y;
     const int r0 = strip * a.aux0;

@@ -23,7 +23,7 @@ __global__ void __launch_bounds__(256) rmx_transpose_kernel(RmxKArgs a) {
     wave = __builtin_amdgcn_readfirstlane(wave);
     if (wave >= nwaves) return;
     int s, tile;
-    wave_to_sample(a, wave, s, tile);
+    wave_to_sample(a, wave, s, tile, false);  // no XCD renumbering in this kernel: batch order keeps the address stream contiguous
     const RmxSample &P = a.table[s];
     const int w = P.src_w, h = P.src_h;  // the window; the output is h columns wide and w rows high
     const int ty = tile / a.aux0, tx = tile - ty * a.aux0;
