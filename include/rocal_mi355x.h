@@ -75,6 +75,7 @@ typedef struct rmx_tensor_desc {
  * `stream` is ignored. own_stream == 0: `stream` is a hipStream_t to borrow (NULL = the device's
  * default stream). */
 RMX_API int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out);
+/* Destroying a context that still has ops is allowed: the context's streams live on until the last of its ops is destroyed. */
 RMX_API int rmx_ctx_destroy(rmx_ctx *ctx);
 RMX_API int rmx_ctx_sync(rmx_ctx *ctx);
 RMX_API void *rmx_ctx_stream(rmx_ctx *ctx);

@@ -390,3 +390,30 @@ def test_errors_are_loud(ctx):
     roi = np.tile(np.array([0, 0, 8, 8], np.uint32), (2, 1))
     with pytest.raises(RuntimeError, match="standard deviation"):
         op.update(roi, [4, 4], [4, 4], None, np.zeros(6, np.float32), np.zeros(6, np.float32))
+
+
+def test_an_op_may_outlive_its_context():
+    """A context destroyed while ops of it are alive (the order a garbage collector may choose) stays usable by those ops:
+    they still launch on its stream, and the last op's destruction frees it."""
+    import torch
+    c = ops.Context(0, stream="own")
+    n, H, W = 4, 16, 24
+    rng = np.random.default_rng(77)
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    a = ops.Flip(c, sd, sd)
+    b = ops.Flip(c, sd, sd)
+    roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
+    one = np.ones(n, np.uint32)
+    a.update(roi, one, 0 * one)
+    b.update(roi, 0 * one, one)
+    c.close()
+    src = torch.from_numpy(img).cuda()
+    o1, o2 = a.alloc_output(), b.alloc_output()
+    a.launch(src, o1)
+    a.close()
+    b.launch(src, o2)
+    torch.cuda.synchronize()
+    b.close()
+    assert np.array_equal(o1.cpu().numpy(), img[:, :, ::-1])
+    assert np.array_equal(o2.cpu().numpy(), img[:, ::-1])
