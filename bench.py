@@ -423,7 +423,8 @@ def main():
     ap.add_argument("--steps", type=int, default=6000)
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--config", type=int, default=1)
-    ap.add_argument("--all", action="store_true", help="also measure the other configurations (one JSON object per configuration, written to bench_all.json in the output folder)")
+    ap.add_argument("--all", action="store_true", help="also measure the other configurations (one JSON object per configuration on stderr, and all of them in the file --all-out names)")
+    ap.add_argument("--all-out", default=None, help="with --all: file that receives every configuration's result as one JSON object")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--rotating-only", action="store_true", help="only the ramp and the rotating timed loop: every launch of the process is of the "
                     "reported kind, so a rocprofv3 kernel summary of this command averages the same thing")
@@ -449,9 +450,10 @@ def main():
                 allres[cfg] = run_config(cfg, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only, args.rotating_only, args.ramp_ms)
                 allres[cfg]["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
                 print("config %d: %s" % (cfg, json.dumps(allres[cfg])), file=sys.stderr)
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_all.json"), "w") as f:
-            json.dump(allres, f, indent=1)
+        if args.all_out:
+            os.makedirs(os.path.dirname(os.path.abspath(args.all_out)), exist_ok=True)
+            with open(args.all_out, "w") as f:
+                json.dump(allres, f, indent=1)
     print(json.dumps(res))
 
 
