@@ -83,7 +83,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_per_cu = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k3_rows = 8, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_slots = 0, tri_per_cu = 0, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -131,6 +131,7 @@ struct rmx_op {
     int mid_lds = 0, mid_strips = 1, mid_rows = 4, mid_wpb = 1, mid_aux1 = 1;
     bool fast_needs_src16 = false;                                   // fn_fast also wants a 16-byte aligned source base
     uint64_t algo_bytes = 0;
+    int tri_rows_in_flight = 0;  // streaming triangular kernel: accumulator sets (2 or 4), 0 for every other kernel
     int stats_mode = 0, stats_per_channel = 1;  // Normalize: what is computed on the device (bit 0 mean, bit 1 standard deviation)
     float stats_scale = 1.0f, stats_shift = 0.0f;
     rmx::KernelFn lds_fn[3] = {};  // kernels whose static LDS size has been asked of the runtime ([0] general, [1] fast, [2] mid)
@@ -316,6 +317,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
         ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
         ctx->tri_tpx = tune_env("RMX_TUNE_TRI_TPX", ctx->tri_tpx, 1, 2);     // output columns per lane of the downscaling kernel
+        ctx->tri_slots = tune_env("RMX_TUNE_TRI_SLOTS", ctx->tri_slots, 0, 4);  // 4: the streaming triangular kernel always keeps four rows in flight
         ctx->deal_xcd = tune_env("RMX_TUNE_DEAL_XCD", ctx->deal_xcd, 0, 1);  // samples dealt round-robin to the XCDs (0: eight runs in batch order)
         ctx->tri_per_cu = tune_env("RMX_TUNE_TRI_PER_CU", ctx->tri_per_cu, 0, 32);  // wavefronts per CU the strip planner counts on (0: by registers and LDS)
     }
@@ -376,9 +378,11 @@ const char *rmx_op_plan(const rmx_op *op) {
     else if (op->fn_mid)
         snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d lds_per_wave=%d waves_per_block=%d fast=0 any_width=1 group=%d",
                  (long long)op->n * op->mid_strips, op->mid_strips, op->mid_rows, op->mid_lds, op->mid_wpb, std::max(1, op->mid_aux1));
-    else
-        snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=0",
-                 (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block);
+    else {
+        int len = snprintf(buf, sizeof(buf), "waves=%lld strips=%d strip_rows=%d tile_w=%d lds_per_wave=%d waves_per_block=%d fast=0",
+                           (long long)op->n * op->strips, op->strips, op->strip_rows, op->tile_w, op->lds_per_wave, op->waves_per_block);
+        if (op->tri_rows_in_flight && len > 0 && len < (int)sizeof(buf)) snprintf(buf + len, sizeof(buf) - len, " rows_in_flight=%d", op->tri_rows_in_flight);
+    }
     return buf;
 }
 const char *rmx_op_kernel_name(const rmx_op *op) { return op ? (op->fn_fast ? op->fast_name : (op->fn_mid ? op->mid_name : op->kernel_name)) : ""; }
@@ -851,6 +855,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         // Streaming form of the downscaling variant (source rows straight into LDS as raw bytes): every source row must start
         // at the same byte phase (row stride a multiple of 4), and four LDS rows of the widest tile plus the table of vertical
         // coefficients must leave room for ten wavefronts per CU at least.
+        op->tri_rows_in_flight = 0;
         bool tdma = down && op->ctx->dma && op->ctx->tri_tpx == 2 && ky <= 16;
         if (tdma) {
             if (op->layout.empty()) tdma = (op->src.w * 3u) % 4u == 0;
@@ -892,8 +897,36 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             const size_t lds = 4 * pitch_max + (64 + 16) * 4 * 4;
             if (lds > 16 * 1024) tdma = false;
             if (tdma) {
-                op->fn = rmx::select_resize_tri_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, &op->kernel_name);
+                // Two output rows in flight instead of four when rows two apart never read the same source row. That holds
+                // for a vertical ratio that is a whole or a half number: every product and sum of the kernel's coordinate
+                // law is then exact in fp32 (multiples of 1/4 below 2^20), the first taps of rows two apart lie exactly
+                // 2 x ratio = taps rows apart, and only the clamp at the window's ends could fold two such rows onto one
+                // source row: when row 2 starts at or above the first source row, or the taps of the last row but two
+                // reach the last one.
+                bool two = op->ctx->tri_slots != 4;
+                for (int i = 0; i < op->n && two; i++) {
+                    const RmxSample &s = t[i];
+                    if (s.dst_w <= 0 || s.dst_h <= 2) continue;
+                    const float twice = s.ry * 2.0f;
+                    const int ylo = s.src_y, yhi = s.src_y + s.src_h - 1;
+                    if (twice != std::floor(twice) || twice > 32.0f || (double)(s.pc_y + s.dst_h) * (double)s.ry + (double)yhi > 1048576.0) {
+                        two = false;
+                        break;
+                    }
+                    const float radius = s.ry > 1.0f ? s.ry : 1.0f;
+                    const float offset = (s.ry - 1) * 0.5f - radius;
+                    const int ksz = (int)std::ceil(radius * 2);
+                    auto loc_of = [&](int r) {
+                        float raw = (float)(s.pc_y + r) * s.ry;
+                        raw = raw + offset;
+                        raw = raw + (float)ylo;
+                        return (int)std::ceil(raw);
+                    };
+                    two = loc_of(2) > ylo && loc_of((int)s.dst_h - 3) + ksz - 1 < yhi;
+                }
+                op->fn = rmx::select_resize_tri_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, two ? 2 : 4, &op->kernel_name);
                 op->lds_per_wave = (int)lds;
+                op->tri_rows_in_flight = two ? 2 : 4;
             }
         }
         if (down && !tdma) {
@@ -923,8 +956,10 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             // MI355X: a batch of equal strips that march in step runs 10-20 % slower than one whose last strip of each
             // image is a short one, so an R that leaves a remainder of at most R/2 rows is preferred.
             if (op->ctx->tri_rows == 0) {
-                // (wavefronts per CU: 16 by the registers of the kernel that stages through registers, 20 by those of the streaming one)
-                const int per_cu = op->ctx->tri_per_cu > 0 ? op->ctx->tri_per_cu : std::max(1, std::min(tdma ? 20 : 16, (160 * 1024) / op->lds_per_wave));
+                // (wavefronts per CU: 16 by the registers of the kernel that stages through registers, 20 by those of the streaming
+                // one, 24 when it keeps two rows in flight)
+                const int by_regs = tdma ? (op->tri_rows_in_flight == 2 ? 24 : 20) : 16;
+                const int per_cu = op->ctx->tri_per_cu > 0 ? op->ctx->tri_per_cu : std::max(1, std::min(by_regs, (160 * 1024) / op->lds_per_wave));
                 const long slots = (long)op->ctx->num_cus * per_cu;
                 double best_cost = 0.0;
                 for (int r = 4; r <= 64; r++) {

@@ -32,9 +32,12 @@ extern __shared__ uint32_t rmx_lds_tdma[];
 
 typedef __attribute__((address_space(3))) float lds_f32;
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) f32x4 lds_f32x4;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+// the coefficients of one source row for the SLOTS output rows in flight, as one LDS access
+template <int SLOTS> struct SlotVec;
+template <> struct SlotVec<4> { typedef f32x4 type; };
+template <> struct SlotVec<2> { typedef f32x2 type; };
 
-constexpr int TS_SLOTS = 4;  // output rows in flight
 constexpr int TS_RPS = 2;    // source rows per step; the ring holds two steps
 constexpr int TS_NCH = 2;    // load instructions per row at most (64 pieces of 16 bytes each)
 constexpr int TS_TAB = 64;   // source rows of the table of vertical coefficients
@@ -87,8 +90,14 @@ RMX_DEV uint32_t elem_bits(float v) {
     else return (uint32_t)o;
 }
 
-template <typename T, int LAYOUT, bool NORM, bool QUANT>
+// SLOTS: output rows in flight. Four cover every downscale (rows four apart never share a source row). Two are enough when
+// rows two apart never do, which the host establishes for ratios that are whole or half numbers (1080 -> 360 rows, any
+// decimation by 2, 3, 4 or 1.5): every source row then enters two accumulator sets instead of four.
+template <typename T, int LAYOUT, bool NORM, bool QUANT, int SLOTS>
 __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel(RmxKArgs a) {
+    constexpr int TS_SLOTS = SLOTS;
+    typedef typename SlotVec<SLOTS>::type slotv;
+    typedef __attribute__((address_space(3))) slotv lds_slotv;
     constexpr int TPX = 2;               // columns per lane: lane and lane + 64
     constexpr int TTW = RMX_WAVE * TPX;  // output columns per wave tile
     const int lane = threadIdx.x & (RMX_WAVE - 1);
@@ -162,7 +171,7 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     const int body = max(ph + 3 * (l_last + 8 - cs) + 8, 16 * nd);
     const int pitch = lm + (((body + 15) >> 4) << 4);
     const int ppr = pitch >> 4;  // pieces per row
-    const int tab_off = a.lds_bytes - TS_SLOTS * (TS_TAB + TS_EDGE) * 4;  // the tables of vertical coefficients
+    const int tab_off = a.lds_bytes - 4 * (TS_TAB + TS_EDGE) * 4;  // the tables of vertical coefficients (sized for four slots)
     // (the host sizes the slice for four rows of the widest tile; a tile that does not fit is left alone)
     if (2 * TS_RPS * pitch > tab_off || ppr > TS_NCH * RMX_WAVE || 3 * (nrep_l + nrep_r) > RMX_WAVE) return;
 
@@ -310,7 +319,7 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     // filter loop reads a row's entry with one broadcast read. Rebuilt every 64 source rows. The first and the last row
     // of the window serve several taps of a row each (clamped tap indices) and take their own path below.
     lds_f32 *cftab = (lds_f32 *)(bufb + tab_off);
-    const lds_f32x4 *cv_next = (const lds_f32x4 *)cftab;  // the table entry of the next source row
+    const lds_slotv *cv_next = (const lds_slotv *)cftab;  // the table entry of the next source row
     int ytab = y_first;
     auto build_table = [&]() {
         const int y = ytab + lane;
@@ -328,7 +337,10 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
                 }
             }
         }
-        *(lds_f32x4 *)(cftab + TS_SLOTS * lane) = f32x4{cf[0], cf[1], cf[2], cf[3]};
+        slotv cfv;
+#pragma unroll
+        for (int k = 0; k < TS_SLOTS; k++) cfv[k] = cf[k];
+        *(lds_slotv *)(cftab + TS_SLOTS * lane) = cfv;
         wave_sync();
     };
 
@@ -381,7 +393,7 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
         // A row inside the window is one tap of every output row that reads it: one pass, coefficients from the table. The
         // first / last row of the window is also read by every tap index that leaves the window: one pass per such tap, in
         // tap order, coefficients computed here by lane p for pass p (rare: twice per image column of strips at most).
-        const lds_f32x4 *cvp = cv_next++;
+        const lds_slotv *cvp = cv_next++;
         int npass = 1;
         if ((uint32_t)(yy - ylo - 1) >= (uint32_t)(yhi - ylo - 1)) {  // yy == ylo or yy == yhi (rows lie inside the window)
             float ec[TS_SLOTS];
@@ -401,12 +413,15 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
                 }
             }
             lds_f32 *etab = cftab + TS_SLOTS * TS_TAB;
-            if (lane < TS_EDGE) *(lds_f32x4 *)(etab + TS_SLOTS * lane) = f32x4{ec[0], ec[1], ec[2], ec[3]};
+            slotv ecv;
+#pragma unroll
+            for (int m = 0; m < TS_SLOTS; m++) ecv[m] = ec[m];
+            if (lane < TS_EDGE) *(lds_slotv *)(etab + TS_SLOTS * lane) = ecv;
             wave_sync();
-            cvp = (const lds_f32x4 *)etab;
+            cvp = (const lds_slotv *)etab;
             npass = max(npass, 1);
         }
-        f32x4 cv4 = cvp[0];
+        slotv cv4 = cvp[0];
         uint32_t w[TPX][NE + 1];
 #pragma unroll
         for (int i = 0; i < TPX; i++) {
@@ -439,11 +454,16 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
         }
         // ---- rows whose last tap was this source row
         while (qlast <= yy) {
-            switch (rsum_idx & (TS_SLOTS - 1)) {
-                case 0: emit(std::integral_constant<int, 0>{}); break;
-                case 1: emit(std::integral_constant<int, 1>{}); break;
-                case 2: emit(std::integral_constant<int, 2>{}); break;
-                default: emit(std::integral_constant<int, 3>{}); break;
+            if constexpr (TS_SLOTS == 2) {
+                if (rsum_idx & 1) emit(std::integral_constant<int, 1>{});
+                else emit(std::integral_constant<int, 0>{});
+            } else {
+                switch (rsum_idx & 3) {
+                    case 0: emit(std::integral_constant<int, 0>{}); break;
+                    case 1: emit(std::integral_constant<int, 1>{}); break;
+                    case 2: emit(std::integral_constant<int, 2>{}); break;
+                    default: emit(std::integral_constant<int, 3>{}); break;
+                }
             }
             rq++;
             rsum_idx++;
@@ -467,7 +487,7 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
             const int nr = min(TS_RPS, y_last - y + 1);
             if (y + nr - ytab > RMX_WAVE) {
                 ytab = y;
-                cv_next = (const lds_f32x4 *)cftab;
+                cv_next = (const lds_slotv *)cftab;
                 build_table();
             }
             if (by_lanes || emitted > 2) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the lanes' own loads, or many rows)
@@ -490,27 +510,33 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     else run(std::integral_constant<int, 8>{});
 }
 
-template <typename T, int LAYOUT>
+template <typename T, int LAYOUT, int SLOTS>
 static KernelFn pick3_tdma(bool norm, bool quant) {
-    if (norm && quant) return (KernelFn)rmx_resize_tri_dma_kernel<T, LAYOUT, true, true>;
-    if (norm) return (KernelFn)rmx_resize_tri_dma_kernel<T, LAYOUT, true, false>;
-    return (KernelFn)rmx_resize_tri_dma_kernel<T, LAYOUT, false, false>;
+    if (norm && quant) return (KernelFn)rmx_resize_tri_dma_kernel<T, LAYOUT, true, true, SLOTS>;
+    if (norm) return (KernelFn)rmx_resize_tri_dma_kernel<T, LAYOUT, true, false, SLOTS>;
+    return (KernelFn)rmx_resize_tri_dma_kernel<T, LAYOUT, false, false, SLOTS>;
 }
 
-KernelFn select_resize_tri_dma_kernel(int dtype, int layout, bool norm, bool quant, const char **name) {
-    *name = "rmx_resize_tri_dma_kernel";
+template <int SLOTS>
+static KernelFn pick_tdma(int dtype, int layout, bool norm, bool quant) {
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return pick3_tdma<float, RMX_NCHW>(norm, quant);
-            case RMX_FP16: return pick3_tdma<__half, RMX_NCHW>(norm, quant);
-            default: return pick3_tdma<uint8_t, RMX_NCHW>(norm, quant);
+            case RMX_FP32: return pick3_tdma<float, RMX_NCHW, SLOTS>(norm, quant);
+            case RMX_FP16: return pick3_tdma<__half, RMX_NCHW, SLOTS>(norm, quant);
+            default: return pick3_tdma<uint8_t, RMX_NCHW, SLOTS>(norm, quant);
         }
     }
     switch (dtype) {
-        case RMX_FP32: return pick3_tdma<float, RMX_NHWC>(norm, quant);
-        case RMX_FP16: return pick3_tdma<__half, RMX_NHWC>(norm, quant);
-        default: return pick3_tdma<uint8_t, RMX_NHWC>(norm, quant);
+        case RMX_FP32: return pick3_tdma<float, RMX_NHWC, SLOTS>(norm, quant);
+        case RMX_FP16: return pick3_tdma<__half, RMX_NHWC, SLOTS>(norm, quant);
+        default: return pick3_tdma<uint8_t, RMX_NHWC, SLOTS>(norm, quant);
     }
+}
+
+// rows_in_flight: 2 when the host has established that output rows two apart never read the same source row, else 4
+KernelFn select_resize_tri_dma_kernel(int dtype, int layout, bool norm, bool quant, int rows_in_flight, const char **name) {
+    *name = "rmx_resize_tri_dma_kernel";
+    return rows_in_flight == 2 ? pick_tdma<2>(dtype, layout, norm, quant) : pick_tdma<4>(dtype, layout, norm, quant);
 }
 
 }  // namespace rmx

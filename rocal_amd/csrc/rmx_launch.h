@@ -13,7 +13,7 @@ KernelFn select_resize_dma_kernel(int dtype, int layout, bool norm, bool quant, 
 KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, int columns_per_lane, const char **name);
-KernelFn select_resize_tri_dma_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
+KernelFn select_resize_tri_dma_kernel(int dtype, int layout, bool norm, bool quant, int rows_in_flight, const char **name);
 KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name);
 KernelFn select_point_kernel(int kind, int dtype, int layout, bool fast, const char **name);
 KernelFn select_transpose_kernel(int dtype, int layout, const char **name);

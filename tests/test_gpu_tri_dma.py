@@ -95,6 +95,65 @@ def test_many_vertical_taps_and_long_strips(ctx, ry, rows):
         c.close()
 
 
+@pytest.fixture(scope="module")
+def ctx_four_rows():
+    from conftest import _ctx_with_env
+    c = _ctx_with_env(RMX_TUNE_TRI_SLOTS=4)
+    yield c
+    c.close()
+
+
+@pytest.mark.parametrize("ry", [1.0, 1.5, 2.0, 2.5, 3.0, 4.0, 6.5])
+@pytest.mark.parametrize("rows", [0, 5])
+def test_whole_and_half_ratios_keep_two_rows_in_flight(ctx, ctx_four_rows, ry, rows):
+    """Vertical ratios that are whole or half numbers: output rows two apart never share a source row, the kernel keeps two
+    accumulator sets instead of four. Windows at the top, in the middle and at the bottom of the source (the clamp at either
+    end), a window of two output rows, mirror, strips of five rows and planned ones; against the oracle and, bit for bit,
+    against the four-row form. A sample of another ratio in the batch sends the whole batch to the four-row form."""
+    from conftest import _ctx_with_env
+    c = _ctx_with_env(RMX_TUNE_TRI_ROWS=rows) if rows else ctx
+    rng = np.random.default_rng(int(ry * 10) + rows)
+    n, OH, OW = 5, 60, 140
+    H, W = int(OH * ry) + 48, 300
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    dh = np.array([OH, 52, 34, 2, OH], np.uint32)  # even heights: the source heights below are whole numbers for half ratios too
+    dw = np.array([OW, 131, 140, 60, 99], np.uint32)
+    sh = np.array([int(d * ry) for d in dh], np.uint32)
+    assert all(float(s) / float(d) == ry for s, d in zip(sh, dh))
+    roi = np.array([[0, 0, W, sh[0]], [4, 17, 280, sh[1]], [16, H - sh[2], 284, sh[2]], [1, 9, 200, sh[3]], [0, 40, 250, sh[4]]], np.uint32)
+    mirror = np.array([1, 0, 1, 0, 0], np.uint32)
+    scale, bias = _scale_bias(n)
+    sd, dd = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, ops.NCHW, ops.FP16)
+    exp = orc.resize(img, roi, dw, dh, OH, OW, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+    src = _gpu(img)
+    op = ops.Resize(c, sd, dd, ops.TRIANGULAR)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert op.kernel_name == "rmx_resize_tri_dma_kernel" and "rows_in_flight=2" in op.plan, op.plan
+    out = op.alloc_output(fill=3)
+    op.launch(src, out)
+    c.sync()
+    _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 3, "ry=%g (%s)" % (ry, op.plan))
+    op4 = ops.Resize(ctx_four_rows, sd, dd, ops.TRIANGULAR)
+    op4.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert "rows_in_flight=4" in op4.plan, op4.plan
+    out4 = op4.alloc_output(fill=3)
+    op4.launch(src, out4)
+    ctx_four_rows.sync()
+    assert np.array_equal(_bits(out.cpu().numpy()), _bits(out4.cpu().numpy()))
+    # one window of another ratio: four rows in flight for the batch, same results for the others
+    roi2, dh2 = roi.copy(), dh.copy()
+    roi2[4, 3] = sh[4] + 3
+    exp2 = orc.resize(img, roi2, dw, dh2, OH, OW, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+    op.update_cmn(roi2, dw, dh2, scale, bias, mirror)
+    assert "rows_in_flight=4" in op.plan, op.plan
+    out2 = op.alloc_output(fill=3)
+    op.launch(src, out2)
+    c.sync()
+    _check_windows(out2.cpu().numpy(), exp2, dw, dh2, ops.NCHW, 3, "mixed ratios (%s)" % op.plan)
+    if rows:
+        c.close()
+
+
 def test_more_than_sixteen_vertical_taps_take_the_other_kernel(ctx):
     rng = np.random.default_rng(3)
     n, H, W = 1, 400, 64
