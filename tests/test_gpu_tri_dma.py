@@ -154,6 +154,41 @@ def test_whole_and_half_ratios_keep_two_rows_in_flight(ctx, ctx_four_rows, ry, r
         c.close()
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_random_whole_and_half_ratios_with_a_crop_behind_the_resize(ctx, seed):
+    """Seeded sweep of the two-row form: per sample a vertical ratio k / 2 (k = 2 .. 12), any horizontal ratio between 1 and 4,
+    a window anywhere in the source, and a crop window inside the resized image (the strip's first output row is then not the
+    image's first), fused resize -> quantise -> crop -> mirror -> normalise against the two oracle nodes."""
+    rng = np.random.default_rng(7000 + seed)
+    n = int(rng.integers(2, 7))
+    k = rng.integers(2, 13, n)
+    dh = (rng.integers(4, 31, n) * 2).astype(np.uint32)          # even: the source height k dh / 2 is a whole number
+    sh = (dh.astype(np.int64) * k // 2).astype(np.uint32)
+    dw = rng.integers(16, 151, n).astype(np.uint32)
+    sw = np.array([int(rng.integers(d, min(4 * d, 400) + 1)) for d in dw], np.uint32)
+    y0 = rng.integers(0, 20, n).astype(np.uint32)
+    x0 = rng.integers(0, 20, n).astype(np.uint32)
+    H, W = int((y0 + sh).max()) + int(rng.integers(0, 5)), (int((x0 + sw).max()) + 3) // 4 * 4
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    roi = np.stack([x0, y0, sw, sh], 1).astype(np.uint32)
+    crop = np.empty((n, 4), np.uint32)
+    for i in range(n):
+        cw, ch = int(rng.integers(1, dw[i] + 1)), int(rng.integers(1, dh[i] + 1))
+        crop[i] = (int(rng.integers(0, dw[i] - cw + 1)), int(rng.integers(0, dh[i] - ch + 1)), cw, ch)
+    OH, OW = int(crop[:, 3].max()), int(crop[:, 2].max())
+    mirror = rng.integers(0, 2, n).astype(np.uint32)
+    scale, bias = _scale_bias(n)
+    mid = orc.resize(img, roi, dw, dh, int(dh.max()), int(dw.max()), interp=orc.TRIANGULAR)
+    exp = orc.crop_mirror_normalize(mid, crop, scale, bias, mirror, OH, OW, ops.NCHW, ops.FP32)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, ops.NCHW, ops.FP32), ops.TRIANGULAR, flags=ops.F_QUANTIZE_U8)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror, crop_roi=crop)
+    assert op.kernel_name == "rmx_resize_tri_dma_kernel" and "rows_in_flight=2" in op.plan, op.plan
+    out = op.alloc_output(fill=5)
+    op.launch(_gpu(img), out)
+    ctx.sync()
+    _check_windows(out.cpu().numpy(), exp, crop[:, 2], crop[:, 3], ops.NCHW, 5, "seed %d (%s)" % (seed, op.plan))
+
+
 def test_more_than_sixteen_vertical_taps_take_the_other_kernel(ctx):
     rng = np.random.default_rng(3)
     n, H, W = 1, 400, 64
