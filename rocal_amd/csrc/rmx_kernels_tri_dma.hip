@@ -253,21 +253,31 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     // every store instruction is then issued by every wavefront, which the count in the wait below relies on)
     uint32_t xoff[TPX], tap_w[TPX], tap_ph[TPX];
     float colsum[TPX], creg[TPX][8];
+    int locx[TPX];
+    float w0x[TPX];
+    bool lead = false;  // some column's first tap has a coefficient other than 0
 #pragma unroll
     for (int i = 0; i < TPX; i++) {
         const int col = xt + lane + RMX_WAVE * i;
         const int colc = min(col, dw - 1);
         xoff[i] = (uint32_t)(hf ? (dw - 1 - colc) : colc) * (uint32_t)(LAYOUT == RMX_NCHW ? sizeof(T) : 3 * sizeof(T));
-        int locx;
-        float w0;
-        tri_loc(ax, pcx + colc, (float)xlo, locx, w0);
+        tri_loc(ax, pcx + colc, (float)xlo, locx[i], w0x[i]);
         float sum = 0.0f;
-        for (int k = 0; k < kx; k++) sum += tri_coeff(w0, ax.radius, k, ax.fscale);
+        for (int k = 0; k < kx; k++) sum += tri_coeff(w0x[i], ax.radius, k, ax.fscale);
         colsum[i] = (sum == 0.0f) ? 1.0f : sum;
+        lead = lead || !(tri_coeff(w0x[i], ax.radius, 0, ax.fscale) == 0.0f);
+    }
+    // When the first tap of every column of the tile has coefficient 0 (ratios that are odd whole numbers: the first tap then
+    // lies a whole radius from the centre), the horizontal pass starts one pixel on with one tap less: fma(p, 0, 0) is the 0
+    // the accumulation starts from anyway. Wave-uniform.
+    const int skip = (kx > 1 && __builtin_amdgcn_ballot_w64(lead) == 0) ? 1 : 0;
+    const int kx_run = kx - skip;
 #pragma unroll
-        for (int k = 0; k < 8; k++) creg[i][k] = (k < kx) ? tri_coeff(w0, ax.radius, k, ax.fscale) : 0.0f;
+    for (int i = 0; i < TPX; i++) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) creg[i][k] = (k < kx_run) ? tri_coeff(w0x[i], ax.radius, k + skip, ax.fscale) : 0.0f;
         // the first tap's byte inside an LDS row (a tap left of the window reads a replica in or behind the margin)
-        const uint32_t tb = (uint32_t)(lm + ph + 3 * (locx - cs));
+        const uint32_t tb = (uint32_t)(lm + ph + 3 * (locx[i] + skip - cs));
         tap_w[i] = tb & ~3u;
         tap_ph[i] = tb & 3u;
     }
@@ -384,9 +394,9 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
     };
 
     // The row in ring slot `slot` is source row yy: filter it and add it to the output rows in flight. NT = taps of the
-    // unrolled horizontal pass (4, 6 or 8 >= kx): taps beyond kx carry coefficient 0 (fma(p, 0, a) == a for the finite p an
-    // unpacked byte always is), so no bound test is needed inside. A column's 3 NT bytes start at byte tap_ph of dword
-    // tap_w: NE + 1 dwords are read and realigned into NE.
+    // unrolled horizontal pass (4, 5, 6 or 8 >= the taps that are run): taps beyond those carry coefficient 0 (fma(p, 0, a) == a
+    // for the finite p an unpacked byte always is), so no bound test is needed inside. A column's 3 NT bytes start at byte
+    // tap_ph of dword tap_w: NE + 1 dwords are read and realigned into NE.
     auto process_row = [&](auto nt, const lds_u8 *srow, int yy) {
         constexpr int NT = decltype(nt)::value;
         constexpr int NE = (3 * NT + 3) / 4;
@@ -505,8 +515,9 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
             half_nxt = t;
         }
     };
-    if (kx <= 4) run(std::integral_constant<int, 4>{});
-    else if (kx <= 6) run(std::integral_constant<int, 6>{});
+    if (kx_run <= 4) run(std::integral_constant<int, 4>{});
+    else if (kx_run == 5) run(std::integral_constant<int, 5>{});
+    else if (kx_run <= 6) run(std::integral_constant<int, 6>{});
     else run(std::integral_constant<int, 8>{});
 }
 
