@@ -267,7 +267,7 @@ __global__ void __launch_bounds__(256, RMX_TDMA_WAVES) rmx_resize_tri_dma_kernel
         colsum[i] = (sum == 0.0f) ? 1.0f : sum;
         lead = lead || !(tri_coeff(w0x[i], ax.radius, 0, ax.fscale) == 0.0f);
     }
-    // When the first tap of every column of the tile has coefficient 0 (ratios that are odd whole numbers: the first tap then
+    // When the first tap of every column of the tile has coefficient 0 (ratios 1 and 3, the odd whole numbers: the first tap then
     // lies a whole radius from the centre), the horizontal pass starts one pixel on with one tap less: fma(p, 0, 0) is the 0
     // the accumulation starts from anyway. Wave-uniform.
     const int skip = (kx > 1 && __builtin_amdgcn_ballot_w64(lead) == 0) ? 1 : 0;

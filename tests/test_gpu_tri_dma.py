@@ -189,6 +189,36 @@ def test_random_whole_and_half_ratios_with_a_crop_behind_the_resize(ctx, seed):
     _check_windows(out.cpu().numpy(), exp, crop[:, 2], crop[:, 3], ops.NCHW, 5, "seed %d (%s)" % (seed, op.plan))
 
 
+@pytest.mark.parametrize("rx", [1, 3, 5])
+def test_odd_whole_horizontal_ratios_skip_their_first_tap(ctx, ctx_staged, rx):
+    """Horizontal ratios 1 and 3: the first tap of every column has coefficient 0 and the streaming kernel runs one tap less
+    (1 and 5 taps: its 4- and 5-tap passes); ratio 5 has ten taps and goes to the ring kernel. Windows at the left and right
+    end of the source (replicas), in the middle, mirrored; a second tile (more than 128 columns); a batch with one window of
+    another ratio, whose wavefronts keep the first tap. Against the oracle, also through the kernel that stages through registers."""
+    rng = np.random.default_rng(50 + rx)
+    n, OH, OW = 4, 24, 150
+    dw = np.array([OW, 140, 31, 150], np.uint32)
+    sw = (dw * rx).astype(np.uint32)
+    sw[3] = sw[3] + 2                                   # ratio (150 rx + 2) / 150: first taps with coefficients
+    W = (int(sw.max()) + 11) // 4 * 4
+    H = 60
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    roi = np.array([[0, 0, sw[0], 48], [W - sw[1], 5, sw[1], 50], [7, 3, sw[2], 36], [1, 0, sw[3], 60]], np.uint32)
+    dh = np.array([OH, 20, 18, 24], np.uint32)
+    mirror = np.array([0, 1, 0, 1], np.uint32)
+    scale, bias = _scale_bias(n)
+    exp = orc.resize(img, roi, dw, dh, OH, OW, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+    for c in (ctx, ctx_staged):
+        op = ops.Resize(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+        op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        if c is ctx:
+            assert op.kernel_name == ("rmx_resize_tri_dma_kernel" if rx < 5 else "rmx_resize_tri_kernel"), op.plan
+        out = op.alloc_output(fill=9)
+        op.launch(_gpu(img), out)
+        c.sync()
+        _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 9, "rx=%d %s" % (rx, op.kernel_name))
+
+
 def test_more_than_sixteen_vertical_taps_take_the_other_kernel(ctx):
     rng = np.random.default_rng(3)
     n, H, W = 1, 400, 64
