@@ -253,6 +253,46 @@ inline uint8_t *slot_extra(rmx_op *op, RmxSample *rows) {
 
 size_t dtype_size(int dtype) { return dtype == RMX_FP32 ? 4 : dtype == RMX_FP16 ? 2 : 1; }
 
+// Width of the x-tiles of the bilinear fast paths for a destination row of w pixels; 0 when no width fits the LDS budget.
+// A lane blends 8 pixels and the lanes of a wavefront are dealt to whole rows: a tile of L = tw / 8 lanes per row runs
+// floor(64 / L) rows per pass, so tiles of 128, 256 and 512 pixels keep every lane busy (1, 2 and 4 passes for 4 rows), and every
+// tile is one more window to wait for. Cost of a width = passes + half the windows per strip of `rows` rows; the candidates are
+// the whole row and the powers of two below it, of which those whose window fits `cap` bytes (need_of(tw)) compete. Measured on 256
+// images to 299 x 299: tiles of 128 + 128 + 43 pixels 75.5 us, of 144 + 144 + 11 (the whole row halved until it fits) 86.6 us.
+struct TileCost {
+    int of_lanes[65];  // twice the cost of a tile of L lanes per row: a window counts half a pass
+    explicit TileCost(int rows) {
+        of_lanes[0] = 0;
+        for (int lanes = 1; lanes <= 64; lanes++) {
+            const int per_pass = 64 / lanes;
+            of_lanes[lanes] = 1 + 2 * ((rows + per_pass - 1) / per_pass);
+        }
+    }
+};
+template <typename NeedOf>
+int pick_tile_width(int w, const TileCost &tc, long cap, NeedOf need_of, long *need_out) {
+    const int whole = std::min(std::max(w, 8), 512);
+    const int cand[7] = {whole, 256, 128, 64, 32, 16, 8};
+    auto tile_cost = [&tc](int t) { return tc.of_lanes[(t + 7) >> 3]; };
+    int best = 0;
+    long best_cost = 0;
+    for (int k = 0; k < 7; k++) {
+        const int tw = cand[k];
+        if (k > 0 && tw >= whole) continue;
+        if (best != 0 && tw < 64) break;  // (narrower tiles only where nothing wider fits)
+        // whole tiles of the row (no division: cand[k] = 512 >> k for k >= 1, and the whole row is one tile unless it is cut at 512)
+        const int full = (k == 0) ? (w < whole ? 0 : (whole == 512 ? w >> 9 : 1)) : (w >> (9 - k)), rest = w - full * tw;
+        const long cost = (long)full * tile_cost(tw) + (rest ? tile_cost(rest) : 0);
+        if (best != 0 && cost >= best_cost) continue;  // (the window's size is only asked for where it could matter)
+        const long need = need_of(tw);
+        if (need > cap) continue;
+        best = tw;
+        best_cost = cost;
+        *need_out = need;
+    }
+    return best;
+}
+
 void plan_streaming(rmx_op *op, int max_rows, int rows_per_strip) {
     op->strip_rows = rows_per_strip;
     op->strips = std::max(1, (max_rows + rows_per_strip - 1) / rows_per_strip);
@@ -1045,6 +1085,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         bool ok = base_ok && widths8;
         // 4 rows and a 10 KB slice measured best on MI355X (more, shorter-lived wavefronts per CU)
         const int rows = op->ctx->fast_rows, cap = op->ctx->fast_lds;
+        const TileCost tile_cost(rows);
         int need_max = 64;
         for (int i = 0; i < op->n && ok; i++) {
             RmxSample &s = t[i];
@@ -1056,21 +1097,17 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             if (s.dst_w <= 0 || s.dst_h <= 0) continue;
             const float magx = (float)(s.src_x + s.src_w + 2), magy = (float)(s.src_y + s.src_h + 2);
             const int nrows = std::max(2, span_bound(std::min<int>(rows, s.dst_h) - 1, s.ry, magy) + 2);
-            int tw = std::min<int>(s.dst_w, 512);
-            for (;;) {
-                const int nc = std::min<int>(s.src_w, span_bound(tw - 1, s.rx, magx) + 2);
-                const long need = (long)nrows * (8 + ((nc + 3) >> 2) * 4) * 4;  // bytes: one dword per pixel + replicas
-                if (need <= cap) {
-                    s.plan[0] = tw;
-                    need_max = std::max<int>(need_max, (int)need);
-                    break;
-                }
-                if (tw <= 8) {
-                    ok = false;  // a window this tall does not fit: the general kernel takes the batch
-                    break;
-                }
-                tw = std::max(8, (tw / 2) / 8 * 8);
+            long need = 0;
+            const int tw = pick_tile_width((int)s.dst_w, tile_cost, cap, [&](int w) {
+                const int nc = std::min<int>(s.src_w, span_bound(w - 1, s.rx, magx) + 2);
+                return (long)nrows * (8 + ((nc + 3) >> 2) * 4) * 4;  // bytes: one dword per pixel + replicas
+            }, &need);
+            if (tw == 0) {
+                ok = false;  // a window this tall does not fit: the general kernel takes the batch
+                break;
             }
+            s.plan[0] = tw;
+            need_max = std::max<int>(need_max, (int)need);
         }
         if (ok) {
             op->fn_fast = rmx::select_resize_fast_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, chain, &op->fast_name);
@@ -1106,21 +1143,17 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 if (s.dst_w <= 0 || s.dst_h <= 0) continue;
                 const float magx = (float)(s.src_x + s.src_w + 2), magy = (float)(s.src_y + s.src_h + 2);
                 const int nrows = std::max(2, span_bound(std::min<int>(rows, s.dst_h) - 1, s.ry, magy) + 2);
-                int tw = std::min<int>(s.dst_w, 512);
-                for (;;) {
-                    const int nc = std::min<int>(s.src_w, span_bound(tw - 1, s.rx, magx) + 2);
-                    const long need = (long)nrows * (1 + ((3 + 3 * (nc + 2) + 8 + 15) >> 4)) * 16;  // margin piece + data + replicas
-                    if (need <= bufcap) {
-                        s.plan[1] = tw;
-                        need_max = std::max<int>(need_max, (int)need);
-                        break;
-                    }
-                    if (tw <= 8) {
-                        dma = false;
-                        break;
-                    }
-                    tw = std::max(8, (tw / 2) / 8 * 8);
+                long need = 0;
+                const int tw = pick_tile_width((int)s.dst_w, tile_cost, bufcap, [&](int w) {
+                    const int nc = std::min<int>(s.src_w, span_bound(w - 1, s.rx, magx) + 2);
+                    return (long)nrows * (1 + ((3 + 3 * (nc + 2) + 8 + 15) >> 4)) * 16;  // margin piece + data + replicas
+                }, &need);
+                if (tw == 0) {
+                    dma = false;
+                    break;
                 }
+                s.plan[1] = tw;
+                need_max = std::max<int>(need_max, (int)need);
             }
             if (dma && need_max <= op->ctx->max_lds_per_block - kStaticLdsMax) {
                 // A wavefront works through `group` windows (of `rows` destination rows) below each other per x-tile, so that the
