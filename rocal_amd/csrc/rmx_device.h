@@ -210,7 +210,14 @@ template <> struct ElemAligned<4> {
 // by the hardware), a partial one element by element. Measured on 256 images resized to 225 x 225 fp16 planes, where odd rows
 // start at odd multiples of 2 bytes: 59.9 -> 47.8 us against a ladder of alignment tests that ended in element-wise stores
 // (interleaved fp16 at 227 x 227: 82.7 -> 47.3 us).
-template <typename T, int N>
+// NT: streaming (non-temporal) stores.
+template <typename T>
+RMX_DEV void store_elem_nt(T *p, T v) {
+    if constexpr (sizeof(T) == 4) __builtin_nontemporal_store(__builtin_bit_cast(uint32_t, v), reinterpret_cast<uint32_t *>(p));
+    else if constexpr (sizeof(T) == 2) __builtin_nontemporal_store(__builtin_bit_cast(uint16_t, v), reinterpret_cast<uint16_t *>(p));
+    else __builtin_nontemporal_store((uint8_t)v, reinterpret_cast<uint8_t *>(p));
+}
+template <typename T, int N, bool NT = false>
 RMX_DEV void store_run(T *p, const T (&e)[N], int cnt) {
     constexpr int BYTES = N * (int)sizeof(T);
     typedef typename ElemAligned<(int)sizeof(T)>::x4 u32x4_e;
@@ -221,13 +228,19 @@ RMX_DEV void store_run(T *p, const T (&e)[N], int cnt) {
             u32x4_e t[BYTES / 16];
             __builtin_memcpy(t, e, BYTES);
 #pragma unroll
-            for (int i = 0; i < BYTES / 16; i++) reinterpret_cast<u32x4_e *>(p)[i] = t[i];
+            for (int i = 0; i < BYTES / 16; i++) {
+                if constexpr (NT) __builtin_nontemporal_store(t[i], reinterpret_cast<u32x4_e *>(p) + i);
+                else reinterpret_cast<u32x4_e *>(p)[i] = t[i];
+            }
             return;
         } else if constexpr (BYTES % 8 == 0) {
             u32x2_e t[BYTES / 8];
             __builtin_memcpy(t, e, BYTES);
 #pragma unroll
-            for (int i = 0; i < BYTES / 8; i++) reinterpret_cast<u32x2_e *>(p)[i] = t[i];
+            for (int i = 0; i < BYTES / 8; i++) {
+                if constexpr (NT) __builtin_nontemporal_store(t[i], reinterpret_cast<u32x2_e *>(p) + i);
+                else reinterpret_cast<u32x2_e *>(p)[i] = t[i];
+            }
             return;
         } else if constexpr (BYTES % 4 == 0) {
             u32x1_e t[BYTES / 4];
@@ -239,7 +252,10 @@ RMX_DEV void store_run(T *p, const T (&e)[N], int cnt) {
     }
 #pragma unroll
     for (int i = 0; i < N; i++)
-        if (i < cnt) p[i] = e[i];
+        if (i < cnt) {
+            if constexpr (NT) store_elem_nt<T>(p + i, e[i]);
+            else p[i] = e[i];
+        }
 }
 
 // Full-group store for callers that have established alignment: N*sizeof(T) is a multiple of 8
@@ -471,7 +487,7 @@ RMX_DEV void store_packed_coalesced(uint32_t *slab, int grp0, int pos, int L, T 
 // Write one lane's group of N horizontally adjacent pixels (v[c][k], k-th pixel of the group)
 // to output row y starting at column x0. `cnt` pixels are valid. When `rev` the group is
 // written in reversed pixel order (horizontal mirror): pixel k goes to column x0 + cnt-1-k.
-template <typename T, int LAYOUT, int N = PX>
+template <typename T, int LAYOUT, int N = PX, bool NT = false>
 RMX_DEV void store_group(T *sample, int H, int W, int y, int x0, int cnt, const float (&v)[3][N], bool rev) {
     if (cnt <= 0) return;
     if constexpr (LAYOUT == RMX_NCHW) {
@@ -494,7 +510,7 @@ RMX_DEV void store_group(T *sample, int H, int W, int y, int x0, int cnt, const 
                 for (int k = 0; k < N; k++) e[k] = OutCvt<T>::cvt(v[c][k]);
             }
             T *p = sample + ((size_t)c * H + y) * W + x0;
-            store_run<T, N>(p, e, cnt);
+            store_run<T, N, NT>(p, e, cnt);
         }
     } else {
         T e[N * 3];
@@ -520,7 +536,7 @@ RMX_DEV void store_group(T *sample, int H, int W, int y, int x0, int cnt, const 
                 for (int c = 0; c < 3; c++) e[k * 3 + c] = OutCvt<T>::cvt(v[c][k]);
         }
         T *p = sample + ((size_t)y * W + x0) * 3;
-        store_run<T, N * 3>(p, e, cnt * 3);
+        store_run<T, N * 3, NT>(p, e, cnt * 3);
     }
 }
 

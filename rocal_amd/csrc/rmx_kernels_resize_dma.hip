@@ -4,7 +4,7 @@
 //            16-byte stores, held back behind the next window's loads (point 3 below);
 //   any      every other width or base (225, 299, 300 ... wide outputs): the same loads, taps and blend, with the columns of
 //            a tile's short last group clamped to its last column, stored at once (whole groups as 16-byte stores at the
-//            element's alignment, the short group element by element). 44 us against 76 us of the general kernel for 256
+//            element's alignment, the short group element by element). 42 us against 76 us of the general kernel for 256
 //            images to 225 x 225 fp16.
 //
 // One wavefront = a strip of destination rows of one sample, one x-tile at a time, as in the staged kernel
@@ -298,7 +298,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
                 }
                 if constexpr (ALIGNED) pack_group<T, LAYOUT>(v, hf, packed);
-                else store_group<T, LAYOUT>(dimg, a.dst_h, a.dst_w, r, x0, cnt, v, hf);
+                else store_group<T, LAYOUT, PX, RMX_DMA_NT>(dimg, a.dst_h, a.dst_w, r, x0, cnt, v, hf);
             }
             if constexpr (!ALIGNED) continue;
             if (DEFER && rs + G >= r1) {  // the window's last pass: held back
