@@ -380,20 +380,33 @@ typedef uint32_t u32x2_v __attribute__((ext_vector_type(2)));
 // 16- and 8-byte stores; NT = streaming (non-temporal). Measured on MI355X at steady clocks: streaming stores take
 // 1.3-1.5 us off the fp16 output of the bilinear fast path (31.3 -> 29.8 us) and off the u8 output of the colour kernel
 // (24.3 -> 23.0 us), change nothing for the warp kernel and cost 5-10 us on fp32 outputs, so only those two use them.
-template <bool NT>
+// EA = 0: the address is aligned to the store's size; 1, 2, 4: only to an element of that many bytes.
+template <bool NT, int EA = 0>
 RMX_DEV void st4(void *p, uint32_t a, uint32_t b, uint32_t c, uint32_t d) {
-    if constexpr (NT) __builtin_nontemporal_store((u32x4_v){a, b, c, d}, reinterpret_cast<u32x4_v *>(p));
+    if constexpr (EA != 0) {
+        typedef typename ElemAligned<EA>::x4 vec;
+        const vec t = {a, b, c, d};
+        if constexpr (NT) __builtin_nontemporal_store(t, reinterpret_cast<vec *>(p));
+        else *reinterpret_cast<vec *>(p) = t;
+    } else if constexpr (NT) __builtin_nontemporal_store((u32x4_v){a, b, c, d}, reinterpret_cast<u32x4_v *>(p));
     else *reinterpret_cast<uint4 *>(p) = make_uint4(a, b, c, d);
 }
-template <bool NT>
+template <bool NT, int EA = 0>
 RMX_DEV void st2(void *p, uint32_t a, uint32_t b) {
-    if constexpr (NT) __builtin_nontemporal_store((u32x2_v){a, b}, reinterpret_cast<u32x2_v *>(p));
+    if constexpr (EA != 0) {
+        typedef typename ElemAligned<EA>::x2 vec;
+        const vec t = {a, b};
+        if constexpr (NT) __builtin_nontemporal_store(t, reinterpret_cast<vec *>(p));
+        else *reinterpret_cast<vec *>(p) = t;
+    } else if constexpr (NT) __builtin_nontemporal_store((u32x2_v){a, b}, reinterpret_cast<u32x2_v *>(p));
     else *reinterpret_cast<uint2 *>(p) = make_uint2(a, b);
 }
 
-template <typename T, int LAYOUT, bool NT = false>
+// ANY: the run may start at any element (else: at a multiple of its store size).
+template <typename T, int LAYOUT, bool NT = false, bool ANY = false>
 RMX_DEV void store_packed(T *sample, int H, int W, int y, int x0, const PackedGroup<T> &g) {
     constexpr int PW = PX * (int)sizeof(T) / 4;  // dwords per channel run
+    constexpr int EA = ANY ? (int)sizeof(T) : 0;
     if constexpr (LAYOUT == RMX_NCHW) {
 #pragma unroll
         for (int c = 0; c < 3; c++) {
@@ -401,10 +414,10 @@ RMX_DEV void store_packed(T *sample, int H, int W, int y, int x0, const PackedGr
             if constexpr (PW % 4 == 0) {
 #pragma unroll
                 for (int i = 0; i < PW / 4; i++)
-                    st4<NT>(reinterpret_cast<uint4 *>(p) + i, g.w[c * PW + 4 * i], g.w[c * PW + 4 * i + 1], g.w[c * PW + 4 * i + 2], g.w[c * PW + 4 * i + 3]);
+                    st4<NT, EA>(reinterpret_cast<char *>(p) + 16 * i, g.w[c * PW + 4 * i], g.w[c * PW + 4 * i + 1], g.w[c * PW + 4 * i + 2], g.w[c * PW + 4 * i + 3]);
             } else {
 #pragma unroll
-                for (int i = 0; i < PW / 2; i++) st2<NT>(reinterpret_cast<uint2 *>(p) + i, g.w[c * PW + 2 * i], g.w[c * PW + 2 * i + 1]);
+                for (int i = 0; i < PW / 2; i++) st2<NT, EA>(reinterpret_cast<char *>(p) + 8 * i, g.w[c * PW + 2 * i], g.w[c * PW + 2 * i + 1]);
             }
         }
     } else {
@@ -412,10 +425,10 @@ RMX_DEV void store_packed(T *sample, int H, int W, int y, int x0, const PackedGr
         constexpr int TW = PackedGroup<T>::WORDS;
         if constexpr (TW % 4 == 0) {
 #pragma unroll
-            for (int i = 0; i < TW / 4; i++) st4<NT>(reinterpret_cast<uint4 *>(p) + i, g.w[4 * i], g.w[4 * i + 1], g.w[4 * i + 2], g.w[4 * i + 3]);
+            for (int i = 0; i < TW / 4; i++) st4<NT, EA>(reinterpret_cast<char *>(p) + 16 * i, g.w[4 * i], g.w[4 * i + 1], g.w[4 * i + 2], g.w[4 * i + 3]);
         } else {
 #pragma unroll
-            for (int i = 0; i < TW / 2; i++) st2<NT>(reinterpret_cast<uint2 *>(p) + i, g.w[2 * i], g.w[2 * i + 1]);
+            for (int i = 0; i < TW / 2; i++) st2<NT, EA>(reinterpret_cast<char *>(p) + 8 * i, g.w[2 * i], g.w[2 * i + 1]);
         }
     }
 }

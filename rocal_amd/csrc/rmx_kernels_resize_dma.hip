@@ -2,10 +2,9 @@
 // stride a multiple of 4: padded batches whose width is a multiple of 4, which the training shapes are). Two forms:
 //   ALIGNED  every written width a multiple of 8 and a 16-byte aligned destination base: a lane's 8 pixels leave as packed
 //            16-byte stores, held back behind the next window's loads (point 3 below);
-//   any      every other width or base (225, 299, 300 ... wide outputs): the same loads, taps and blend, with the columns of
-//            a tile's short last group clamped to its last column, stored at once (whole groups as 16-byte stores at the
-//            element's alignment, the short group element by element). 42 us against 76 us of the general kernel for 256
-//            images to 225 x 225 fp16.
+//   any      every other width or base (225, 299, 300 ... wide outputs): the same loads, taps, blend and held-back stores;
+//            the stores are 16-byte stores at the element's alignment, and the short last group of a row is moved left until
+//            it is whole. 35 us against 76 us of the general kernel for 256 images to 225 x 225 fp16.
 //
 // One wavefront = a strip of destination rows of one sample, one x-tile at a time, as in the staged kernel
 // (rmx_kernels_resize_fast.hip), but the source window travels from global memory straight into LDS
@@ -63,8 +62,8 @@ struct DmaTile {
 
 // CHAIN: a colour node between the (quantised) resize and the normalisation, see chain_colour().
 // ALIGNED: every written width is a multiple of 8 and the destination base is 16-byte aligned (whole groups, packed 16-byte
-// stores, stores held back); otherwise any width and any base: the last group of a row may be partial and groups are stored
-// element-wise where their address asks for it.
+// stores, stores held back); otherwise any width and any base: groups are stored at the alignment of an element, and only a
+// tile narrower than 8 pixels has a partial group, stored element by element.
 template <typename T, int LAYOUT, bool NORM, bool QUANT, int CHAIN, bool ALIGNED>
 __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     static_assert(CHAIN == CHAIN_NONE || QUANT, "a colour node in the chain reads the u8 output of the resize node");
@@ -203,9 +202,16 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         const int L = ALIGNED ? g.tw / PX : (g.tw + PX - 1) / PX;  // lanes per destination row
         G = RMX_WAVE / L;                                          // destination rows per pass
         lr = lane / L;
-        const int t0 = g.xt + (lane - lr * L) * PX;
+        int t0 = g.xt + (lane - lr * L) * PX;
         const int last = g.xt + g.tw - 1;  // last column of the tile
-        if constexpr (!ALIGNED) cnt = min(PX, last + 1 - t0);
+        if constexpr (!ALIGNED) {
+            // The short last group of a row moves left until it is whole: it then recomputes up to seven pixels of the group
+            // before it and stores the same values to the same places, and every lane has 8 pixels, 16-byte stores and no
+            // element-wise path (which, taken by one lane, costs the wavefront half a pass more). Only a tile narrower than 8
+            // pixels keeps a short group.
+            if (g.tw >= PX) t0 = min(t0, last + 1 - PX);
+            cnt = min(PX, last + 1 - t0);
+        }
         lane_on = lr < G && cnt > 0;
 #pragma unroll
         for (int k = 0; k < PX; k++) {
@@ -226,7 +232,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
     // in registers until the next window's loads have been started (the LDS slice is free once the blend has read it):
     // memory operations of a wavefront complete in issue order, so the wait for those loads, which allows the DEFERRED
     // youngest operations (the held-back stores) to be outstanding, never waits for a store to reach memory.
-    constexpr bool DEFER = ALIGNED && sizeof(T) <= 2;  // (an fp32 run is 24 registers: stored at once)
+    constexpr bool DEFER = sizeof(T) <= 2;  // (an fp32 run is 24 registers: stored at once)
     // The FEWEST store instructions a held-back group can become (more are harmless, fewer would let a load slip through the
     // wait): three planes are three instructions; an interleaved run is contiguous and the compiler merges its stores up to
     // 16 bytes each: 48 bytes of fp16 are three, 24 bytes of u8 two. tests/test_dma_waitcnt_cpu.py checks the generated code.
@@ -267,6 +273,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         for (int rs = r0; rs < r1; rs += G) {
             const int r = rs + lr;
             const bool on = lane_on && r < r1;
+            bool full = on;  // lanes with a whole group of 8 pixels (the any-width form stores a short last group element-wise, at once)
             if (on) {
                 float sy = src_coord_d(pcy + r, ry, offy, fylo);
                 float fy = floorf(sy);
@@ -297,15 +304,15 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     }
                     v[0][k] = o0; v[1][k] = o1; v[2][k] = o2;
                 }
-                if constexpr (ALIGNED) pack_group<T, LAYOUT>(v, hf, packed);
+                if constexpr (!ALIGNED) full = cnt == PX;
+                if (full) pack_group<T, LAYOUT>(v, hf, packed);
                 else store_group<T, LAYOUT, PX, RMX_DMA_NT>(dimg, a.dst_h, a.dst_w, r, x0, cnt, v, hf);
             }
-            if constexpr (!ALIGNED) continue;
             if (DEFER && rs + G >= r1) {  // the window's last pass: held back
-                packed_on = on;
+                packed_on = full;
                 packed_r = r;
-            } else if (on) {
-                store_packed<T, LAYOUT, RMX_DMA_NT>(dimg, a.dst_h, a.dst_w, r, x0, packed);
+            } else if (full) {
+                store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, r, x0, packed);
             }
         }
 
@@ -323,10 +330,12 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
             a_v = issue(ng, nr0, min(nr0 + wrows, r_end));
         }
         asm volatile("" ::: "memory");  // the held-back stores are issued after those loads, not before
-        if (DEFER && packed_on) store_packed<T, LAYOUT, RMX_DMA_NT>(dimg, a.dst_h, a.dst_w, packed_r, x0, packed);
+        if (DEFER && packed_on) store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, packed_r, x0, packed);
         asm volatile("" ::: "memory");
         if (!more) break;
-        held = true;
+        // (the aligned form always holds stores back: lane 0 has a whole group in every last pass; a tile of the any-width
+        // form that is narrower than 8 pixels has none, and then no store was issued behind the loads)
+        held = ALIGNED ? true : (__builtin_amdgcn_ballot_w64(packed_on) != 0);
         if (ntile != tile) taps(ng);  // while the loads are in flight
         g = ng;
         tile = ntile;
