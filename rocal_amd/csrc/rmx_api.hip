@@ -590,7 +590,7 @@ static int create_k1(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const r
     int rc = make_op(ctx, kind, src, dst, roi_type, out);
     if (rc) return rc;
     (*out)->norm = norm;
-    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, norm, false, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, norm, 0, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -632,12 +632,25 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
     for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
     op->fn_fast = nullptr;
     if (aligned) {
-        op->fn_fast = rmx::select_cmn_kernel(op->dst.dtype, op->dst.layout, op->norm, true, &op->fast_name);
+        op->fn_fast = rmx::select_cmn_kernel(op->dst.dtype, op->dst.layout, op->norm, 1, &op->fast_name);
         op->fast_strips = op->strips;
         op->fast_lds = 0;
         op->fast_rows = op->aux0;
         op->fast_wpb = op->waves_per_block;
         op->fast_needs_src16 = false;
+    }
+    // the same pipeline for rows of any width from 8 pixels on and a destination at any element (also what an aligned plan
+    // falls back to when the destination base it is launched on is not 16-byte aligned)
+    bool wide8 = true;
+    for (int i = 0; i < op->n && wide8; i++) wide8 = t[i].dst_w >= 8 || t[i].dst_w <= 0 || t[i].dst_h <= 0;
+    op->fn_mid = nullptr;
+    if (wide8) {
+        op->fn_mid = rmx::select_cmn_kernel(op->dst.dtype, op->dst.layout, op->norm, 2, &op->mid_name);
+        op->mid_strips = op->strips;
+        op->mid_lds = 0;
+        op->mid_rows = op->aux0;
+        op->mid_wpb = op->waves_per_block;
+        op->mid_aux1 = op->aux1;
     }
     if (open_slot) {  // the caller fills the side table of the slot and commits it
         *open_slot = slot;
@@ -692,7 +705,7 @@ int rmx_create_normalize(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_ten
     int rc = make_op(ctx, OP_NORMALIZE, src, dst, roi_type, out, 72);
     if (rc) return rc;
     (*out)->norm = true;
-    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, true, false, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, true, 0, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -742,7 +755,7 @@ int rmx_create_transpose(rmx_ctx *ctx, const rmx_tensor_desc *src, const rmx_ten
     if (rc) return rc;
     (*out)->aux1 = swap ? 1 : 0;
     if (swap) (*out)->fn = rmx::select_transpose_kernel(dst->dtype, dst->layout, &(*out)->kernel_name);
-    else (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, false, false, &(*out)->kernel_name);
+    else (*out)->fn = rmx::select_cmn_kernel(dst->dtype, dst->layout, false, 0, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -1303,7 +1316,7 @@ static int create_color(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, cons
     int rc = make_op(ctx, kind, src, dst, roi_type, out);
     if (rc) return rc;
     const bool twist = (kind == OP_COLOR_TWIST || kind == OP_HUE || kind == OP_SATURATION);
-    (*out)->fn = rmx::select_color_kernel(twist ? 1 : 0, dst->dtype, dst->layout, false, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_color_kernel(twist ? 1 : 0, dst->dtype, dst->layout, 0, &(*out)->kernel_name);
     return RMX_OK;
 }
 
@@ -1344,12 +1357,24 @@ static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const 
     op->fn_fast = nullptr;
     if (aligned) {
         const bool twist = (op->kind == OP_COLOR_TWIST || op->kind == OP_HUE || op->kind == OP_SATURATION);
-        op->fn_fast = rmx::select_color_kernel(twist ? 1 : 0, op->dst.dtype, op->dst.layout, true, &op->fast_name);
+        op->fn_fast = rmx::select_color_kernel(twist ? 1 : 0, op->dst.dtype, op->dst.layout, 1, &op->fast_name);
         op->fast_strips = op->strips;
         op->fast_lds = 0;
         op->fast_rows = op->aux0;
         op->fast_wpb = op->waves_per_block;
         op->fast_needs_src16 = false;
+    }
+    // the same pipeline for rows of any width from 8 pixels on and a destination at any element
+    bool wide8 = true;
+    for (int i = 0; i < op->n && wide8; i++) wide8 = t[i].dst_w >= 8 || t[i].dst_w <= 0 || t[i].dst_h <= 0;
+    op->fn_mid = nullptr;
+    if (wide8) {
+        op->fn_mid = rmx::select_color_kernel((op->kind == OP_COLOR_TWIST || op->kind == OP_HUE || op->kind == OP_SATURATION) ? 1 : 0, op->dst.dtype, op->dst.layout, 2, &op->mid_name);
+        op->mid_strips = op->strips;
+        op->mid_lds = 0;
+        op->mid_rows = op->aux0;
+        op->mid_wpb = op->waves_per_block;
+        op->mid_aux1 = op->aux1;
     }
     return commit_slot(op, slot);
 }
@@ -1429,7 +1454,7 @@ int rmx_update_color_temperature(rmx_op *op, const uint32_t *src_roi, const int3
 static int create_point(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out) {
     int rc = make_op(ctx, kind, src, dst, roi_type, out, kind == OP_GAMMA ? 256 : 0);
     if (rc) return rc;
-    (*out)->fn = rmx::select_point_kernel(kind == OP_BLEND ? 1 : 0, dst->dtype, dst->layout, false, &(*out)->kernel_name);
+    (*out)->fn = rmx::select_point_kernel(kind == OP_BLEND ? 1 : 0, dst->dtype, dst->layout, 0, &(*out)->kernel_name);
     if (kind == OP_GAMMA) {
         (*out)->lut_gamma.assign((size_t)(*out)->n, std::numeric_limits<float>::quiet_NaN());
         (*out)->lut_cache.assign((size_t)(*out)->n * 256, 0);
@@ -1478,12 +1503,24 @@ static int update_point(rmx_op *op, const uint32_t *roi, const float *p0, const 
     for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
     op->fn_fast = nullptr;
     if (aligned) {
-        op->fn_fast = rmx::select_point_kernel(op->kind == OP_BLEND ? 1 : 0, op->dst.dtype, op->dst.layout, true, &op->fast_name);
+        op->fn_fast = rmx::select_point_kernel(op->kind == OP_BLEND ? 1 : 0, op->dst.dtype, op->dst.layout, 1, &op->fast_name);
         op->fast_strips = op->strips;
         op->fast_lds = 0;
         op->fast_rows = op->aux0;
         op->fast_wpb = op->waves_per_block;
         op->fast_needs_src16 = false;
+    }
+    // the same pipeline for rows of any width from 8 pixels on and a destination at any element
+    bool wide8 = true;
+    for (int i = 0; i < op->n && wide8; i++) wide8 = t[i].dst_w >= 8 || t[i].dst_w <= 0 || t[i].dst_h <= 0;
+    op->fn_mid = nullptr;
+    if (wide8) {
+        op->fn_mid = rmx::select_point_kernel(op->kind == OP_BLEND ? 1 : 0, op->dst.dtype, op->dst.layout, 2, &op->mid_name);
+        op->mid_strips = op->strips;
+        op->mid_lds = 0;
+        op->mid_rows = op->aux0;
+        op->mid_wpb = op->waves_per_block;
+        op->mid_aux1 = op->aux1;
     }
     return commit_slot(op, slot);
 }

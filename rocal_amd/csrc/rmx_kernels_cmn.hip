@@ -10,6 +10,11 @@
 // to four row steps are issued back to back before the first one is used, and the stores follow, so a
 // wavefront pays one memory round trip per strip instead of one per row step (loads and stores share one
 // in-order counter on this hardware: a load issued behind a store waits for that store as well).
+// ANY variant of it (crops of 225, 299 ... pixels, a destination at any element): the same pipeline; the short last group of
+// a row is moved left until it is whole (it then recomputes up to seven pixels of its neighbour and stores the same values to
+// the same places), and a group leaves as 16-byte stores at the element's own alignment. 128 crops of 299 x 299 to fp16
+// planes: 30.4 us through the general path (row by row, element-wise stores for the short group, which cost the whole
+// wavefront), 20 us at 296 or 304.
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
@@ -19,10 +24,14 @@
 
 namespace rmx {
 
-template <typename T, int LAYOUT, bool NORM, bool FAST>
+enum { CMN_GENERAL = 0, CMN_FAST = 1, CMN_FAST_ANY = 2 };
+
+template <typename T, int LAYOUT, bool NORM, int MODE>
 __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
+    constexpr bool FAST = MODE != CMN_GENERAL;
+    constexpr bool ANY = MODE == CMN_FAST_ANY;
     // LDS slab through which the lanes of a row exchange their runs before storing (see store_packed_coalesced)
-    constexpr bool COALESCE = FAST && coalesce_pays<T, LAYOUT>();
+    constexpr bool COALESCE = MODE == CMN_FAST && coalesce_pays<T, LAYOUT>();
     uint32_t *slab = nullptr;
     if constexpr (COALESCE) {
         __shared__ __attribute__((aligned(16))) uint32_t slabs[4 * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>()];
@@ -68,7 +77,8 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
         const int G = RMX_WAVE / L;        // rows per step
         const int lr = lane / L;
         const int g = lane - lr * L;
-        const int gx = xt + g * PX;               // first output column of this lane's group
+        int gx = xt + g * PX;                     // first output column of this lane's group
+        if constexpr (ANY) gx = min(gx, cw - PX);  // (the host admits this variant for rows of 8 pixels and more)
         const int cnt = min(PX, cw - gx);         // valid pixels in the group
         const bool active = lr < G;
         // source column of group pixel 0 (mirror reads the mirrored run and reverses it)
@@ -101,7 +111,7 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
                 PackedGroup<T> packed;
                 pack_group<T, LAYOUT>(v, hf, packed);
                 if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT, RMX_K1_NT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
-                else store_packed<T, LAYOUT, RMX_K1_NT>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                else store_packed<T, LAYOUT, RMX_K1_NT && !(ANY && sizeof(T) == 4), ANY>(dimg, a.dst_h, a.dst_w, r, gx, packed);
             };
             // every wide load of this wavefront's strip stays inside the batch buffer (the first and the last row bound the rest)
             bool lane_safe = true;
@@ -189,24 +199,26 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
 }
 
 template <typename T, int LAYOUT>
-static KernelFn pick_variant(bool norm, bool fast) {
-    if (fast) return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, true> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, true>;
-    return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, false> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, false>;
+static KernelFn pick_variant(bool norm, int mode) {
+    if (mode == CMN_FAST) return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, CMN_FAST> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, CMN_FAST>;
+    if (mode == CMN_FAST_ANY) return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, CMN_FAST_ANY> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, CMN_FAST_ANY>;
+    return norm ? (KernelFn)rmx_cmn_kernel<T, LAYOUT, true, CMN_GENERAL> : (KernelFn)rmx_cmn_kernel<T, LAYOUT, false, CMN_GENERAL>;
 }
 
 template <typename T>
-static KernelFn pick_layout(int layout, bool norm, bool fast) {
-    if (layout == RMX_NCHW) return pick_variant<T, RMX_NCHW>(norm, fast);
-    return pick_variant<T, RMX_NHWC>(norm, fast);
+static KernelFn pick_layout(int layout, bool norm, int mode) {
+    if (layout == RMX_NCHW) return pick_variant<T, RMX_NCHW>(norm, mode);
+    return pick_variant<T, RMX_NHWC>(norm, mode);
 }
 
-KernelFn select_cmn_kernel(int dtype, int layout, bool norm, bool fast, const char **name) {
+// mode: 0 the general kernel, 1 whole groups and 16-byte aligned destination rows, 2 rows of 8 pixels and more at any alignment
+KernelFn select_cmn_kernel(int dtype, int layout, bool norm, int mode, const char **name) {
     static const char *names[3] = {"rmx_cmn_kernel<float", "rmx_cmn_kernel<__half", "rmx_cmn_kernel<unsigned char"};
     *name = names[dtype];
     switch (dtype) {
-        case RMX_FP32: return pick_layout<float>(layout, norm, fast);
-        case RMX_FP16: return pick_layout<__half>(layout, norm, fast);
-        default: return pick_layout<uint8_t>(layout, norm, fast);
+        case RMX_FP32: return pick_layout<float>(layout, norm, mode);
+        case RMX_FP16: return pick_layout<__half>(layout, norm, mode);
+        default: return pick_layout<uint8_t>(layout, norm, mode);
     }
 }
 

@@ -14,8 +14,13 @@ namespace rmx {
 enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
 
 
-template <typename T, int LAYOUT, int KIND, bool FAST>
+// MODE: 0 the general form; 1 whole 8-pixel groups and 16-byte aligned destination rows; 2 rows of 8 pixels and more at any
+// alignment: the pipeline of 1, the short last group of a row moved left until it is whole (it recomputes up to seven pixels of
+// its neighbour and stores the same values to the same places), groups stored at the element's own alignment.
+template <typename T, int LAYOUT, int KIND, int MODE>
 __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
+    constexpr bool FAST = MODE != 0;
+    constexpr bool ANY = MODE == 2;
     __shared__ ColorTables tabs;
     const float *rcp = tabs.rcp;
     const SectorRow *sect = tabs.sect;
@@ -28,7 +33,7 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     // fp32 and interleaved fp16 outputs: the lanes of a row exchange their runs through LDS before storing (store_packed_coalesced)
-    constexpr bool COALESCE = FAST && coalesce_pays<T, LAYOUT>();
+    constexpr bool COALESCE = MODE == 1 && coalesce_pays<T, LAYOUT>();
     uint32_t *slab = nullptr;
     if constexpr (COALESCE) {
         __shared__ __attribute__((aligned(16))) uint32_t slabs[4 * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>()];
@@ -81,7 +86,8 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
         const int G = RMX_WAVE / L;
         const int lr = lane / L;
         const int g = lane - lr * L;
-        const int gx = xt + g * PX;
+        int gx = xt + g * PX;
+        if constexpr (ANY) gx = min(gx, w - PX);  // (the host admits this form for rows of 8 pixels and more)
         const int cnt = min(PX, w - gx);
         if constexpr (FAST) {
             // whole groups and aligned destination rows: the loads of up to NI row steps go out together,
@@ -129,7 +135,7 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
                         PackedGroup<T> packed;
                         pack_group_dir<T, LAYOUT, false>(v, packed);
                         if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
-                        else store_packed<T, LAYOUT, sizeof(T) == 1>(dimg, a.dst_h, a.dst_w, r, gx, packed);  // u8: streaming stores
+                        else store_packed<T, LAYOUT, sizeof(T) == 1, ANY>(dimg, a.dst_h, a.dst_w, r, gx, packed);  // u8: streaming stores
                     }
                 }
             }
@@ -147,26 +153,30 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     }
 }
 
-template <int KIND, bool FAST>
+template <int KIND, int MODE>
 static KernelFn pick(int dtype, int layout) {
     if (layout == RMX_NCHW) {
         switch (dtype) {
-            case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NCHW, KIND, FAST>;
-            case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NCHW, KIND, FAST>;
-            default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NCHW, KIND, FAST>;
+            case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NCHW, KIND, MODE>;
+            case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NCHW, KIND, MODE>;
+            default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NCHW, KIND, MODE>;
         }
     }
     switch (dtype) {
-        case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NHWC, KIND, FAST>;
-        case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NHWC, KIND, FAST>;
-        default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NHWC, KIND, FAST>;
+        case RMX_FP32: return (KernelFn)rmx_color_kernel<float, RMX_NHWC, KIND, MODE>;
+        case RMX_FP16: return (KernelFn)rmx_color_kernel<__half, RMX_NHWC, KIND, MODE>;
+        default: return (KernelFn)rmx_color_kernel<uint8_t, RMX_NHWC, KIND, MODE>;
     }
 }
 
-KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name) {
+template <int KIND>
+static KernelFn pick_mode(int mode, int dtype, int layout) {
+    return mode == 1 ? pick<KIND, 1>(dtype, layout) : (mode == 2 ? pick<KIND, 2>(dtype, layout) : pick<KIND, 0>(dtype, layout));
+}
+
+KernelFn select_color_kernel(int kind, int dtype, int layout, int mode, const char **name) {
     *name = "rmx_color_kernel";
-    if (fast) return kind == COLOR_TWIST ? pick<COLOR_TWIST, true>(dtype, layout) : pick<COLOR_LINEAR, true>(dtype, layout);
-    return kind == COLOR_TWIST ? pick<COLOR_TWIST, false>(dtype, layout) : pick<COLOR_LINEAR, false>(dtype, layout);
+    return kind == COLOR_TWIST ? pick_mode<COLOR_TWIST>(mode, dtype, layout) : pick_mode<COLOR_LINEAR>(mode, dtype, layout);
 }
 
 }  // namespace rmx

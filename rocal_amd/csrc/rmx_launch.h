@@ -6,7 +6,7 @@
 namespace rmx {
 typedef void (*KernelFn)(RmxKArgs);
 
-KernelFn select_cmn_kernel(int dtype, int layout, bool norm, bool fast, const char **name);
+KernelFn select_cmn_kernel(int dtype, int layout, bool norm, int mode, const char **name);
 KernelFn select_resize_linear_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name);
 KernelFn select_resize_fast_kernel(int dtype, int layout, bool norm, bool quant, int chain, const char **name);
 KernelFn select_resize_dma_kernel(int dtype, int layout, bool norm, bool quant, int chain, bool aligned, const char **name);
@@ -14,8 +14,8 @@ KernelFn select_resize_nearest_kernel(int dtype, int layout, bool norm, bool qua
 KernelFn select_resize_tri_kernel(int dtype, int layout, bool norm, bool quant, const char **name);
 KernelFn select_resize_tri_down_kernel(int dtype, int layout, bool norm, bool quant, int columns_per_lane, const char **name);
 KernelFn select_resize_tri_dma_kernel(int dtype, int layout, bool norm, bool quant, int rows_in_flight, const char **name);
-KernelFn select_color_kernel(int kind, int dtype, int layout, bool fast, const char **name);
-KernelFn select_point_kernel(int kind, int dtype, int layout, bool fast, const char **name);
+KernelFn select_color_kernel(int kind, int dtype, int layout, int mode, const char **name);
+KernelFn select_point_kernel(int kind, int dtype, int layout, int mode, const char **name);
 KernelFn select_transpose_kernel(int dtype, int layout, const char **name);
 KernelFn select_warp_kernel(int interp, int dtype, int layout, bool raw, const char **name);
 // LDS pitch, in 16-byte pieces, at which the raw form of the warp kernel stages every box that fits it
