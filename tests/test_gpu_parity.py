@@ -417,3 +417,55 @@ def test_an_op_may_outlive_its_context():
     b.close()
     assert np.array_equal(o1.cpu().numpy(), img[:, :, ::-1])
     assert np.array_equal(o2.cpu().numpy(), img[:, ::-1])
+
+
+@pytest.mark.parametrize("w", [8, 9, 11, 15, 16, 17, 23, 65, 129])
+def test_rows_of_every_small_width_through_the_pipelined_forms(ctx, w):
+    """Widths just above the 8-pixel group: the last group of a row is moved left until it is whole and overlaps its neighbour
+    by 7 .. 1 pixels (width 8: a single group; 65, 129: the overlap falls into a second 64-lane tile of the bilinear kernel or
+    behind 8 and 16 whole groups). CropMirrorNormalize (fp16 and fp32 planes, interleaved u8, mirrored and not) and the fused bilinear
+    resize on destination tensors exactly as wide as the rows (rows at odd element offsets), ColorTwist on a window."""
+    rng = np.random.default_rng(600 + w)
+    n, H, W = 4, 40, 160
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    src = _gpu(img)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    mirror = np.array([0, 1, 1, 0], np.uint32)
+    scale, bias = _mean_std(n)
+    crop = np.array([[0, 0, w, 33], [3, 2, w, 37], [W - w, 0, w, 40], [1, 5, w, 9]], np.uint32)
+    for layout, dtype in ((ops.NCHW, ops.FP16), (ops.NHWC, ops.UINT8), (ops.NCHW, ops.FP32)):
+        norm = dtype != ops.UINT8
+        sc, bi = (scale, bias) if norm else (np.ones(3 * n, np.float32), np.zeros(3 * n, np.float32))
+        exp = orc.crop_mirror_normalize(img, crop, sc, bi, mirror, 40, w, layout, dtype)
+        op = ops.CropMirrorNormalize(ctx, sd, ops.desc(n, 40, w, layout, dtype))
+        op.update(crop, sc, bi, mirror)
+        out = op.alloc_output()
+        op.launch(src, out)
+        got = _cpu(out, ctx)
+        for i in range(n):
+            hh = int(crop[i, 3])
+            a, b = (got[i, :, :hh], exp[i, :, :hh]) if layout == ops.NCHW else (got[i, :hh], exp[i, :hh])
+            assert np.array_equal(a, b), "cmn w=%d layout=%d dtype=%d sample %d" % (w, layout, dtype, i)
+    alpha, beta = np.full(n, 1.2, np.float32), np.full(n, 4.0, np.float32)
+    hue, sat = np.array([0, 40, 200, 310], np.float32), np.array([1.0, 0.5, 1.5, 0.0], np.float32)
+    exp = orc.color_twist(img, crop, alpha, beta, hue, sat)  # (the window's result at the top left of a source-sized tensor)
+    op = ops.ColorTwist(ctx, sd, sd)
+    op.update(crop, alpha, beta, hue, sat)
+    out = op.alloc_output()
+    op.launch(src, out)
+    got = _cpu(out, ctx)
+    for i in range(n):
+        hh = int(crop[i, 3])
+        assert np.array_equal(got[i, :hh, :w], exp[i, :hh, :w]), "twist w=%d sample %d" % (w, i)
+    roi = np.array([[0, 0, W, H], [5, 3, 120, 30], [40, 0, 120, 40], [0, 10, 77, 25]], np.uint32)
+    dw, dh = np.full(n, w, np.uint32), np.array([21, 30, 17, 8], np.uint32)
+    exp = orc.resize(img, roi, dw, dh, 30, w, interp=orc.LINEAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16,
+                     flags=orc.F_QUANTIZE_U8)
+    op = ops.Resize(ctx, sd, ops.desc(n, 30, w, ops.NCHW, ops.FP16), ops.LINEAR, flags=ops.F_QUANTIZE_U8)
+    op.update_cmn(roi, dw, dh, scale, bias, mirror)
+    assert op.kernel_name == "rmx_resize_dma_kernel", op.plan
+    out = op.alloc_output()
+    op.launch(src, out)
+    got = _cpu(out, ctx)
+    for i in range(n):
+        assert np.array_equal(got[i, :, :dh[i]].view(np.uint16), exp[i, :, :dh[i]].view(np.uint16)), "resize w=%d sample %d" % (w, i)
