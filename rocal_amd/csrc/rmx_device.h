@@ -497,6 +497,49 @@ RMX_DEV void store_packed_coalesced(uint32_t *slab, int grp0, int pos, int L, T 
     }
 }
 
+// The same for fp32 rows of any width at any (4-byte) alignment, whose last run overlaps its neighbour: a lane's run of W
+// dwords goes to the slab at its own offset `off` (dwords) in the row group's segment of `total` dwords, overlapping runs
+// writing the same values; the segment then leaves as 16-byte pieces at 16-byte aligned addresses, consecutive lanes writing
+// consecutive pieces (the slab is read at the matching, dword-aligned offset), and the up to three dwords in front of the
+// first piece and behind the last one by one. (16-byte stores at addresses that are only dword-aligned were measured as slow
+// as no exchange at all: 128 crops of 225 x 225 to fp32 planes 27.1 us either way.)
+template <int W, bool NT>
+RMX_DEV void store_run_coalesced_any(uint32_t *slab, uint8_t *seg, int grp0, int l, int L, int off, int total, const uint32_t *w) {
+    typedef typename ElemAligned<4>::x4 vec;
+    uint32_t *grp = slab + grp0 * W;
+#pragma unroll
+    for (int j = 0; j < W / 4; j++) *reinterpret_cast<vec *>(grp + off + 4 * j) = (vec){w[4 * j], w[4 * j + 1], w[4 * j + 2], w[4 * j + 3]};
+    wave_sync();
+    const int head = min((int)((4u - (uint32_t)(((uintptr_t)seg >> 2) & 3u)) & 3u), total);  // dwords in front of the first aligned piece
+    const int body = (total - head) >> 2;                                                   // aligned pieces
+    for (int idx = l; idx < body; idx += L) {
+        const vec v = *reinterpret_cast<const vec *>(grp + head + 4 * idx);
+        st4<NT>(seg + (size_t)(head + 4 * idx) * 4, v.x, v.y, v.z, v.w);
+    }
+    const int loose = total - 4 * body;  // head + tail, at most six dwords
+    for (int e = l; e < loose; e += L) {
+        const int i = e < head ? e : 4 * body + e;
+        reinterpret_cast<uint32_t *>(seg)[i] = grp[i];
+    }
+    wave_sync();  // the slab is reused by the next call
+}
+
+// xs: first column of the row group, tw: its width in pixels; x0: first column of this lane's run (fp32 only).
+template <typename T, int LAYOUT, bool NT = false>
+RMX_DEV void store_packed_coalesced_any(uint32_t *slab, int grp0, int l, int L, int xs, int tw, T *sample, int H, int W, int y, int x0, const PackedGroup<T> &g) {
+    static_assert(sizeof(T) == 4, "runs of whole dwords per pixel");
+    if constexpr (LAYOUT == RMX_NCHW) {
+#pragma unroll
+        for (int c = 0; c < 3; c++) {
+            T *seg = sample + ((size_t)c * H + y) * W + xs;
+            store_run_coalesced_any<PX, NT>(slab, reinterpret_cast<uint8_t *>(seg), grp0, l, L, x0 - xs, tw, &g.w[c * PX]);
+        }
+    } else {
+        T *seg = sample + ((size_t)y * W + xs) * 3;
+        store_run_coalesced_any<PX * 3, NT>(slab, reinterpret_cast<uint8_t *>(seg), grp0, l, L, 3 * (x0 - xs), 3 * tw, g.w);
+    }
+}
+
 // Write one lane's group of N horizontally adjacent pixels (v[c][k], k-th pixel of the group)
 // to output row y starting at column x0. `cnt` pixels are valid. When `rev` the group is
 // written in reversed pixel order (horizontal mirror): pixel k goes to column x0 + cnt-1-k.

@@ -14,7 +14,10 @@
 // a row is moved left until it is whole (it then recomputes up to seven pixels of its neighbour and stores the same values to
 // the same places), and a group leaves as 16-byte stores at the element's own alignment. 128 crops of 299 x 299 to fp16
 // planes: 30.4 us through the general path (row by row, element-wise stores for the short group, which cost the whole
-// wavefront), 20 us at 296 or 304.
+// wavefront), 22 us in this form, 20 us at 296 or 304. fp32 rows pass through the LDS slab as in the aligned form and leave as
+// 16-byte pieces at 16-byte aligned addresses (60.3 -> 41.4 us; 32 us at 304). What is left of the difference belongs to the
+// memory system: rows whose pitch is no multiple of a cache line share lines with their neighbours (the aligned form itself
+// takes 23.0 instead of 16.7 us for 224-pixel fp32 rows at a pitch of 232).
 #include "rmx_device.h"
 #include "rmx_launch.h"
 
@@ -31,7 +34,7 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
     constexpr bool FAST = MODE != CMN_GENERAL;
     constexpr bool ANY = MODE == CMN_FAST_ANY;
     // LDS slab through which the lanes of a row exchange their runs before storing (see store_packed_coalesced)
-    constexpr bool COALESCE = MODE == CMN_FAST && coalesce_pays<T, LAYOUT>();
+    constexpr bool COALESCE = (MODE == CMN_FAST && coalesce_pays<T, LAYOUT>()) || (ANY && sizeof(T) == 4);
     uint32_t *slab = nullptr;
     if constexpr (COALESCE) {
         __shared__ __attribute__((aligned(16))) uint32_t slabs[4 * RMX_WAVE * coalesce_slab_dwords<T, LAYOUT>()];
@@ -110,8 +113,9 @@ __global__ void __launch_bounds__(256) rmx_cmn_kernel(RmxKArgs a) {
                 }
                 PackedGroup<T> packed;
                 pack_group<T, LAYOUT>(v, hf, packed);
-                if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT, RMX_K1_NT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
-                else store_packed<T, LAYOUT, RMX_K1_NT && !(ANY && sizeof(T) == 4), ANY>(dimg, a.dst_h, a.dst_w, r, gx, packed);
+                if constexpr (COALESCE && ANY) store_packed_coalesced_any<T, LAYOUT, RMX_K1_NT>(slab, lane - g, g, L, min(xt, cw - PX), xt + tw - min(xt, cw - PX), dimg, a.dst_h, a.dst_w, r, gx, packed);  // (a tile narrower than 8 pixels: its one group reaches back into the tile before)
+                else if constexpr (COALESCE) store_packed_coalesced<T, LAYOUT, RMX_K1_NT>(slab, lane - g, g, L, dimg, a.dst_h, a.dst_w, r, gx, packed);
+                else store_packed<T, LAYOUT, RMX_K1_NT, ANY>(dimg, a.dst_h, a.dst_w, r, gx, packed);
             };
             // every wide load of this wavefront's strip stays inside the batch buffer (the first and the last row bound the rest)
             bool lane_safe = true;
