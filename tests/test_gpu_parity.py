@@ -469,3 +469,42 @@ def test_rows_of_every_small_width_through_the_pipelined_forms(ctx, w):
     got = _cpu(out, ctx)
     for i in range(n):
         assert np.array_equal(got[i, :, :dh[i]].view(np.uint16), exp[i, :, :dh[i]].view(np.uint16)), "resize w=%d sample %d" % (w, i)
+
+
+@pytest.mark.parametrize("w", [513, 515, 519, 1031])
+def test_rows_wider_than_a_tile_with_a_narrow_rest(ctx, w):
+    """Rows one tile of 512 pixels (64 lanes x 8) and 1 .. 7 pixels wide: the rest's single group reaches back into the tile
+    before it. CropMirrorNormalize in every format (fp32 runs pass through the LDS slab) and ColorTwist, mirrored and not."""
+    rng = np.random.default_rng(700 + w)
+    n, H, W = 3, 12, w + 9
+    img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+    src = _gpu(img)
+    sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
+    mirror = np.array([0, 1, 1], np.uint32)
+    scale, bias = _mean_std(n)
+    crop = np.array([[0, 0, w, 12], [9, 1, w, 10], [4, 0, w, 7]], np.uint32)
+    for layout in (ops.NCHW, ops.NHWC):
+        for dtype in (ops.FP16, ops.FP32, ops.UINT8):
+            norm = dtype != ops.UINT8
+            sc, bi = (scale, bias) if norm else (np.ones(3 * n, np.float32), np.zeros(3 * n, np.float32))
+            exp = orc.crop_mirror_normalize(img, crop, sc, bi, mirror, 12, w, layout, dtype)
+            op = ops.CropMirrorNormalize(ctx, sd, ops.desc(n, 12, w, layout, dtype))
+            op.update(crop, sc, bi, mirror)
+            out = op.alloc_output()
+            op.launch(src, out)
+            got = _cpu(out, ctx)
+            for i in range(n):
+                hh = int(crop[i, 3])
+                a, b = (got[i, :, :hh], exp[i, :, :hh]) if layout == ops.NCHW else (got[i, :hh], exp[i, :hh])
+                assert np.array_equal(a.view(np.uint8), b.view(np.uint8)), "cmn w=%d layout=%d dtype=%d sample %d" % (w, layout, dtype, i)
+    alpha, beta = np.full(n, 1.2, np.float32), np.full(n, 4.0, np.float32)
+    hue, sat = np.array([0, 40, 200], np.float32), np.array([1.0, 0.5, 1.5], np.float32)
+    exp = orc.color_twist(img, crop, alpha, beta, hue, sat)
+    op = ops.ColorTwist(ctx, sd, sd)
+    op.update(crop, alpha, beta, hue, sat)
+    out = op.alloc_output()
+    op.launch(src, out)
+    got = _cpu(out, ctx)
+    for i in range(n):
+        hh = int(crop[i, 3])
+        assert np.array_equal(got[i, :hh, :w], exp[i, :hh, :w]), "twist w=%d sample %d" % (w, i)
