@@ -357,7 +357,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->warp_wpb = tune_env("RMX_TUNE_WARP_WPB", ctx->warp_wpb, 1, 4);
         ctx->tri_ring = tune_env("RMX_TUNE_TRI_RING", ctx->tri_ring, 0, 1);  // 1: always the ring kernel
         ctx->tri_tpx = tune_env("RMX_TUNE_TRI_TPX", ctx->tri_tpx, 1, 2);     // output columns per lane of the downscaling kernel
-        ctx->tri_slots = tune_env("RMX_TUNE_TRI_SLOTS", ctx->tri_slots, 0, 4);  // 4: the streaming triangular kernel always keeps four rows in flight
+        ctx->tri_slots = tune_env("RMX_TUNE_TRI_SLOTS", ctx->tri_slots, 0, 4);  // 4: the streaming triangular kernel always keeps four rows in flight (batches that need eight go to the ring kernel)
         ctx->deal_xcd = tune_env("RMX_TUNE_DEAL_XCD", ctx->deal_xcd, 0, 1);  // samples dealt round-robin to the XCDs (0: eight runs in batch order)
         ctx->tri_per_cu = tune_env("RMX_TUNE_TRI_PER_CU", ctx->tri_per_cu, 0, 32);  // wavefronts per CU the strip planner counts on (0: by registers and LDS)
     }
@@ -870,14 +870,19 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         // Downscaling variant: no ring. Usable when every sample shrinks vertically, has at most 8 horizontal
         // taps, and no source row is read by output rows more than three apart (four rows are in flight):
         // first row of r+4 strictly below the last row of r, evaluated with the kernel's own fp32 law.
+        // A sample that grows vertically (two taps, several output rows per source row) needs eight rows in flight, which
+        // the streaming form has for ratios from about 0.26 on: first row of r+8 strictly below the last row of r.
         bool down = kx_cap <= 8 && !op->ctx->tri_ring;
+        int flight = 4;  // rows in flight the batch needs
         for (int i = 0; i < op->n && down; i++) {
             const RmxSample &s = t[i];
             if (s.dst_w <= 0 || s.dst_h <= 0) continue;
-            if (!(s.ry >= 1.0f)) {
+            if (!(s.ry > 0.0f)) {  // (also a NaN)
                 down = false;
                 break;
             }
+            const int apart = s.ry >= 1.0f ? 4 : 8;
+            flight = std::max(flight, apart);
             const float radius = s.ry > 1.0f ? s.ry : 1.0f;
             const float offset = (s.ry - 1) * 0.5f - radius;
             const int ksz = (int)std::ceil(radius * 2);
@@ -888,19 +893,19 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 raw = raw + (float)ylo;
                 return (int)std::ceil(raw);
             };
-            if (s.dst_h <= 4) continue;
-            // Interior rows: the first taps of rows four apart lie at least floor(4*ry - rounding slack) source rows
+            if (s.dst_h <= apart) continue;
+            // Interior rows: the first taps of rows `apart` apart lie at least floor(apart*ry - rounding slack) source rows
             // apart, which must reach past the ksz taps of the upper row. At the window's ends the clamp can fold two
-            // rows onto the same source row: that happens exactly when row 4 starts at or above the first source row,
-            // or the last-but-four row's taps reach the last one (first taps are monotone in the row index).
+            // rows onto the same source row: that happens exactly when row `apart` starts at or above the first source
+            // row, or the taps of the last row but `apart` reach the last one (first taps are monotone in the row index).
             const double slack = 8.0 * 5.9604645e-8 * (double)(s.src_y + s.src_h + 2);
-            if ((int)std::floor(4.0 * (double)s.ry - slack) >= ksz) {
-                down = loc_of(4) > ylo && loc_of(s.dst_h - 5) + ksz - 1 < yhi;
+            if ((int)std::floor((double)apart * (double)s.ry - slack) >= ksz) {
+                down = loc_of(apart) > ylo && loc_of(s.dst_h - apart - 1) + ksz - 1 < yhi;
                 continue;
             }
-            for (int r = 0; r + 4 < s.dst_h && down; r++) {  // ratios just above 1: walk the rows
+            for (int r = 0; r + apart < s.dst_h && down; r++) {  // ratios just above 1 or just above 1/4: walk the rows
                 const int last = std::max(std::min(loc_of(r) + ksz - 1, yhi), ylo);
-                const int first = std::max(std::min(loc_of(r + 4), yhi), ylo);
+                const int first = std::max(std::min(loc_of(r + apart), yhi), ylo);
                 down = first > last;
             }
         }
@@ -910,6 +915,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         // coefficients must leave room for ten wavefronts per CU at least.
         op->tri_rows_in_flight = 0;
         bool tdma = down && op->ctx->dma && op->ctx->tri_tpx == 2 && ky <= 16;
+        if (flight > 4 && (!tdma || op->ctx->tri_slots == 4)) down = tdma = false;  // (only the streaming form has eight)
         if (tdma) {
             if (op->layout.empty()) tdma = (op->src.w * 3u) % 4u == 0;
             else
@@ -947,7 +953,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             }
             // ring of four source rows (six were measured: 18 instead of 20 wavefronts per CU, a fifth slower) + vertical
             // coefficients: 64 source rows and 16 passes x 4 slots
-            const size_t lds = 4 * pitch_max + (64 + 16) * 4 * 4;
+            const size_t lds = 4 * pitch_max + (64 + 16) * (size_t)flight * 4;
             if (lds > 16 * 1024) tdma = false;
             if (tdma) {
                 // Two output rows in flight instead of four when rows two apart never read the same source row. That holds
@@ -956,7 +962,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                 // 2 x ratio = taps rows apart, and only the clamp at the window's ends could fold two such rows onto one
                 // source row: when row 2 starts at or above the first source row, or the taps of the last row but two
                 // reach the last one.
-                bool two = op->ctx->tri_slots != 4;
+                bool two = op->ctx->tri_slots != 4 && flight == 4;
                 for (int i = 0; i < op->n && two; i++) {
                     const RmxSample &s = t[i];
                     if (s.dst_w <= 0 || s.dst_h <= 2) continue;
@@ -977,11 +983,12 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
                     };
                     two = loc_of(2) > ylo && loc_of((int)s.dst_h - 3) + ksz - 1 < yhi;
                 }
-                op->fn = rmx::select_resize_tri_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, two ? 2 : 4, &op->kernel_name);
+                op->tri_rows_in_flight = two ? 2 : flight;
+                op->fn = rmx::select_resize_tri_dma_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, op->tri_rows_in_flight, &op->kernel_name);
                 op->lds_per_wave = (int)lds;
-                op->tri_rows_in_flight = two ? 2 : 4;
             }
         }
+        if (!tdma && flight > 4) down = false;  // (the kernel that stages through registers keeps four rows in flight)
         if (down && !tdma) {
             tile_w = 64 * op->ctx->tri_tpx;
             op->fn = rmx::select_resize_tri_down_kernel(op->dst.dtype, op->dst.layout, op->norm, op->quant, op->ctx->tri_tpx, &op->kernel_name);
@@ -1011,7 +1018,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             if (op->ctx->tri_rows == 0) {
                 // (wavefronts per CU: 16 by the registers of the kernel that stages through registers, 20 by those of the streaming
                 // one, 24 when it keeps two rows in flight)
-                const int by_regs = tdma ? (op->tri_rows_in_flight == 2 ? 24 : 20) : 16;
+                const int by_regs = tdma ? (op->tri_rows_in_flight == 2 ? 24 : (op->tri_rows_in_flight == 8 ? 16 : 20)) : 16;
                 const int per_cu = op->ctx->tri_per_cu > 0 ? op->ctx->tri_per_cu : std::max(1, std::min(by_regs, (160 * 1024) / op->lds_per_wave));
                 const long slots = (long)op->ctx->num_cus * per_cu;
                 double best_cost = 0.0;

@@ -219,6 +219,55 @@ def test_odd_whole_horizontal_ratios_skip_their_first_tap(ctx, ctx_staged, rx):
         _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 9, "rx=%d %s" % (rx, op.kernel_name))
 
 
+@pytest.mark.parametrize("layout,dtype", [(ops.NCHW, ops.FP16), (ops.NHWC, ops.UINT8), (ops.NCHW, ops.FP32)])
+@pytest.mark.parametrize("rows", [0, 7])
+def test_windows_that_grow_keep_eight_rows_in_flight(ctx, ctx_four_rows, layout, dtype, rows):
+    """A batch of windows some of which shrink and some of which grow (vertical ratios 0.28 .. 2.6, as RandomResizedCrop makes
+    them): the streaming kernel keeps eight output rows in flight. Windows at the top and at the bottom of the source (the
+    clamp), mirrored, growing in one direction and shrinking in the other; against the oracle and, bit for bit, against the
+    ring kernel. A window that grows by more than the eight rows allow sends the batch to the ring kernel."""
+    from conftest import _ctx_with_env
+    c = _ctx_with_env(RMX_TUNE_TRI_ROWS=rows) if rows else ctx
+    rng = np.random.default_rng(8100 + 10 * layout + dtype + rows)
+    n, H, W, OH, OW = 7, 160, 200, 64, 96
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    roi = np.array([[0, 0, W, H], [4, 0, 40, 18], [100, H - 23, 96, 23], [8, 30, 150, 29], [0, 100, 30, 60], [60, 0, 131, 58], [20, 10, 27, 150]], np.uint32)
+    dw = np.array([OW, 96, 88, 41, 96, 96, 80], np.uint32)
+    dh = np.array([OH, 64, 64, 64, 57, 64, 58], np.uint32)    # vertical ratios 2.5, 0.28, 0.36, 0.45, 1.05, 0.91, 2.59
+    mirror = np.array([0, 1, 0, 1, 1, 0, 1], np.uint32)
+    scale, bias = _scale_bias(n)
+    norm = dtype != ops.UINT8
+    kw = dict(interp=orc.TRIANGULAR, mirror=mirror, scale=scale if norm else None, bias=bias if norm else None, layout=layout, dtype=dtype)
+    exp = orc.resize(img, roi, dw, dh, OH, OW, **kw)
+    sd, dd = ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, layout, dtype)
+    src = _gpu(img)
+
+    def run(cx, r, h):
+        op = ops.Resize(cx, sd, dd, ops.TRIANGULAR)
+        if norm:
+            op.update_cmn(r, dw, h, scale, bias, mirror)
+        else:
+            op.update(r, dw, h, mirror)
+        out = op.alloc_output(fill=4)
+        op.launch(src, out)
+        cx.sync()
+        return op, out.cpu().numpy()
+
+    op, got = run(c, roi, dh)
+    assert op.kernel_name == "rmx_resize_tri_dma_kernel" and "rows_in_flight=8" in op.plan, op.plan
+    _check_windows(got, exp, dw, dh, layout, 4, "eight rows (%s)" % op.plan)
+    op4, got4 = run(ctx_four_rows, roi, dh)
+    assert op4.kernel_name == "rmx_resize_tri_kernel", op4.plan
+    assert np.array_equal(_bits(got), _bits(got4))
+    roi2 = roi.copy()
+    roi2[1, 3] = 12                                            # 12 rows to 64: ratio 0.19
+    op2, got2 = run(c, roi2, dh)
+    assert op2.kernel_name == "rmx_resize_tri_kernel", op2.plan
+    _check_windows(got2, orc.resize(img, roi2, dw, dh, OH, OW, **kw), dw, dh, layout, 4, "ring kernel")
+    if rows:
+        c.close()
+
+
 def test_more_than_sixteen_vertical_taps_take_the_other_kernel(ctx):
     rng = np.random.default_rng(3)
     n, H, W = 1, 400, 64
