@@ -9,11 +9,19 @@
 // with a reader + decoder, this API takes decoded batches that already sit in device memory:
 //   rocalDeviceSource()      declares the input tensor (u8 RGB, NHWC, padded to max_height x max_width)
 //   rocalDeviceSourceFeed()  hands the next batch: device pointer + per-sample width/height
-// and an output is read through rocalTensorBuffer() / rocalTensorRoi(), or written straight into memory the caller owns
-// (rocalTensorSetBuffer, e.g. the data pointer of a torch tensor).
+// and an output is read as in the reference, through rocalGetOutputTensors(ctx)->at(i)->copy_data(...) / ->buffer() /
+// ->copy_roi(...) (rocal_api_tensor.h:38-93, rocal_api_data_transfer.h:43,83), or written straight into memory the caller owns
+// (rocalTensor::set_mem_handle / rocalTensorSetBuffer, e.g. the data pointer of a torch tensor).
+//
+// rocalRun() enqueues the batch on the context's stream and returns; the wait for it is where the consumer takes the
+// result: rocalGetOutputTensors, rocalTensor::copy_data / buffer, rocalCopyToOutput, rocalToTensor and rocalTensorBuffer
+// return only when the batch is complete (the reference separates producer and consumer the same way, through its output
+// ring buffer: ring_buffer.cpp:118-119, master_graph.cpp:1019-1043). A consumer that works on a HIP stream of its own
+// can make that stream wait instead of the host: rocalOutputsWaitOnStream.
 #ifndef ROCAL_API_MI355X_H
 #define ROCAL_API_MI355X_H
 #include <cstddef>
+#include <cstdint>
 #include <vector>
 
 // rocAL/include/api/rocal_api_types.h:326-366
@@ -36,16 +44,60 @@ enum RocalResizeInterpolationType {
 #define ROCAL_API_CALL __attribute__((visibility("default")))
 
 typedef void *RocalContext;
-typedef void *RocalTensor;
 typedef void *RocalFloatParam;
 typedef void *RocalIntParam;
 
-// rocAL/include/api/rocal_api_types.h:112-128,151-158,208-268
+// rocAL/include/api/rocal_api_types.h:112-128,151-158,208-268,372-391
 enum RocalStatus { ROCAL_OK = 0, ROCAL_CONTEXT_INVALID, ROCAL_RUNTIME_ERROR, ROCAL_UPDATE_PARAMETER_FAILED, ROCAL_INVALID_PARAMETER_TYPE };
 enum RocalProcessMode { ROCAL_PROCESS_GPU = 0, ROCAL_PROCESS_CPU = 1 };
 enum RocalTensorLayout { ROCAL_NHWC = 0, ROCAL_NCHW = 1, ROCAL_NONE = 9 };
 enum RocalTensorOutputType { ROCAL_FP32 = 0, ROCAL_FP16 = 1, ROCAL_UINT8 = 2 };
 enum RocalOutputMemType { ROCAL_MEMCPY_HOST = 0, ROCAL_MEMCPY_GPU = 1, ROCAL_MEMCPY_PINNED = 2 };
+enum RocalTensorBackend { ROCAL_CPU = 0, ROCAL_GPU = 1 };
+enum class RocalROICordsType { ROCAL_LTRB = 0, ROCAL_XYWH = 1 };
+
+/* ---- tensors (rocAL/include/api/rocal_api_tensor.h:38-93): the reference's abstract classes, member for member. Every
+   augmentation entry point takes and returns a RocalTensor; the tensors of a context live until rocalRelease.
+     buffer()         device address of the tensor's batch (waits for the batch that is being computed);
+     copy_data(p, t)  copies data_size() bytes to p: device memory for ROCAL_MEMCPY_GPU, host (pageable or pinned) memory for
+                      ROCAL_MEMCPY_HOST / ROCAL_MEMCPY_PINNED; returns 0 (tensor.cpp:419-454);
+     copy_data(p, x, y, cols, rows)  the window at (x, y) of every sample's first plane, densely packed, to host memory
+                      (tensor.cpp:456-476 reads host memory there; this build copies from the device);
+     dims()/strides() in the order of the layout ({N,H,W,C} or {N,C,H,W}), strides in bytes (tensor.h:250-255);
+     shape()          {max_width, max_height};  copy_roi(p): 4 unsigned per sample, x y w h (get_roi_dims_size() == 2);
+     set_mem_handle(p) the node that produces the tensor writes to p from the next run on (16-byte aligned device memory). ---- */
+class rocalTensor {
+   public:
+    virtual ~rocalTensor() = default;
+    virtual void *buffer() = 0;
+    virtual unsigned copy_data(void *user_buffer, RocalOutputMemType external_mem_type = ROCAL_MEMCPY_HOST) = 0;
+    virtual unsigned copy_data(void *user_buffer, unsigned int x_offset, unsigned int y_offset, unsigned int max_cols, unsigned int max_rows) = 0;
+    virtual unsigned num_of_dims() = 0;
+    virtual unsigned batch_size() = 0;
+    virtual std::vector<size_t> dims() = 0;
+    virtual std::vector<size_t> strides() = 0;
+    virtual RocalTensorLayout layout() = 0;
+    virtual RocalTensorBackend backend() = 0;
+    virtual RocalTensorOutputType data_type() = 0;
+    virtual RocalOutputMemType mem_type() = 0;
+    virtual size_t data_size() = 0;
+    virtual RocalROICordsType roi_type() = 0;
+    virtual size_t get_roi_dims_size() = 0;
+    virtual void copy_roi(void *roi_buffer) = 0;
+    virtual std::vector<size_t> shape() = 0;
+    virtual void set_dims(std::vector<size_t> dims) = 0;
+    virtual void set_mem_handle(void *buffer) = 0;
+    virtual void set_tensor_layout(RocalTensorLayout layout) = 0;
+    virtual uint64_t data_type_size() = 0;
+};
+class rocalTensorList {
+   public:
+    virtual ~rocalTensorList() = default;
+    virtual uint64_t size() = 0;
+    virtual rocalTensor *at(size_t index) = 0;
+};
+typedef rocalTensor *RocalTensor;
+typedef rocalTensorList *RocalTensorList;
 
 /* ---- context (rocal_api.h:83-110). Only ROCAL_PROCESS_GPU exists: there is no CPU path. ---- */
 extern "C" RocalContext ROCAL_API_CALL rocalCreate(size_t batch_size, RocalProcessMode affinity, int gpu_id = 0, size_t cpu_thread_count = 1,
@@ -54,6 +106,11 @@ extern "C" RocalStatus ROCAL_API_CALL rocalVerify(RocalContext context);
 extern "C" RocalStatus ROCAL_API_CALL rocalRun(RocalContext context);
 extern "C" RocalStatus ROCAL_API_CALL rocalRelease(RocalContext context);
 extern "C" const char *ROCAL_API_CALL rocalGetErrorMessage(RocalContext context);
+// Which neighbour the bilinear kernels take at the right / lower edge of a source window (no counterpart in the reference's
+// API; call it before the first resize node is added). 0, the default: the last pixel of the window (the textbook rule).
+// 1: the last-but-one, as the reference's own device kernel clamps (rocAL/rocAL_hip/rocal_hip_kernels.cpp:339-345,356-362).
+// The environment variable ROCAL_BILINEAR_EDGE (0 / 1, or "device") sets the default that rocalCreate starts from.
+extern "C" RocalStatus ROCAL_API_CALL rocalSetBilinearEdgeRule(RocalContext context, int device_rule);
 
 /* ---- timing (rocal_api_info.h:106, rocal_api_types.h:79-84): microseconds accumulated since the last call, which resets them.
    process_time brackets Graph::process() as the reference's does (master_graph.cpp:1015-1017): the launches of a batch and the
@@ -89,6 +146,12 @@ extern "C" RocalStatus ROCAL_API_CALL rocalPackedSourcePush(RocalContext context
 // returns an error instead of blocking.
 extern "C" RocalStatus ROCAL_API_CALL rocalPackedSourceWait(RocalContext context, RocalTensor source);
 extern "C" size_t ROCAL_API_CALL rocalPackedSourceLevel(RocalContext context, RocalTensor source);
+// Shut-down of the ring, as the reference's loaders do it (image_loader.cpp:84,126-127: unblock_writer / unblock_reader):
+// wakes a loader thread blocked in rocalPackedSourcePlaceImage and a consumer blocked in rocalPackedSourceWait; they and
+// every later caller get an error ("released") instead of a slot. rocalRelease does this for every packed source and frees
+// the slots only when no thread is inside one of these calls any more.
+extern "C" RocalStatus ROCAL_API_CALL rocalPackedSourceStop(RocalContext context, RocalTensor source);
+/* ---- flat getters over the same tensors for callers without C++ (ctypes): extras, not in the reference ---- */
 extern "C" void *ROCAL_API_CALL rocalTensorBuffer(RocalTensor tensor);
 // Binds an output tensor to device memory the caller owns (at least rocalTensorDataSize bytes, 16-byte aligned), before or
 // after rocalVerify and as often as wanted between runs: the node that produces the tensor writes there directly. Stands where
@@ -105,6 +168,16 @@ extern "C" RocalStatus ROCAL_API_CALL rocalTensorInfo(RocalTensor tensor, size_t
 /* ---- tensors the caller wants to read after a run (rocal_api_data_transfer.h:75): called before rocalVerify, as the Python
    pipeline does for what define_graph returns; a tensor created with is_output = true is an output already. ---- */
 extern "C" void ROCAL_API_CALL rocalSetOutputs(RocalContext p_context, unsigned int num_of_outputs, std::vector<RocalTensor> &output_images);
+
+/* ---- results of the last rocalRun (rocal_api_data_transfer.h:43,83). Both wait until the batch is complete.
+   rocalGetOutputTensors: the list of output tensors, owned by the context. rocalCopyToOutput: the single output tensor to
+   host memory, out_size = its data_size() (master_graph.cpp:859-927). ---- */
+extern "C" RocalTensorList ROCAL_API_CALL rocalGetOutputTensors(RocalContext context);
+extern "C" RocalStatus ROCAL_API_CALL rocalCopyToOutput(RocalContext context, unsigned char *out_ptr, size_t out_size);
+// Makes a HIP stream of the caller (hipStream_t as void *, null = the default stream) wait for the batch of the last rocalRun
+// instead of the host: what a framework that consumes the output on its own stream calls (no counterpart in the reference,
+// whose consumer is the host thread).
+extern "C" RocalStatus ROCAL_API_CALL rocalOutputsWaitOnStream(RocalContext context, void *stream);
 
 /* ---- u8 output -> float tensor (rocal_api_data_transfer.h:45-66). out_ptr is device memory: only ROCAL_MEMCPY_GPU exists. ---- */
 extern "C" RocalStatus ROCAL_API_CALL rocalToTensor(RocalContext rocal_context, void *out_ptr, RocalTensorLayout tensor_format,

@@ -23,6 +23,8 @@ _SIGS = {
     "rocalPackedSource": (_vp, [_vp, _u, _u, _b, _u, C.c_size_t]),
     "rocalPackedSourcePlaceImage": (_vp, [_vp, _vp, _u, _u, _u, C.POINTER(_u)]),
     "rocalPackedSourcePush": (_i, [_vp, _vp]), "rocalPackedSourceWait": (_i, [_vp, _vp]), "rocalPackedSourceLevel": (C.c_size_t, [_vp, _vp]),
+    "rocalPackedSourceStop": (_i, [_vp, _vp]), "rocalSetBilinearEdgeRule": (_i, [_vp, _i]), "rocalOutputsWaitOnStream": (_i, [_vp, _vp]),
+    "rocalCopyToOutput": (_i, [_vp, _vp, C.c_size_t]), "rocalpy_output_tensors": (_i, [_vp, _vp, _u]),
     "rocalTensorBuffer": (_vp, [_vp]), "rocalTensorRoi": (C.POINTER(_u), [_vp]), "rocalTensorDataSize": (C.c_size_t, [_vp]),
     "rocalTensorSetBuffer": (_i, [_vp, _vp, _vp]),
     "rocalTensorInfo": (_i, [_vp, C.POINTER(C.c_size_t), C.POINTER(_i), C.POINTER(_i)]),
@@ -98,6 +100,23 @@ class Backend:
 
     def rocalRelease(self, handle):
         return host().rocalRelease(handle)
+
+    def setBilinearEdgeRule(self, handle, device_rule):
+        return host().rocalSetBilinearEdgeRule(handle, 1 if device_rule else 0)
+
+    def getOutputTensors(self, handle):
+        """rocalGetOutputTensors: waits for the batch of the last run and returns the handles of the output tensors."""
+        arr = (C.c_void_p * 64)()
+        n = host().rocalpy_output_tensors(handle, arr, 64)
+        if n < 0:
+            raise RuntimeError("rocalGetOutputTensors failed: " + self.getErrorMessage(handle))
+        return [arr[i] for i in range(n)]
+
+    def outputsWaitOnStream(self, handle, stream):
+        return host().rocalOutputsWaitOnStream(handle, stream)
+
+    def copyToOutput(self, handle, ptr, size):
+        return host().rocalCopyToOutput(handle, ptr, size)
 
     def getErrorMessage(self, handle):
         return host().rocalGetErrorMessage(handle).decode()
@@ -175,6 +194,9 @@ class Backend:
 
     def packedSourceWait(self, handle, source):
         return host().rocalPackedSourceWait(handle, source)
+
+    def packedSourceStop(self, handle, source):
+        return host().rocalPackedSourceStop(handle, source)
 
     def packedSourceLevel(self, handle, source):
         return int(host().rocalPackedSourceLevel(handle, source))

@@ -149,6 +149,13 @@ int check_desc(const rmx_tensor_desc *d, const char *what) {
     return RMX_OK;
 }
 
+// Size of one table slot: n rows, n source layout entries and n side-table entries, rounded up to the 16-byte pieces in
+// which the upload kernel copies it.
+size_t slot_bytes(const rmx_op *op) {
+    const size_t raw = (sizeof(RmxSample) + sizeof(RmxSrcLayout) + op->extra_per_sample) * (size_t)op->n;
+    return (raw + 15) & ~(size_t)15;
+}
+
 int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor_desc *dst, int roi_type, rmx_op **out, size_t extra_per_sample = 0) {
     if (!ctx) return fail(RMX_ERR_INVALID, "context is NULL");
     if (!out) return fail(RMX_ERR_INVALID, "output handle pointer is NULL");
@@ -171,7 +178,8 @@ int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor
     op->roi_type = roi_type;
     op->n = (int)src->n;
     op->extra_per_sample = extra_per_sample;
-    size_t bytes = (sizeof(RmxSample) + sizeof(RmxSrcLayout) + extra_per_sample) * (size_t)op->n;
+    // (the upload kernel moves whole 16-byte pieces: a slot is a whole number of them)
+    const size_t bytes = slot_bytes(op);
     for (int i = 0; i < TABLE_RING; i++) {
         hipError_t e = hipHostMalloc((void **)&op->h_table[i], bytes, hipHostMallocDefault);
         if (e == hipSuccess) e = hipMalloc((void **)&op->d_table[i], bytes);
@@ -210,7 +218,8 @@ int commit_slot(rmx_op *op, int slot) {
     // slower, 56.8 -> 73.0 us with a wait per batch and 38.5 -> 41.7 us without, on the RandomResizedCrop batch.)
     hipStream_t us = op->ctx->stream;
     if (op->ctx->upload_kernel) {
-        const int n16 = (int)((bytes + 15) / 16);  // (the slots are allocated in whole rows of 128 bytes and 16-byte entries)
+        const int n16 = (int)((bytes + 15) / 16);
+        if ((size_t)n16 * 16 > slot_bytes(op)) return fail(RMX_ERR_INVALID, "parameter table of %zu bytes exceeds its slot of %zu", bytes, slot_bytes(op));
         hipLaunchKernelGGL(rmx_table_upload_kernel, dim3((unsigned)std::min(8, (n16 + 255) / 256)), dim3(256), 0, us,
                            reinterpret_cast<const uint4 *>(op->h_table[slot]), reinterpret_cast<uint4 *>(op->d_table[slot]), n16);
         HIP_TRY(hipGetLastError());

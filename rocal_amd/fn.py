@@ -186,9 +186,11 @@ def blend(*inputs, ratio=None, device=None, output_layout=types.NHWC, output_dty
 
 
 # ---- fn.py: normalize (axes, mean, stddev, scale, shift) and transpose (perm) on image tensors
-def normalize(*inputs, axes=[], mean=[], stddev=[], scale=1.0, shift=0.0, output_dtype=types.FLOAT):
-    """axes: the reduced axes (0 height, 1 width, 2 channels); empty mean / stddev are computed per sample."""
-    return b.normalize(_handle(), inputs[0], axes, mean, stddev, False, scale, shift, output_dtype)
+def normalize(*inputs, axes=[], mean=[], stddev=[], scale=1.0, shift=0.0, output_datatype=types.FLOAT, output_dtype=None):
+    """axes: the reduced axes (0 height, 1 width, 2 channels); empty mean / stddev are computed per sample.
+    The keyword is `output_datatype` as in the reference (rocAL_pybind/amd/rocal/fn.py:1216); `output_dtype`, the spelling of
+    every other operator, is accepted as well."""
+    return b.normalize(_handle(), inputs[0], axes, mean, stddev, False, scale, shift, output_datatype if output_dtype is None else output_dtype)
 
 
 def transpose(*inputs, perm=[], output_layout=types.NHWC, output_dtype=types.UINT8):

@@ -122,9 +122,25 @@ RocalStatus rocalRun(RocalContext p_context) {
     return ROCAL_OK;
 }
 
+// Loader threads blocked on a packed source are woken and turned away first (image_loader.cpp:84,126-127); the
+// destructor of the graph frees the rings only when they have left.
 RocalStatus rocalRelease(RocalContext p_context) {
     if (!p_context) return ROCAL_CONTEXT_INVALID;
-    delete static_cast<Context *>(p_context);
+    auto *context = static_cast<Context *>(p_context);
+    context->master_graph->stop_sources();
+    delete context;
+    return ROCAL_OK;
+}
+
+RocalStatus rocalSetBilinearEdgeRule(RocalContext p_context, int device_rule) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->set_edge_rule(device_rule != 0);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
     return ROCAL_OK;
 }
 
@@ -206,11 +222,25 @@ RocalStatus rocalPackedSourcePush(RocalContext p_context, RocalTensor p_source) 
     return ROCAL_OK;
 }
 
+RocalStatus rocalPackedSourceStop(RocalContext p_context, RocalTensor p_source) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->packed_buffer(static_cast<Tensor *>(p_source))->stop();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
 RocalStatus rocalPackedSourceWait(RocalContext p_context, RocalTensor p_source) {
     if (!p_context) return ROCAL_CONTEXT_INVALID;
     auto *context = static_cast<Context *>(p_context);
     try {
-        context->master_graph->packed_buffer(static_cast<Tensor *>(p_source))->block_if_empty();
+        PackedCircularBuffer *ring = context->master_graph->packed_buffer(static_cast<Tensor *>(p_source));
+        ring->block_if_empty();
+        if (ring->stopped()) THROW("the packed batch buffer was released")
     } catch (const std::exception &e) {
         report(context, e);
         return ROCAL_RUNTIME_ERROR;
@@ -282,9 +312,53 @@ long long unsigned rocalGetParameterUpdateTime(RocalContext p_context) {
     return r;
 }
 
-void *rocalTensorBuffer(RocalTensor t) { return t ? static_cast<Tensor *>(t)->buffer() : nullptr; }
+void *rocalTensorBuffer(RocalTensor t) {
+    try {
+        return t ? t->buffer() : nullptr;  // (waits for the batch that is being computed)
+    } catch (const std::exception &e) {
+        std::cerr << e.what() << std::endl;
+        return nullptr;
+    }
+}
 const unsigned *rocalTensorRoi(RocalTensor t) { return t ? reinterpret_cast<const unsigned *>(static_cast<Tensor *>(t)->info().roi()) : nullptr; }
 size_t rocalTensorDataSize(RocalTensor t) { return t ? static_cast<Tensor *>(t)->info().data_size() : 0; }
+
+/* ------------------------------------------------------------------ results (rocal_api_data_transfer.cpp:54-68,110-121) */
+
+RocalTensorList rocalGetOutputTensors(RocalContext p_context) {
+    if (!p_context) return nullptr;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        return context->master_graph->get_output_tensors();
+    } catch (const std::exception &e) {
+        report(context, e);
+        return nullptr;
+    }
+}
+
+RocalStatus rocalCopyToOutput(RocalContext p_context, unsigned char *out_ptr, size_t out_size) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->copy_output(out_ptr, out_size);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
+
+RocalStatus rocalOutputsWaitOnStream(RocalContext p_context, void *stream) {
+    if (!p_context) return ROCAL_CONTEXT_INVALID;
+    auto *context = static_cast<Context *>(p_context);
+    try {
+        context->master_graph->outputs_wait_on_stream(stream);
+    } catch (const std::exception &e) {
+        report(context, e);
+        return ROCAL_RUNTIME_ERROR;
+    }
+    return ROCAL_OK;
+}
 
 /* ------------------------------------------------------------------ output conversion (rocal_api_data_transfer.cpp:30-52) */
 

@@ -1,9 +1,12 @@
 // Test driver of the host layer, run by the test-suite as a child process.
 //   host_check params <seed>            prints, as JSON, what the parameter system produces (no GPU needed)
+//   host_check ring                      the shut-down protocol of the loader ring on a ring in host memory (no GPU needed)
 //   host_check pipeline <scenario> <dir> builds a pipeline through the rocal* API, feeds <dir>/input.bin
 //                                        twice and writes every output batch + ROI to <dir> (needs the GPU)
 #include <hip/hip_runtime_api.h>
 
+#include <atomic>
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -11,6 +14,7 @@
 #include <iostream>
 #include <sstream>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "rocal_host.h"
@@ -353,9 +357,102 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
 
 }  // namespace
 
+// A loader thread blocked on a full ring must leave with an exception when the ring is stopped or released, never with a
+// slot that is still full; release() must not free the slots before the thread has left. Prints one line per check.
+int run_ring() {
+    auto fill = [](PackedCircularBuffer &ring, unsigned char v) {
+        for (size_t i = 0; i < 2; i++) {
+            uint32_t stride = 0;
+            unsigned char *p = ring.place_image(i, 5, 3, &stride);
+            if (stride != 16) throw std::runtime_error("row stride");
+            memset(p, v, (size_t)stride * 3);
+        }
+        ring.push();
+    };
+    bool ok = true;
+    auto say = [&](const char *what, bool good) {
+        std::cout << what << " " << (good ? "ok" : "FAILED") << std::endl;
+        ok = ok && good;
+    };
+    for (int how = 0; how < 3; how++) {  // 0: stop(), 1: release(), 2: unblock_writer() while the ring stays full
+        PackedCircularBuffer ring(-1, nullptr);
+        ring.init(2, 4096, 3);  // depth 3: two batches fill it (the third spot is the reader's)
+        fill(ring, 1);
+        fill(ring, 2);
+        say("level_after_two_pushes", ring.level() == 2);
+        std::atomic<int> state{0};  // 1: about to block, 2: left with an exception, 3: was handed a slot
+        std::string message;
+        std::thread loader([&] {
+            state = 1;
+            try {
+                uint32_t stride = 0;
+                ring.place_image(0, 5, 3, &stride);
+                state = 3;
+            } catch (const std::exception &e) {
+                message = e.what();
+                state = 2;
+            }
+        });
+        while (state.load() == 0) std::this_thread::yield();
+        std::this_thread::sleep_for(std::chrono::milliseconds(50));
+        say("loader_blocked_on_full_ring", state.load() == 1);
+        const auto t0 = std::chrono::steady_clock::now();
+        if (how == 0) ring.stop();
+        else if (how == 1) ring.release();
+        else ring.unblock_writer();
+        loader.join();
+        const double ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+        say(how == 0 ? "stop_wakes_loader" : how == 1 ? "release_wakes_loader" : "unblock_without_room_is_an_error", state.load() == 2 && ms < 1000.0);
+        say("message", message.find(how == 2 ? "full" : "released") != std::string::npos);
+        if (how == 0) {
+            bool threw = false;
+            try {
+                ring.get_read_buffer_dev();
+            } catch (const std::exception &) {
+                threw = true;
+            }
+            say("reader_turned_away_after_stop", threw);
+            ring.reset();  // a new epoch: the ring takes batches again
+            fill(ring, 3);
+            say("ring_usable_after_reset", ring.level() == 1 && static_cast<unsigned char *>(ring.get_read_buffer_dev())[0] == 3);
+            ring.pop();
+        }
+        if (how == 2) {
+            // the reader's side still holds both batches, oldest first
+            say("oldest_batch_intact", static_cast<unsigned char *>(ring.get_read_buffer_dev())[0] == 1);
+            ring.pop();
+            fill(ring, 4);  // room again
+            say("writer_continues_after_pop", ring.level() == 2);
+        }
+    }
+    {
+        // a consumer blocked on an empty ring is woken the same way
+        PackedCircularBuffer ring(-1, nullptr);
+        ring.init(2, 4096, 2);
+        std::atomic<int> state{0};
+        std::thread reader([&] {
+            state = 1;
+            try {
+                ring.get_read_buffer_dev();
+                state = 3;
+            } catch (const std::exception &) {
+                state = 2;
+            }
+        });
+        while (state.load() == 0) std::this_thread::yield();
+        std::this_thread::sleep_for(std::chrono::milliseconds(50));
+        ring.release();
+        reader.join();
+        say("release_wakes_reader", state.load() == 2);
+    }
+    std::cout << (ok ? "ring ok" : "ring FAILED") << std::endl;
+    return ok ? 0 : 1;
+}
+
 int main(int argc, char **argv) {
+    if (argc >= 2 && !strcmp(argv[1], "ring")) return run_ring();
     if (argc >= 3 && !strcmp(argv[1], "params")) return run_params((unsigned)strtoul(argv[2], nullptr, 10));
     if (argc >= 4 && !strcmp(argv[1], "pipeline")) return run_pipeline(argv[2], argv[3]);
-    std::cerr << "usage: host_check params <seed> | pipeline <scenario> <dir>" << std::endl;
+    std::cerr << "usage: host_check params <seed> | ring | pipeline <scenario> <dir>" << std::endl;
     return 1;
 }

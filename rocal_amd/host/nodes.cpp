@@ -211,7 +211,8 @@ bool ResizeFamilyNode::try_absorb_chain(Node *colour, Node *next) {
 void ResizeFamilyNode::create_resize_op(int interpolation) {
     const TensorInfo &out = (_absorbed ? _absorbed->output()[0] : _outputs[0])->info();
     rmx_tensor_desc s = _inputs[0]->info().desc(), d = out.desc();
-    const uint32_t flags = (_absorbed ? RMX_F_QUANTIZE_U8 : 0) | (_absorbed_colour ? _absorbed_colour->chain_colour_kind() : 0);
+    const uint32_t flags = (_absorbed ? RMX_F_QUANTIZE_U8 : 0) | (_absorbed_colour ? _absorbed_colour->chain_colour_kind() : 0) |
+                           (_graph->edge_device_rule ? RMX_F_EDGE_REF : 0);
     check(rmx_create_resize(_graph->get(), &s, &d, interpolation, (int)RocalROIType::XYWH, flags, &_node), "rmx_create_resize");
 }
 
@@ -243,8 +244,8 @@ void ResizeFamilyNode::update_resize_op(const std::vector<uint32_t> &window, con
 
 void ResizeFamilyNode::launch() {
     Tensor *in = _inputs[0], *out = _absorbed ? _absorbed->output()[0] : _outputs[0];
-    if (!in->buffer() || !out->buffer()) THROW("tensor without a device buffer at launch")
-    check(rmx_op_launch(_node, in->buffer(), out->buffer()), "rmx_op_launch");
+    if (!in->handle() || !out->handle()) THROW("tensor without a device buffer at launch")
+    check(rmx_op_launch(_node, in->handle(), out->handle()), "rmx_op_launch");
 }
 
 void ResizeFamilyNode::adjust_out_roi_size(unsigned src_w, unsigned src_h, unsigned &dst_w, unsigned &dst_h, RocalResizeScalingMode mode, unsigned max_w,
@@ -755,8 +756,8 @@ void BlendNode::update_node() {
 
 void BlendNode::launch() {
     Tensor *in1 = _inputs[0], *in2 = _inputs[1], *out = _outputs[0];
-    if (!in1->buffer() || !in2->buffer() || !out->buffer()) THROW("tensor without a device buffer at launch")
-    check(rmx_op_launch2(_node, in1->buffer(), in2->buffer(), out->buffer()), "rmx_op_launch2");
+    if (!in1->handle() || !in2->handle() || !out->handle()) THROW("tensor without a device buffer at launch")
+    check(rmx_op_launch2(_node, in1->handle(), in2->handle(), out->handle()), "rmx_op_launch2");
 }
 
 /* ======================================================================= warp affine / rotate */

@@ -2,6 +2,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include <cstdlib>
+
 #include "exception.h"
 
 #define HIP_OK(call, what)                                                                        \
@@ -12,6 +14,25 @@
 
 PackedCircularBuffer::PackedCircularBuffer(int device, void *consumer_stream) : _device(device), _consumer_stream(consumer_stream) {}
 
+// Counts the calling thread into the ring for the length of a call that touches the slots, and refuses it once the ring
+// is closing: release() frees the slots only when the count is back at 0.
+struct PackedCircularBuffer::Inside {
+    explicit Inside(PackedCircularBuffer &b) : _b(b) {
+        std::unique_lock<std::mutex> lock(_b._lock);
+        if (_b._closing) THROW("the packed batch buffer was released")
+        _b._inside++;
+    }
+    ~Inside() {
+        bool idle;
+        {
+            std::unique_lock<std::mutex> lock(_b._lock);
+            idle = --_b._inside == 0;
+        }
+        if (idle) _b._idle.notify_all();
+    }
+    PackedCircularBuffer &_b;
+};
+
 PackedCircularBuffer::~PackedCircularBuffer() { release(); }
 
 void PackedCircularBuffer::init(size_t batch_size, size_t slot_bytes, size_t buff_depth) {
@@ -21,11 +42,21 @@ void PackedCircularBuffer::init(size_t batch_size, size_t slot_bytes, size_t buf
     _batch_size = batch_size;
     _slot_bytes = (slot_bytes + 255) / 256 * 256;
     _buff_depth = buff_depth;
-    HIP_OK(hipSetDevice(_device), "hipSetDevice");
-    hipStream_t s;
-    HIP_OK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreateWithFlags");
-    _copy_stream = s;
-    for (size_t i = 0; i < buff_depth; i++) {
+    for (size_t i = 0; _device < 0 && i < buff_depth; i++) {
+        void *h = malloc(_slot_bytes);
+        if (!h) THROW("out of host memory for a packed batch slot")
+        _host_buffer_ptrs.push_back(static_cast<unsigned char *>(h));
+        _dev_buffer.push_back(h);
+        _copied.push_back(nullptr);
+        _consumed.push_back(nullptr);
+    }
+    if (_device >= 0) {
+        HIP_OK(hipSetDevice(_device), "hipSetDevice");
+        hipStream_t s;
+        HIP_OK(hipStreamCreateWithFlags(&s, hipStreamNonBlocking), "hipStreamCreateWithFlags");
+        _copy_stream = s;
+    }
+    for (size_t i = 0; _device >= 0 && i < buff_depth; i++) {
         void *h = nullptr, *d = nullptr;
         hipEvent_t a, b;
         // pinned memory is allocated, never registered; 16 spare bytes behind the slot keep the kernels' wide loads inside it
@@ -47,11 +78,41 @@ void PackedCircularBuffer::init(size_t batch_size, size_t slot_bytes, size_t buf
     }
     _placed.assign(batch_size, false);
     _write_pos = 0;
+    _closing = false;
     _initialized = true;
+}
+
+void PackedCircularBuffer::stop() {
+    {
+        std::unique_lock<std::mutex> lock(_lock);
+        _closing = true;
+    }
+    _wait_for_load.notify_all();
+    _wait_for_unload.notify_all();
+}
+
+bool PackedCircularBuffer::stopped() {
+    std::unique_lock<std::mutex> lock(_lock);
+    return _closing;
 }
 
 void PackedCircularBuffer::release() {
     if (!_initialized) return;
+    stop();
+    {
+        // a loader thread that was blocked in place_image() leaves with an exception; the slots stay until it has left
+        std::unique_lock<std::mutex> lock(_lock);
+        _idle.wait(lock, [&] { return _inside == 0; });
+    }
+    if (_device < 0) {
+        for (unsigned char *h : _host_buffer_ptrs) free(h);
+        _host_buffer_ptrs.clear();
+        _dev_buffer.clear();
+        _copied.clear();
+        _consumed.clear();
+        _initialized = false;
+        return;
+    }
     (void)hipSetDevice(_device);
     (void)hipStreamSynchronize(static_cast<hipStream_t>(_copy_stream));
     for (size_t i = 0; i < _buff_depth; i++) {
@@ -71,7 +132,12 @@ void PackedCircularBuffer::release() {
 
 unsigned char *PackedCircularBuffer::get_write_buffer() {
     if (!_initialized) THROW("Circular buffer not initialized")
+    Inside in(*this);
     block_if_full();
+    std::unique_lock<std::mutex> lock(_lock);
+    // woken without room (stop() or unblock_writer()): the slot at the write pointer is still the reader's or the copy's
+    if (_closing) THROW("the packed batch buffer was released")
+    if (full()) THROW("the packed batch buffer is full (the writer was unblocked without a free slot)")
     return _host_buffer_ptrs[_write_ptr];
 }
 
@@ -80,8 +146,9 @@ unsigned char *PackedCircularBuffer::place_image(size_t index, uint32_t width, u
     if (index >= _batch_size) THROW("image index " + TOSTR(index) + " outside the batch of " + TOSTR(_batch_size))
     if (width == 0 || height == 0) THROW("image " + TOSTR(index) + " is empty")
     if (_placed[index]) THROW("image " + TOSTR(index) + " was placed twice in one batch")
+    Inside in(*this);
     unsigned char *base = get_write_buffer();
-    if (_write_pos == 0) {
+    if (_write_pos == 0 && _device >= 0) {
         // first image of a batch: the copy that last read this pinned slot has finished (a consumer that does not wait for
         // its batches can be a whole ring behind the loader)
         HIP_OK(hipSetDevice(_device), "hipSetDevice");
@@ -105,16 +172,19 @@ unsigned char *PackedCircularBuffer::place_image(size_t index, uint32_t width, u
 
 void PackedCircularBuffer::push() {
     if (!_initialized) return;
+    Inside in(*this);
     for (size_t i = 0; i < _batch_size; i++)
         if (!_placed[i]) THROW("push: image " + TOSTR(i) + " of the batch was not placed")
     PackedLayout &l = _layout[_write_ptr];
     l.bytes = _write_pos;
-    HIP_OK(hipSetDevice(_device), "hipSetDevice");
-    auto cs = static_cast<hipStream_t>(_copy_stream);
-    // the kernels that read this device slot the last time round have finished before it is overwritten
-    HIP_OK(hipStreamWaitEvent(cs, static_cast<hipEvent_t>(_consumed[_write_ptr]), 0), "hipStreamWaitEvent");
-    HIP_OK(hipMemcpyAsync(_dev_buffer[_write_ptr], _host_buffer_ptrs[_write_ptr], l.bytes, hipMemcpyHostToDevice, cs), "hipMemcpyAsync of a packed batch");
-    HIP_OK(hipEventRecord(static_cast<hipEvent_t>(_copied[_write_ptr]), cs), "hipEventRecord");
+    if (_device >= 0) {
+        HIP_OK(hipSetDevice(_device), "hipSetDevice");
+        auto cs = static_cast<hipStream_t>(_copy_stream);
+        // the kernels that read this device slot the last time round have finished before it is overwritten
+        HIP_OK(hipStreamWaitEvent(cs, static_cast<hipEvent_t>(_consumed[_write_ptr]), 0), "hipStreamWaitEvent");
+        HIP_OK(hipMemcpyAsync(_dev_buffer[_write_ptr], _host_buffer_ptrs[_write_ptr], l.bytes, hipMemcpyHostToDevice, cs), "hipMemcpyAsync of a packed batch");
+        HIP_OK(hipEventRecord(static_cast<hipEvent_t>(_copied[_write_ptr]), cs), "hipEventRecord");
+    }
     {
         std::unique_lock<std::mutex> lock(_names_buff_lock);
         _circ_buff_data_info.push(_last_data_info);
@@ -131,9 +201,15 @@ void PackedCircularBuffer::push() {
 
 void *PackedCircularBuffer::get_read_buffer_dev() {
     if (!_initialized) THROW("Circular buffer not initialized")
+    Inside in(*this);
     block_if_empty();
-    if (empty()) THROW("the packed batch buffer is empty")  // (unblocked without a batch)
-    HIP_OK(hipStreamWaitEvent(static_cast<hipStream_t>(_consumer_stream), static_cast<hipEvent_t>(_copied[_read_ptr]), 0), "hipStreamWaitEvent");
+    {
+        std::unique_lock<std::mutex> lock(_lock);
+        if (_closing) THROW("the packed batch buffer was released")
+        if (empty()) THROW("the packed batch buffer is empty")  // (unblocked without a batch)
+    }
+    if (_device >= 0)
+        HIP_OK(hipStreamWaitEvent(static_cast<hipStream_t>(_consumer_stream), static_cast<hipEvent_t>(_copied[_read_ptr]), 0), "hipStreamWaitEvent");
     return _dev_buffer[_read_ptr];
 }
 
@@ -150,9 +226,11 @@ DecodedDataInfo &PackedCircularBuffer::get_decoded_data_info() {
 
 void PackedCircularBuffer::pop() {
     if (!_initialized) return;
-    if (empty()) THROW("pop on an empty packed batch buffer")
+    Inside in(*this);
+    if (level() == 0) THROW("pop on an empty packed batch buffer")
     // whatever has been enqueued on the consumer stream so far reads the slot: the writer's next copy into it waits for that
-    HIP_OK(hipEventRecord(static_cast<hipEvent_t>(_consumed[_read_ptr]), static_cast<hipStream_t>(_consumer_stream)), "hipEventRecord");
+    if (_device >= 0)
+        HIP_OK(hipEventRecord(static_cast<hipEvent_t>(_consumed[_read_ptr]), static_cast<hipStream_t>(_consumer_stream)), "hipEventRecord");
     {
         std::unique_lock<std::mutex> lock(_names_buff_lock);
         if (!_circ_buff_data_info.empty()) _circ_buff_data_info.pop();
@@ -170,23 +248,32 @@ size_t PackedCircularBuffer::level() {
     return _level;
 }
 
+// Empties the ring for a new epoch (circular_buffer.cpp:333-343). Threads blocked on it are woken and turned away first,
+// and the call waits until they have left; the ring then takes batches again.
 void PackedCircularBuffer::reset() {
+    stop();
     std::unique_lock<std::mutex> lock(_lock);
+    _idle.wait(lock, [&] { return _inside == 0; });
     _write_ptr = _read_ptr = _level = 0;
     _write_pos = 0;
     _placed.assign(_batch_size, false);
-    while (!_circ_buff_data_info.empty()) _circ_buff_data_info.pop();
+    {
+        std::unique_lock<std::mutex> names(_names_buff_lock);
+        while (!_circ_buff_data_info.empty()) _circ_buff_data_info.pop();
+    }
+    _released_reader = _released_writer = false;
+    _closing = false;
 }
 
 void PackedCircularBuffer::block_if_empty() {
     std::unique_lock<std::mutex> lock(_lock);
-    _wait_for_load.wait(lock, [&] { return !empty() || _released_reader; });
+    _wait_for_load.wait(lock, [&] { return !empty() || _released_reader || _closing; });
     _released_reader = false;
 }
 
 void PackedCircularBuffer::block_if_full() {
     std::unique_lock<std::mutex> lock(_lock);
-    _wait_for_unload.wait(lock, [&] { return !full() || _released_writer; });
+    _wait_for_unload.wait(lock, [&] { return !full() || _released_writer || _closing; });
     _released_writer = false;
 }
 

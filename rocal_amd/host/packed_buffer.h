@@ -32,11 +32,19 @@ struct PackedLayout {
 
 class PackedCircularBuffer {
    public:
-    // consumer_stream: the stream the kernels that read the batches run on (hipStream_t as void *)
+    // consumer_stream: the stream the kernels that read the batches run on (hipStream_t as void *).
+    // device < 0: a ring in plain host memory (the reference's RocalMemType::HOST): no device slots, no copies, no HIP call;
+    // get_read_buffer_dev() then returns the host slot.
     PackedCircularBuffer(int device, void *consumer_stream);
     ~PackedCircularBuffer();
     // slot_bytes: capacity of a slot (packed bytes of the largest batch); buff_depth slots, one of which is the one being read
     void init(size_t batch_size, size_t slot_bytes, size_t buff_depth);
+    // Shut-down, as the reference's loaders do it before they let go of their buffer (image_loader.cpp:84,126-127,241:
+    // unblock_writer / unblock_reader): stop() wakes every thread blocked on the ring and turns it, and every later caller,
+    // away with an exception ("released") instead of a slot; it is sticky until reset(). release() stops the ring, waits
+    // until no thread is inside one of its calls any more and only then frees the slots.
+    void stop();
+    bool stopped();
     void release();
     // ---- writer side (loader thread)
     unsigned char *get_write_buffer();  // pinned host memory of the slot being filled; blocks the caller if the buffer is full
@@ -78,4 +86,8 @@ class PackedCircularBuffer {
     std::condition_variable _wait_for_load, _wait_for_unload;
     size_t _write_ptr = 0, _read_ptr = 0, _level = 0;
     bool _initialized = false, _released_reader = false, _released_writer = false;
+    bool _closing = false;           // stop() was called: nobody is handed a slot any more
+    size_t _inside = 0;              // threads inside a call that touches the slots
+    std::condition_variable _idle;   // signalled when _inside falls to 0
+    struct Inside;                   // scope guard that counts a thread in and out
 };

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime_api.h>
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <iostream>
 
 #include "meta.h"
@@ -85,6 +87,62 @@ void Tensor::update_tensor_roi(const std::vector<uint32_t> &width, const std::ve
     }
 }
 
+void *Tensor::buffer() {
+    if (_owner) _owner->wait_outputs();
+    return _buffer;
+}
+
+std::vector<size_t> Tensor::strides() {
+    const std::vector<size_t> &d = _info.dims();
+    std::vector<size_t> s(d.size(), _info.data_type_size());
+    for (int i = (int)d.size() - 2; i >= 0; i--) s[i] = s[i + 1] * d[i + 1];
+    return s;
+}
+
+// tensor.cpp:419-454
+unsigned Tensor::copy_data(void *user_buffer, RocalOutputMemType external_mem_type) {
+    if (!_buffer) return 0;
+    if (!user_buffer) THROW("copy_data: null destination")
+    if (_owner) _owner->wait_outputs();
+    hipMemcpyKind kind;
+    if (external_mem_type == ROCAL_MEMCPY_GPU) kind = hipMemcpyDeviceToDevice;
+    else if (external_mem_type == ROCAL_MEMCPY_HOST || external_mem_type == ROCAL_MEMCPY_PINNED) kind = hipMemcpyDeviceToHost;
+    else THROW("copy_data requested mem type not supported")
+    hipError_t e = hipMemcpy(user_buffer, _buffer, _info.data_size(), kind);
+    if (e != hipSuccess) THROW(std::string("copy_data::hipMemcpy failed: ") + hipGetErrorName(e))
+    return 0;
+}
+
+// tensor.cpp:456-476: per sample, max_rows rows of max_cols elements from (x_offset, y_offset) of the sample's first
+// plane (rows of max_shape[0] elements), densely packed into host memory. One 2-D copy per sample.
+unsigned Tensor::copy_data(void *user_buffer, unsigned int x_offset, unsigned int y_offset, unsigned int max_cols, unsigned int max_rows) {
+    if (!_buffer) return 0;
+    if (!user_buffer) THROW("copy_data: null destination")
+    if (_owner) _owner->wait_outputs();
+    const size_t es = _info.data_type_size(), w = _info.max_shape()[0], h = _info.max_shape()[1];
+    const size_t row_elems = _info.layout() == RocalTensorlayout::NHWC ? w * _info.get_channels() : w;
+    if ((size_t)x_offset + max_cols > row_elems || (size_t)y_offset + max_rows > h) THROW("copy_data: the window exceeds the tensor")
+    const size_t sample_bytes = _info.data_size() / _info.batch_size();
+    for (size_t i = 0; i < _info.batch_size(); i++) {
+        const unsigned char *src = static_cast<const unsigned char *>(_buffer) + i * sample_bytes + ((size_t)y_offset * row_elems + x_offset) * es;
+        unsigned char *dst = static_cast<unsigned char *>(user_buffer) + i * (size_t)max_rows * max_cols * es;
+        hipError_t e = hipMemcpy2D(dst, (size_t)max_cols * es, src, row_elems * es, (size_t)max_cols * es, max_rows, hipMemcpyDeviceToHost);
+        if (e != hipSuccess) THROW(std::string("copy_data::hipMemcpy2D failed: ") + hipGetErrorName(e))
+    }
+    return 0;
+}
+
+void Tensor::copy_roi(void *roi_buffer) {
+    if (!roi_buffer) THROW("copy_roi: null destination")
+    memcpy(roi_buffer, _info.roi(), sizeof(Roi2DCords) * _info.batch_size());
+}
+
+void Tensor::set_mem_handle(void *buffer) {
+    if (!buffer) THROW("Invalid buffer pointer passed")
+    if (_owner) _owner->bind_output(this, buffer);
+    else _buffer = buffer;
+}
+
 /* ---------------------------------------------------------------- Graph */
 
 Graph::Graph(int gpu_id, void *stream) {
@@ -131,7 +189,6 @@ Graph::Status Graph::verify() {
 Graph::Status Graph::process() {
     for (Node *n : _order)
         if (!n->fused_away) n->launch();
-    if (rmx_ctx_sync(_ctx) != RMX_OK) THROW(std::string("rmx_ctx_sync failed: ") + rmx_last_error())
     return Status::OK;
 }
 
@@ -178,8 +235,8 @@ void Node::release() {
 
 void Node::launch() {
     Tensor *in = _inputs[0], *out = _outputs[0];
-    if (!in->buffer() || !out->buffer()) THROW("tensor without a device buffer at launch")
-    check(rmx_op_launch(_node, in->buffer(), out->buffer()), "rmx_op_launch");
+    if (!in->handle() || !out->handle()) THROW("tensor without a device buffer at launch")
+    check(rmx_op_launch(_node, in->handle(), out->handle()), "rmx_op_launch");
 }
 
 void Node::check(int status, const char *what) {
@@ -199,16 +256,30 @@ std::vector<uint32_t> Node::roi_as_array(const Roi2DCords *roi) const {
 
 /* ---------------------------------------------------------------- MasterGraph */
 
-MasterGraph::MasterGraph(size_t batch_size, int gpu_id, void *stream) : _batch_size(batch_size), _gpu_id(gpu_id), _graph(std::make_shared<Graph>(gpu_id, stream)) {}
+MasterGraph::MasterGraph(size_t batch_size, int gpu_id, void *stream) : _batch_size(batch_size), _gpu_id(gpu_id), _graph(std::make_shared<Graph>(gpu_id, stream)) {
+    hipEvent_t e;
+    if (hipEventCreateWithFlags(&e, hipEventDisableTiming) != hipSuccess) THROW("hipEventCreate failed")
+    _done = e;
+    const char *edge = getenv("ROCAL_BILINEAR_EDGE");
+    _graph->edge_device_rule = edge && (!strcmp(edge, "1") || !strcmp(edge, "device"));
+}
 
 MasterGraph::~MasterGraph() {
+    // loader threads blocked on a packed source leave with an exception before anything they use is freed
+    stop_sources();
+    _packed_sources.clear();
+    try {
+        wait_outputs();
+    } catch (...) {
+    }
+    if (_done) (void)hipEventDestroy(static_cast<hipEvent_t>(_done));
     if (_to_tensor_op) rmx_op_destroy(_to_tensor_op);
     _nodes.clear();
     for (void *p : _owned_buffers) (void)hipFree(p);
 }
 
 Tensor *MasterGraph::create_tensor(const TensorInfo &info, bool is_output) {
-    _tensors.emplace_back(new Tensor(info));
+    _tensors.emplace_back(new Tensor(info, this));
     Tensor *t = _tensors.back().get();
     t->is_output = is_output;
     if (is_output) _outputs.push_back(t);
@@ -232,7 +303,7 @@ void MasterGraph::build() {
     for (auto &n : _nodes) n->create(_graph);
     for (auto &n : _nodes) {
         Tensor *out = n->output()[0];
-        if (out->elided || out->buffer()) continue;
+        if (out->elided || out->handle()) continue;
         void *p = nullptr;
         if (hipMalloc(&p, out->info().data_size() + 64) != hipSuccess) THROW("hipMalloc of " + TOSTR(out->info().data_size()) + " bytes failed")
         if (hipMemset(p, 0, out->info().data_size() + 64) != hipSuccess) THROW("hipMemset failed")
@@ -318,6 +389,50 @@ void MasterGraph::run() {
     }
     StopWatch w(_time_us[1]);
     _graph->process();
+    if (hipEventRecord(static_cast<hipEvent_t>(_done), static_cast<hipStream_t>(stream())) != hipSuccess) THROW("hipEventRecord failed")
+    _pending = true;
+}
+
+void *MasterGraph::stream() const { return rmx_ctx_stream(_graph->get()); }
+
+// The wait counts as process time, which in the reference brackets the (synchronous) vxProcessGraph: master_graph.cpp:1015-1017.
+void MasterGraph::wait_outputs() {
+    if (!_pending) return;
+    StopWatch w(_time_us[1]);
+    _pending = false;
+    const hipError_t e = hipEventSynchronize(static_cast<hipEvent_t>(_done));
+    if (e != hipSuccess) THROW(std::string("waiting for the batch failed: ") + hipGetErrorString(e))
+}
+
+void MasterGraph::outputs_wait_on_stream(void *stream) {
+    if (!_pending) return;
+    if (hipStreamWaitEvent(static_cast<hipStream_t>(stream), static_cast<hipEvent_t>(_done), 0) != hipSuccess) THROW("hipStreamWaitEvent failed")
+}
+
+TensorList *MasterGraph::get_output_tensors() {
+    if (!_built) THROW("rocalVerify must be called before rocalGetOutputTensors")
+    wait_outputs();
+    _output_list.clear();
+    for (Tensor *t : _outputs) _output_list.push_back(t);
+    return &_output_list;
+}
+
+void MasterGraph::copy_output(unsigned char *out_ptr, size_t bytes) {
+    if (!_built) THROW("rocalVerify must be called before rocalCopyToOutput")
+    if (_outputs.size() != 1) THROW("Cannot copy, Multiple output tensors present in the list")
+    if (!out_ptr) THROW("rocalCopyToOutput needs an output pointer")
+    if (bytes != _outputs[0]->info().data_size()) THROW("rocalCopyToOutput: out_size " + TOSTR(bytes) + " is not the output's " + TOSTR(_outputs[0]->info().data_size()) + " bytes")
+    StopWatch w(_time_us[2]);
+    _outputs[0]->copy_data(out_ptr, ROCAL_MEMCPY_HOST);
+}
+
+void MasterGraph::stop_sources() {
+    for (auto &p : _packed_sources) p.second->stop();
+}
+
+void MasterGraph::set_edge_rule(bool device_rule) {
+    if (!_nodes.empty()) THROW("the bilinear edge rule must be chosen before the first node is added")
+    _graph->edge_device_rule = device_rule;
 }
 
 void MasterGraph::enable_meta_data() {
@@ -340,7 +455,7 @@ void MasterGraph::to_tensor(void *out_ptr, RocalTensorlayout format, float multi
     if (info.data_type() != RocalTensorDataType::UINT8) THROW("The output tensor is not of UINT8 type")
     if (info.layout() != RocalTensorlayout::NHWC) THROW("The output tensor is not interleaved RGB")
     if (!out_ptr) THROW("rocalToTensor needs a device output pointer")
-    if (!src->buffer()) THROW("The output tensor has no buffer yet")
+    if (!src->handle()) THROW("The output tensor has no buffer yet")
     rmx_tensor_desc s = info.desc(), d = s;
     if (max_roi_height == 0 || max_roi_width == 0) {
         max_roi_height = s.h;
@@ -360,6 +475,8 @@ void MasterGraph::to_tensor(void *out_ptr, RocalTensorlayout format, float multi
     }
     const float mul[3] = {multiplier0, multiplier1, multiplier2}, add[3] = {offset0, offset1, offset2};
     if (rmx_update_to_tensor(_to_tensor_op, mul, add, reverse_channels ? 1 : 0) != RMX_OK) THROW("rmx_update_to_tensor: " + std::string(rmx_last_error()))
-    if (rmx_op_launch(_to_tensor_op, src->buffer(), out_ptr) != RMX_OK) THROW("rmx_op_launch: " + std::string(rmx_last_error()))
+    // (same stream as the batch's launches: the conversion runs behind them, and the wait below covers both)
+    if (rmx_op_launch(_to_tensor_op, src->handle(), out_ptr) != RMX_OK) THROW("rmx_op_launch: " + std::string(rmx_last_error()))
     if (rmx_ctx_sync(_graph->get()) != RMX_OK) THROW("rmx_ctx_sync: " + std::string(rmx_last_error()))
+    _pending = false;
 }

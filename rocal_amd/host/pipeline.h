@@ -1,8 +1,8 @@
 // Tensor / Graph / Node / pipeline context of the hot path, with rocAL's interface
 // (rocAL/include/pipeline/tensor.h:65-309, graph.h:29-44, node.h:30-63, master_graph.h:245-263) on top of
 // the C ABI in include/rocal_mi355x.h. A Node owns one rmx_op; Graph::process() launches the nodes in
-// creation order on one stream and waits, which is what vxProcessGraph does for the reference
-// (rocAL/source/pipeline/graph.cpp:96-103).
+// creation order on one stream (vxProcessGraph of the reference, rocAL/source/pipeline/graph.cpp:96-103) and
+// records an event behind them; the wait for that event is where a consumer takes an output (MasterGraph::wait_outputs).
 #pragma once
 #include <cstdint>
 #include <list>
@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "exception.h"
+#include "rocal_api_mi355x.h"
 #include "rocal_mi355x.h"
 
 // rocAL/include/pipeline/commons.h:45-70,110-113 (same numeric values as the C ABI's enums)
@@ -66,11 +67,36 @@ class TensorInfo {
     std::shared_ptr<Roi2DCords> _roi;
 };
 
-class Tensor {
+class MasterGraph;
+
+// rocAL/include/pipeline/tensor.h:316-388: the tensor behind the public rocalTensor interface.
+class Tensor : public rocalTensor {
    public:
-    explicit Tensor(const TensorInfo &info) : _info(info) {}
+    explicit Tensor(const TensorInfo &info, MasterGraph *owner = nullptr) : _info(info), _owner(owner) {}
     const TensorInfo &info() const { return _info; }
-    void *buffer() const { return _buffer; }
+    // the device address as the graph sees it (no wait): nodes, launches, bindings
+    void *handle() const { return _buffer; }
+    // ---- rocalTensor (what a consumer calls: buffer() and the copies wait for the batch that is being computed)
+    void *buffer() override;
+    unsigned copy_data(void *user_buffer, RocalOutputMemType external_mem_type) override;
+    unsigned copy_data(void *user_buffer, unsigned int x_offset, unsigned int y_offset, unsigned int max_cols, unsigned int max_rows) override;
+    unsigned num_of_dims() override { return (unsigned)_info.dims().size(); }
+    unsigned batch_size() override { return (unsigned)_info.batch_size(); }
+    std::vector<size_t> dims() override { return _info.dims(); }
+    std::vector<size_t> strides() override;
+    RocalTensorLayout layout() override { return (RocalTensorLayout)_info.layout(); }
+    RocalTensorBackend backend() override { return ROCAL_GPU; }
+    RocalTensorOutputType data_type() override { return (RocalTensorOutputType)_info.data_type(); }
+    RocalOutputMemType mem_type() override { return ROCAL_MEMCPY_GPU; }
+    size_t data_size() override { return _info.data_size(); }
+    RocalROICordsType roi_type() override { return (RocalROICordsType)_info.roi_type(); }
+    size_t get_roi_dims_size() override { return 2; }
+    void copy_roi(void *roi_buffer) override;
+    std::vector<size_t> shape() override { return _info.max_shape(); }
+    void set_dims(std::vector<size_t>) override { THROW("the dimensions of a pipeline tensor are fixed by the node that produces it") }
+    void set_mem_handle(void *buffer) override;
+    void set_tensor_layout(RocalTensorLayout) override { THROW("the layout of a pipeline tensor is fixed by the node that produces it") }
+    uint64_t data_type_size() override { return _info.data_type_size(); }
     // The loader / ring buffer hands a new device buffer every batch (tensor.cpp:478-489).
     void swap_handle(void *device_ptr) { _buffer = device_ptr; }
     // Clamps to the padded maxima like Tensor::update_tensor_roi (tensor.cpp:193-220).
@@ -84,8 +110,21 @@ class Tensor {
 
    private:
     TensorInfo _info;
+    MasterGraph *_owner = nullptr;
     void *_buffer = nullptr;
     const PackedLayout *_ragged = nullptr;
+};
+
+// rocAL/include/pipeline/tensor.h:391-422
+class TensorList : public rocalTensorList {
+   public:
+    uint64_t size() override { return _tensor_list.size(); }
+    Tensor *at(size_t index) override { return _tensor_list.at(index); }
+    void push_back(Tensor *t) { _tensor_list.push_back(t); }
+    void clear() { _tensor_list.clear(); }
+
+   private:
+    std::vector<Tensor *> _tensor_list;
 };
 
 class Node;
@@ -96,10 +135,13 @@ class Graph {
     explicit Graph(int gpu_id, void *stream = nullptr);
     ~Graph();
     Status verify();
-    Status process();
+    Status process();  // enqueues the launches of every node; does not wait
     Status release();
     rmx_ctx *get() { return _ctx; }
     void add(Node *n) { _order.push_back(n); }
+    // bilinear resize nodes clamp the right / lower neighbour at the last-but-one pixel of the window, as the reference's
+    // device kernel does (rocAL/rocAL_hip/rocal_hip_kernels.cpp:339-345), instead of at the last pixel
+    bool edge_device_rule = false;
 
    private:
     rmx_ctx *_ctx = nullptr;
@@ -161,7 +203,18 @@ class MasterGraph {
         return node;
     }
     void build();
+    // One batch: parameters renewed, nodes updated, launches enqueued, an event recorded behind them. Does not wait.
     void run();
+    // Blocks until the batch of the last run() is complete (the consumer side of the reference's output ring buffer:
+    // ring_buffer.cpp:118-119 block_if_empty, called from get_output_tensors / copy_output, master_graph.cpp:859-938).
+    void wait_outputs();
+    void outputs_wait_on_stream(void *stream);
+    TensorList *get_output_tensors();                        // master_graph.cpp:929-938
+    void copy_output(unsigned char *out_ptr, size_t bytes);  // master_graph.cpp:859-927
+    void stop_sources();                                     // wakes every thread blocked on a packed source
+    void set_edge_rule(bool device_rule);
+    bool edge_rule() const { return _graph->edge_device_rule; }
+    void *stream() const;
     void set_output(Tensor *t);  // master_graph.cpp:337-349
     // A source tensor fed through a ring of packed batches (stands where the loader module and its CircularBuffer stand,
     // master_graph.cpp:1116-1160 / image_loader.cpp:115-170): run() takes the oldest batch of every such source.
@@ -201,6 +254,9 @@ class MasterGraph {
     std::shared_ptr<BoundingBoxGraph> _meta_graph;
     std::shared_ptr<MetaDataBatch> _input_meta, _output_meta;
     bool _built = false;
+    void *_done = nullptr;   // hipEvent_t behind the launches of the last run()
+    bool _pending = false;   // a run() has been enqueued and nobody has waited for it yet
+    TensorList _output_list;
     std::vector<std::pair<Tensor *, std::unique_ptr<PackedCircularBuffer>>> _packed_sources;
     double _time_us[3] = {0.0, 0.0, 0.0};
     // the conversion op of to_tensor(), rebuilt when the requested format changes

@@ -61,6 +61,15 @@ PY_API int rocalpy_set_outputs(RocalContext ctx, unsigned n, RocalTensor *tensor
     return 0;
 }
 
+// rocalGetOutputTensors for callers without C++: waits for the batch, writes up to `cap` tensor handles, returns their number (-1: error).
+PY_API int rocalpy_output_tensors(RocalContext ctx, RocalTensor *out, unsigned cap) {
+    RocalTensorList l = rocalGetOutputTensors(ctx);
+    if (!l) return -1;
+    const unsigned n = (unsigned)l->size();
+    for (unsigned i = 0; i < n && i < cap; i++) out[i] = l->at(i);
+    return (int)(n < cap ? n : cap);
+}
+
 PY_API void rocalpy_timing(RocalContext ctx, unsigned long long out[5]) {
     out[4] = rocalGetParameterUpdateTime(ctx);
     const TimingInfo t = rocalGetTimingInfo(ctx);

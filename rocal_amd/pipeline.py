@@ -72,10 +72,31 @@ class Pipeline:
         return self
 
     def rocal_run(self):
+        """Enqueues one batch on the pipeline's stream and returns; get_output_tensors() (or wait_on_stream) is where the
+        consumer waits for it, as in the reference (pipeline.py: rocal_run, then get_output_tensors in the iterators)."""
         status = b.rocalRun(self._handle)
         if status != types.OK:
             raise RuntimeError("rocalRun failed: " + b.getErrorMessage(self._handle))
         return status
+
+    def get_output_tensors(self):
+        """Waits for the batch of the last rocal_run and returns the output tensors (rocAL_pybind/amd/rocal/pipeline.py:
+        get_output_tensors). A tensor bound with bind_output is complete in the caller's memory from here on."""
+        return b.getOutputTensors(self._handle)
+
+    def wait_on_stream(self, stream=None):
+        """Makes a HIP stream (a torch.cuda.Stream, default: torch's current stream) wait for the batch of the last rocal_run
+        instead of the host: work queued on it afterwards sees the outputs."""
+        import torch
+        s = stream if stream is not None else torch.cuda.current_stream()
+        if b.outputsWaitOnStream(self._handle, s.cuda_stream) != types.OK:
+            raise RuntimeError("wait_on_stream failed: " + b.getErrorMessage(self._handle))
+
+    def set_bilinear_edge_rule(self, device_rule):
+        """True: bilinear resizes clamp the right / lower neighbour at the last-but-one pixel of the window, as the reference's
+        device kernel does; False (default): at the last pixel. Before the first resize node is added."""
+        if b.setBilinearEdgeRule(self._handle, device_rule) != types.OK:
+            raise RuntimeError("set_bilinear_edge_rule failed: " + b.getErrorMessage(self._handle))
 
     def copyToExternalTensor(self, array, multiplier, offset, reverse_channels, tensor_format, tensor_dtype, max_roi_height=0, max_roi_width=0):
         import ctypes
@@ -127,6 +148,11 @@ class Pipeline:
         """Blocks until the loader has pushed a batch (rocal_run on an empty ring raises instead of blocking)."""
         if b.packedSourceWait(self._handle, source) != types.OK:
             raise RuntimeError("wait_for_batch failed: " + b.getErrorMessage(self._handle))
+
+    def stop_source(self, source):
+        """Wakes a loader thread blocked in place_image and a consumer blocked in wait_for_batch; they, and every later caller,
+        get an exception. release() does this for every packed source before it frees anything."""
+        return b.packedSourceStop(self._handle, source)
 
     def queued_batches(self, source):
         return b.packedSourceLevel(self._handle, source)

@@ -127,6 +127,8 @@ def test_flip_warp_rotate_crop(rec):
 def test_normalize_and_transpose(rec):
     fn.normalize("in")
     assert rec.calls[-1] == ("normalize", "H", "in", [], [], [], False, 1.0, 0.0, types.FLOAT)
+    fn.normalize("in", output_datatype=types.FLOAT16)  # the reference's spelling of the keyword (fn.py:1216)
+    assert rec.calls[-1] == ("normalize", "H", "in", [], [], [], False, 1.0, 0.0, types.FLOAT16)
     fn.normalize("in", axes=[0, 1], mean=[1.0], stddev=[2.0], scale=3.0, shift=4.0, output_dtype=types.FLOAT16)
     assert rec.calls[-1] == ("normalize", "H", "in", [0, 1], [1.0], [2.0], False, 3.0, 4.0, types.FLOAT16)
     fn.transpose("in", perm=[2, 0, 1], output_layout=types.NCHW)

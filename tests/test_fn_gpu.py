@@ -49,6 +49,7 @@ def test_random_resized_crop_colour_twist_cmn_into_a_torch_tensor():
         mine.zero_()
         pipe.feed(src, dimg, [w for w, _ in ROIS], [h for _, h in ROIS])
         pipe.rocal_run()
+        pipe.get_output_tensors()  # the consumer's wait for the batch
         got = mine.cpu().numpy()
         assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), "batch %d: %d values differ" % (batch, int((got != exp).sum()))
         assert np.array_equal(np.array(pipe.output_roi(out))[:, 2:], crop[:, 2:])
@@ -73,6 +74,7 @@ def test_warp_affine_and_flip_pipeline():
     pipe.build()
     pipe.feed(src, torch.from_numpy(img).cuda(), [w for w, _ in ROIS], [h for _, h in ROIS])
     pipe.rocal_run()
+    pipe.get_output_tensors()  # the consumer's wait for the batch
     # matrix [x0, x1, y0, y1, o0, o1] reaches the node as rocAL's fill order x0, y0, x1, y1, o0, o1 (node_warp_affine.cpp:43-48)
     m = np.stack([orc.affine_from_rocal([1.05, -0.08, 0.1, 0.95, 3.0, -2.0])] * N)
     roi = np.array([[0, 0, w, h] for w, h in ROIS], np.uint32)
@@ -96,6 +98,7 @@ def test_output_through_dlpack():
     dimg = torch.from_numpy(img).cuda()
     pipe.feed(src, dimg, [w for w, _ in ROIS], [h for _, h in ROIS])
     pipe.rocal_run()
+    pipe.get_output_tensors()  # the consumer's wait for the batch
     t = torch.from_dlpack(pipe.output_dlpack(out))
     assert t.is_cuda and t.dtype == torch.float32 and tuple(t.shape) == (N, 3, 32, 40)
     from rocal_amd import backend

@@ -299,3 +299,18 @@ def test_decoder_crop_windows_statistics():
     assert abs(np.mean(np.log(ratio))) < 0.05      # log-uniform about 1 (fit conditioning leaves a small tilt)
     free = 640 - got[:, 2]
     assert abs(np.mean(got[free > 50, 0] / free[free > 50]) - 0.5) < 0.03
+
+
+def test_loader_ring_shutdown_protocol():
+    """The ring of packed batches in host memory (no HIP call on this path): a loader thread blocked on the full ring is woken
+    by stop() / release() / unblock_writer() and leaves with an exception, never with a slot that is still full; release() frees
+    the slots only after the thread has left; a consumer blocked on the empty ring is woken the same way; reset() reopens
+    the ring (rocAL/source/loaders/image/image_loader.cpp:84,126-127,241; circular_buffer.cpp:299-343)."""
+    exe = os.path.join(ROOT, "rocal_amd", "lib", "host_check")
+    p = subprocess.run([exe, "ring"], capture_output=True, text=True, timeout=60)
+    assert p.returncode == 0, (p.stdout, p.stderr)
+    lines = p.stdout.strip().splitlines()
+    assert lines[-1] == "ring ok" and all(l.endswith(" ok") for l in lines)
+    for name in ("stop_wakes_loader", "release_wakes_loader", "unblock_without_room_is_an_error", "release_wakes_reader",
+                 "reader_turned_away_after_stop", "ring_usable_after_reset", "oldest_batch_intact", "writer_continues_after_pop"):
+        assert name + " ok" in lines

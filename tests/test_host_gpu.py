@@ -127,10 +127,14 @@ def test_random_resized_crop_colour_cmn_runs_as_one_kernel(tmp_path, scenario):
         assert np.array_equal(roi[:, 2:], crop[:, 2:])
 
 
-def test_caller_built_against_the_public_header_alone(tmp_path):
+@pytest.mark.parametrize("edge", ["textbook", "device"])
+def test_caller_built_against_the_public_header_alone(tmp_path, edge):
     """tests/cpp/api_caller.cpp sees include/rocal_api_mi355x.h and nothing else of this repository: CropResize -> ColorTwist ->
-    CropMirrorNormalize, two batches, the output bound to memory the caller allocated (rocalTensorSetBuffer), the timers of
-    rocalGetTimingInfo. Same expected values as the three reference nodes run one after the other."""
+    CropMirrorNormalize, two batches, read as a program written for rocAL reads them (rocalGetOutputTensors(ctx)->at(0)->copy_data,
+    dims, strides, copy_roi, rocalCopyToOutput), the second with the output bound to memory the caller allocated (set_mem_handle);
+    the timers of rocalGetTimingInfo. Same expected values as the three reference nodes run one after the other, under both
+    rules for the right / lower neighbour at a window's edge (ROCAL_BILINEAR_EDGE: the textbook clamp, and the last-but-one
+    pixel of the reference's device kernel, rocal_hip_kernels.cpp:339-345)."""
     img = _image()
     img.tofile(tmp_path / "input.bin")
     with open(tmp_path / "meta.txt", "w") as f:
@@ -138,17 +142,23 @@ def test_caller_built_against_the_public_header_alone(tmp_path):
         for w, h in ROIS:
             f.write("%d %d\n" % (w, h))
     exe = os.path.join(ROOT, "rocal_amd", "lib", "api_caller")
-    print("api_caller", flush=True)
-    p = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=110)
+    print("api_caller", edge, flush=True)
+    env = dict(os.environ)
+    env.pop("ROCAL_BILINEAR_EDGE", None)
+    if edge == "device":
+        env["ROCAL_BILINEAR_EDGE"] = "device"
+    p = subprocess.run([exe, str(tmp_path)], capture_output=True, text=True, timeout=110, env=env)
     assert p.returncode == 0, (p.returncode, p.stdout, p.stderr)
     assert "intermediates_elided 1" in p.stdout and p.stdout.strip().endswith("ok")
     t = dict(zip(*[iter(p.stdout.split("timing_us ")[1].split("\n")[0].split())] * 2))
-    assert int(t["process"]) > 0 and int(t["update"]) > 0 and int(t["load"]) == 0 and int(t["transfer"]) == 0
+    assert int(t["process"]) > 0 and int(t["update"]) > 0 and int(t["load"]) == 0 and int(t["transfer"]) > 0  # (transfer: rocalCopyToOutput)
     assert "timing_after_reset 0" in p.stdout
     s = orc.FParam.simple
     window = np.stack([orc.random_crop(s(0.5), s(1.2), s(0.3), s(0.7), w, h) for w, h in ROIS])
     full = np.full(N, 64, np.uint32)
-    mid = orc.resize(img, window, full, full, 64, 64, interp=orc.LINEAR)
+    mid = orc.resize(img, window, full, full, 64, 64, interp=orc.LINEAR, flags=orc.F_BILINEAR_EDGE_QUIRK if edge == "device" else 0)
+    if edge == "device":  # the two rules differ on this input (else the second run would prove nothing)
+        assert not np.array_equal(mid, orc.resize(img, window, full, full, 64, 64, interp=orc.LINEAR))
     mid_w, mid_h = np.minimum(window[:, 2], 64), np.minimum(window[:, 3], 64)
     one = lambda v: np.full(N, v, np.float32)
     mid_roi = np.stack([np.zeros(N), np.zeros(N), mid_w, mid_h], -1).astype(np.uint32)

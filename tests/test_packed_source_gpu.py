@@ -59,7 +59,9 @@ def test_packed_batches_through_the_ring():
     assert pipe.queued_batches(src) == 2
     for k in range(5):
         mine.zero_()
+        torch.cuda.synchronize()  # (the pipeline's stream is not ordered against torch's)
         pipe.rocal_run()
+        pipe.get_output_tensors()  # the consumer's wait for the batch
         got = mine.cpu().numpy()
         exp = _expect(batches[k][2], batches[k][0])
         assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), "batch %d: %d values differ" % (k, int((got != exp).sum()))
@@ -91,6 +93,7 @@ def test_packed_source_errors():
     pipe.place_image(src, 1, np.zeros((3, 8, 3), np.uint8))
     pipe.push(src)
     pipe.rocal_run()
+    pipe.get_output_tensors()  # the consumer's wait for the batch
     pipe.release()
 
 
@@ -120,15 +123,59 @@ def test_loader_thread_and_consumer():
         except Exception as e:  # noqa: BLE001
             failed.append(e)
 
-    th = threading.Thread(target=loader, daemon=True)  # (a failing check below must not leave the interpreter waiting for it)
+    th = threading.Thread(target=loader)
     th.start()
-    for k in range(8):
-        pipe.wait_for_batch(src)
-        mine.zero_()  # the nodes write the valid region of every sample only
-        pipe.rocal_run()
-        got = mine.cpu().numpy()  # (waits for the run)
-        exp = _expect(batches[k][2], batches[k][0])
-        assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), "batch %d" % k
-    th.join(timeout=30)
-    assert not th.is_alive() and not failed
+    try:
+        for k in range(8):
+            pipe.wait_for_batch(src)
+            mine.zero_()  # the nodes write the valid region of every sample only
+            torch.cuda.synchronize()
+            pipe.rocal_run()
+            pipe.get_output_tensors()  # the consumer's wait for the batch
+            got = mine.cpu().numpy()
+            exp = _expect(batches[k][2], batches[k][0])
+            assert np.array_equal(got.view(np.uint16), exp.view(np.uint16)), "batch %d" % k
+        th.join(timeout=30)
+        assert not th.is_alive() and not failed
+    finally:
+        pipe.release()  # (wakes the loader if a check above failed while it was blocked on the full ring)
+        th.join(timeout=30)
+
+
+def test_release_wakes_a_loader_blocked_on_the_full_ring():
+    """The shut-down protocol of the reference's loaders (image_loader.cpp:84,126-127: unblock_writer / unblock_reader before the
+    buffer goes): a loader thread, not a daemon, blocked in place_image on a full ring; release() from the main thread; the
+    thread leaves within a second with the error recorded, and never with a slot that was still full."""
+    import threading
+    import time
+    pipe = Pipeline(batch_size=N, device_id=0, seed=5)
+    with pipe:
+        src = pipe.packed_source(WMAX, HMAX, queue_depth=2)
+        out = fn.crop_mirror_normalize(src, crop=(40, 40), mean=MEAN, std=STD, mirror=0, output_layout=types.NCHW, output_dtype=types.FLOAT16)
+        pipe.set_outputs(out)
+    pipe.build()
+    _, images, _ = _batch(7)
+    state = {"pushed": 0, "error": None}
+
+    def loader():
+        try:
+            for _ in range(4):  # the ring holds one finished batch: the second batch's first image blocks
+                for i in range(N):
+                    pipe.place_image(src, i, images[i])
+                pipe.push(src)
+                state["pushed"] += 1
+        except Exception as e:  # noqa: BLE001
+            state["error"] = e
+
+    th = threading.Thread(target=loader)
+    th.start()
+    deadline = time.time() + 10
+    while state["pushed"] < 1 and time.time() < deadline:
+        time.sleep(0.01)
+    time.sleep(0.2)
+    assert th.is_alive() and state["pushed"] == 1 and state["error"] is None  # blocked on the full ring
+    t0 = time.time()
     pipe.release()
+    th.join(timeout=5)
+    assert not th.is_alive() and time.time() - t0 < 1.0
+    assert state["pushed"] == 1 and "released" in str(state["error"])
