@@ -36,6 +36,12 @@
 #ifndef RMX_DMA_NT
 #define RMX_DMA_NT (sizeof(T) == 2)  // fp16: streaming stores
 #endif
+// Measurement builds only (results are wrong): bit 0 leaves out the loads of the source window, bit 1 the stores of the
+// result, bit 2 the blend (one LDS read per row, no arithmetic: the kernel's memory traffic with next to no instructions),
+// so that a timing shows what each part costs by itself. 0 in the library.
+#ifndef RMX_DMA_EXPERIMENT
+#define RMX_DMA_EXPERIMENT 0
+#endif
 
 namespace rmx {
 
@@ -163,7 +169,8 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                     for (int r = 0; r < nrows; r++) {
                         const int ysrc = max(min(a_v + r, yhi), ylo);
                         const uint8_t *rowp = base4 + ((uint32_t)ysrc * row_stride + g.col4);
-                        __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(bufb + (r * g.ppr + c0) * 16), 16, 0, RMX_LDS_LOAD_AUX);
+                        if constexpr (!(RMX_DMA_EXPERIMENT & 1))
+                            __builtin_amdgcn_global_load_lds((glb_ptr_t)(rowp + lane_off), (lds_ptr_t)(bufb + (r * g.ppr + c0) * 16), 16, 0, RMX_LDS_LOAD_AUX);
                     }
                 }
             }
@@ -284,6 +291,11 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                 float v[3][PX];
 #pragma unroll
                 for (int k = 0; k < PX; k++) {
+                    if constexpr (RMX_DMA_EXPERIMENT & 4) {
+                        const float t = k ? v[0][0] : __builtin_bit_cast(float, *(const lds_u32 *)(row0 + bo4[0]) + *(const lds_u32 *)(row1 + bo4[0]));
+                        v[0][k] = v[1][k] = v[2][k] = t;
+                        continue;
+                    }
                     const lds_u32 *q0 = (const lds_u32 *)(row0 + bo4[k]);
                     const lds_u32 *q1 = (const lds_u32 *)(row1 + bo4[k]);
                     const uint32_t a0 = q0[0], a1 = q0[1], a2 = q0[2], b0 = q1[0], b1 = q1[1], b2 = q1[2];
@@ -312,7 +324,8 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                 packed_on = full;
                 packed_r = r;
             } else if (full) {
-                store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, r, x0, packed);
+                if constexpr (RMX_DMA_EXPERIMENT & 2) asm volatile("" ::"v"(packed.w[0]), "v"(packed.w[PackedGroup<T>::WORDS - 1]));
+                else store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, r, x0, packed);
             }
         }
 
@@ -330,7 +343,10 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
             a_v = issue(ng, nr0, min(nr0 + wrows, r_end));
         }
         asm volatile("" ::: "memory");  // the held-back stores are issued after those loads, not before
-        if (DEFER && packed_on) store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, packed_r, x0, packed);
+        if (DEFER && packed_on) {
+            if constexpr (RMX_DMA_EXPERIMENT & 2) asm volatile("" ::"v"(packed.w[0]), "v"(packed.w[PackedGroup<T>::WORDS - 1]));
+            else store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, packed_r, x0, packed);
+        }
         asm volatile("" ::: "memory");
         if (!more) break;
         // (the aligned form always holds stores back: lane 0 has a whole group in every last pass; a tile of the any-width
