@@ -317,22 +317,85 @@ def time_updates(op, update_fn, launchers, steps, sets=12):
     return update_ms, serial_ms, piped_ms
 
 
-def copy_ceiling(ctx, nbytes=1 << 30, reps=20):
+def stream_ceilings(ctx, nbytes=1 << 30, reps=12):
+    """What the memory system of this box gives a kernel with no arithmetic, on 1 GiB buffers (four times the last-level
+    cache): a copy (bytes read + bytes written per second), a pass that only reads and one that only writes, each the best
+    over 4 / 8 / 16 / 32 workgroups per compute unit of the library's streaming probe. GB/s."""
     import torch
     a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
     a.zero_()
-    for _ in range(3):
-        ctx.copy_bytes(a, b, nbytes)
-    torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for _ in range(reps):
-        ctx.copy_bytes(a, b, nbytes)
-    e1.record()
-    torch.cuda.synchronize()
-    ms = e0.elapsed_time(e1) / reps
-    return 2.0 * nbytes / (ms * 1e-3) / 1e9  # read + write
+    b.zero_()
+    out = {}
+    for mode, name, factor in ((0, "copy", 2.0), (1, "read_only", 1.0), (2, "write_only", 1.0)):
+        best = (0.0, 0)
+        for g in (4, 8, 16, 32):
+            for _ in range(3):
+                ctx.stream_probe(mode, a, b, nbytes, g)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                ctx.stream_probe(mode, a, b, nbytes, g)
+            e1.record()
+            torch.cuda.synchronize()
+            rate = factor * nbytes / (e0.elapsed_time(e1) / reps * 1e-3) / 1e9
+            best = max(best, (rate, g))
+        out[name] = best
+    del a, b
+    torch.cuda.empty_cache()
+    return out
+
+
+def rocal_protocol(batches=400, pairs=4):
+    """C1 through the reference's own entry points, as a rocAL program runs a batch: rocalCreate -> rocalDeviceSource ->
+    rocalCropResize (random windows, renewed per batch by the C++ ParameterFactory) -> rocalCropMirrorNormalize (random mirror)
+    -> rocalVerify; the two nodes run as one launch. Sources and destinations rotate over `pairs` buffers (4 x 315 MB of
+    padded sources). Returns milliseconds per batch:
+      serial     feed, rocalRun, rocalGetOutputTensors (the consumer's wait) for every batch, by the host clock;
+      pipelined  the same without the per-batch wait (one wait at the end): the host runs ahead of the GPU;
+      process / update  the library's own timers for the serial loop (rocalGetTimingInfo().process_time: launches + the wait;
+                 rocalGetParameterUpdateTime: parameter renewal + node updates), per batch."""
+    import torch
+    from rocal_amd import fn, types, workloads as wl
+    from rocal_amd.pipeline import Pipeline, b
+    n = 256
+    c = wl.config1(n)
+    pipe = Pipeline(batch_size=n, device_id=0, seed=1235)
+    with pipe:
+        src = pipe.device_source(640, 640)
+        a = fn.resize_crop(src, resize_width=224, resize_height=224)
+        out = fn.crop_mirror_normalize(a, crop=(224, 224), mean=[float(x) for x in wl.MEAN], std=[float(x) for x in wl.STD],
+                                       mirror=b.createIntRand([0, 1], [0.5, 0.5], 2), output_layout=types.NCHW, output_dtype=types.FLOAT16)
+        pipe.set_outputs(out)
+    pipe.build()
+    srcs = [torch.from_numpy(c["img"]).cuda() for _ in range(pairs)]
+    dsts = [torch.empty((n, 3, 224, 224), dtype=torch.float16, device="cuda") for _ in range(pairs)]
+    W, H = [int(x) for x in c["W"]], [int(x) for x in c["H"]]
+
+    def one(i, wait):
+        pipe.feed(src, srcs[i % pairs], W, H)
+        pipe.bind_output(out, dsts[i % pairs])
+        pipe.rocal_run()
+        if wait:
+            pipe.get_output_tensors()
+    for i in range(50):
+        one(i, True)
+    pipe.timing_info()
+    t0 = time.perf_counter()
+    for i in range(batches):
+        one(i, True)
+    serial = (time.perf_counter() - t0) * 1e3 / batches
+    t = pipe.timing_info()
+    t0 = time.perf_counter()
+    for i in range(batches):
+        one(i, False)
+    pipe.get_output_tensors()
+    piped = (time.perf_counter() - t0) * 1e3 / batches
+    pipe.release()
+    del srcs, dsts
+    torch.cuda.empty_cache()
+    return {"serial": serial, "pipelined": piped, "process": t["process_time"] * 1e-3 / batches, "update": t["parameter_update_time"] * 1e-3 / batches}
 
 
 def cpu_baseline(cpu_fn, n, budget_s=12.0):
@@ -443,12 +506,23 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     from rocal_amd import ops
     ctx = ops.Context(0)
-    ceiling = copy_ceiling(ctx)
+    streams = stream_ceilings(ctx)
+    ceiling = streams["copy"][0]
     res = run_config(args.config, ctx, args.steps, args.warmup, not args.no_cpu and not args.rotating_only and not args.resident_only,
                      args.rotating_only, args.ramp_ms, args.resident_only)
     res["metric"] = "images/s + HBM GB/s (% peak), RandomResizedCrop+CMN 224^2 fp16, batch 256" if args.config == 1 else "images/s"
     res["roofline"]["copy_ceiling_GBps"] = round(ceiling, 1)
     res["roofline"]["frac_of_copy_ceiling"] = round(res["roofline"]["achieved"] / ceiling, 4)
+    res["roofline"]["read_only_GBps"] = round(streams["read_only"][0], 1)
+    res["roofline"]["write_only_GBps"] = round(streams["write_only"][0], 1)
+    res["roofline"]["stream_probe_groups_per_cu"] = {k: v[1] for k, v in streams.items()}
+    if args.config == 1 and not args.rotating_only and not args.resident_only:
+        rp = rocal_protocol()
+        res["config"]["rocal_run_ms_per_batch"] = round(rp["process"] + rp["update"], 6)
+        res["config"]["rocal_run_process_ms"] = round(rp["process"], 6)
+        res["config"]["rocal_run_update_ms"] = round(rp["update"], 6)
+        res["config"]["rocal_run_host_ms_per_batch"] = round(rp["serial"], 6)
+        res["config"]["rocal_run_pipelined_ms_per_batch"] = round(rp["pipelined"], 6)
     if args.all:
         allres = {args.config: res}
         for cfg in sorted(WORKLOADS):

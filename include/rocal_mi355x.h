@@ -260,6 +260,11 @@ RMX_API int rmx_update_rotate(rmx_op *op, const uint32_t *src_roi, const float *
 /* ---- measurement helper: plain device-to-device streaming copy (nbytes, 16-byte multiples),
  *      used to establish the copy ceiling of the box and the scale of rocprof's byte counters. */
 RMX_API int rmx_copy_bytes(rmx_ctx *ctx, const void *src, void *dst, size_t nbytes);
+/* ---- measurement helper: one streaming pass of the same shape as the copy (every workgroup walks a contiguous chunk, four
+ *      16-byte pieces per lane in flight, non-temporal loads and stores) in one of three modes: 0 copies src to dst,
+ *      1 only reads src (dst is not written), 2 only writes dst (src is not read); groups_per_cu workgroups per compute
+ *      unit (0: the library's default). Establishes what the memory system gives reads, writes and both together. */
+RMX_API int rmx_stream_probe(rmx_ctx *ctx, int mode, const void *src, void *dst, size_t nbytes, int groups_per_cu);
 
 #ifdef __cplusplus
 }

@@ -79,6 +79,7 @@ _SIGS = {
     "rmx_create_transpose": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), _vp, C.c_int, C.POINTER(_vp)],
     "rmx_update_transpose": [_vp, _vp],
     "rmx_copy_bytes": [_vp, _vp, _vp, C.c_size_t],
+    "rmx_stream_probe": [_vp, C.c_int, _vp, _vp, C.c_size_t, C.c_int],
     "rmx_resize_cmn_noalloc": [_vp, C.POINTER(TensorDesc), C.POINTER(TensorDesc), C.c_int, C.c_int, C.c_uint32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp],
 }
 _RESTYPES = {"rmx_last_error": C.c_char_p, "rmx_version": C.c_char_p, "rmx_ctx_stream": _vp,

@@ -1722,4 +1722,16 @@ int rmx_copy_bytes(rmx_ctx *ctx, const void *src, void *dst, size_t nbytes) {
     return RMX_OK;
 }
 
+int rmx_stream_probe(rmx_ctx *ctx, int mode, const void *src, void *dst, size_t nbytes, int groups_per_cu) {
+    if (!ctx || !src || !dst) return fail(RMX_ERR_INVALID, "context/source/destination is NULL");
+    if (mode < 0 || mode > 2) return fail(RMX_ERR_INVALID, "mode must be 0 (copy), 1 (read only) or 2 (write only)");
+    if (groups_per_cu < 0 || groups_per_cu > 64) return fail(RMX_ERR_INVALID, "groups_per_cu out of range (0..64)");
+    if (nbytes % 16 != 0) return fail(RMX_ERR_INVALID, "nbytes must be a multiple of 16");
+    if ((((uintptr_t)src) | ((uintptr_t)dst)) & 15u) return fail(RMX_ERR_INVALID, "buffers must be 16-byte aligned");
+    HIP_TRY(hipSetDevice(ctx->device));
+    rmx::launch_stream(ctx->stream, mode, src, dst, nbytes, ctx->num_cus, groups_per_cu);
+    HIP_TRY(hipGetLastError());
+    return RMX_OK;
+}
+
 }  // extern "C"

@@ -27,4 +27,6 @@ constexpr int kWarpRawPieces = RMX_WARP_RAW_PIECES;
 void launch_stats(hipStream_t stream, const RmxKArgs &a, unsigned long long *counters, RmxSample *table, const float *given, int mode, int per_channel,
                   float scale, float shift, bool reduce);
 void launch_copy(hipStream_t stream, const void *src, void *dst, size_t nbytes, int num_cus);
+// mode 0 copy, 1 read only, 2 write only; groups_per_cu 0 = the default (16)
+void launch_stream(hipStream_t stream, int mode, const void *src, void *dst, size_t nbytes, int num_cus, int groups_per_cu);
 }  // namespace rmx

@@ -63,6 +63,10 @@ class Context:
     def copy_bytes(self, src, dst, nbytes):
         check(_lib.lib().rmx_copy_bytes(self._h, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), nbytes))
 
+    def stream_probe(self, mode, src, dst, nbytes, groups_per_cu=0):
+        """One streaming pass: mode 0 copies src to dst, 1 only reads src, 2 only writes dst."""
+        check(_lib.lib().rmx_stream_probe(self._h, mode, C.c_void_p(src.data_ptr()), C.c_void_p(dst.data_ptr()), nbytes, groups_per_cu))
+
     def close(self):
         if self._h:
             _lib.lib().rmx_ctx_destroy(self._h)
