@@ -114,6 +114,9 @@ struct rmx_op {
     RmxSample *d_table[TABLE_RING] = {};
     hipEvent_t uploaded[TABLE_RING] = {};
     int cur = -1;  // slot of the last update, -1 before the first
+    // A launch of this op was recorded into a HIP graph: the graph's kernel node holds the address of the table slot of the
+    // last update, which the ring would hand out again four updates later. Such an op keeps its parameters: updates are refused.
+    bool captured = false;
 
     // launch plan of the last update
     rmx::KernelFn fn = nullptr;
@@ -196,6 +199,9 @@ int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor
 
 // Next table slot; waits until the upload that last used it has completed.
 int next_slot(rmx_op *op, RmxSample **row) {
+    if (op->captured)
+        return fail(RMX_ERR_INVALID, "a launch of this op was recorded into a HIP graph, whose replays read the parameter rows of the update before the capture: "
+                                     "the op keeps those parameters (create another op for new ones, or record rmx_resize_cmn_noalloc, which carries its rows in the graph)"), -2;
     int slot = (op->cur + 1) % TABLE_RING;
     HIP_TRY(hipSetDevice(op->ctx->device));
     HIP_TRY(hipEventSynchronize(op->uploaded[slot]));
@@ -539,6 +545,10 @@ static int launch_table(rmx_op *op, const RmxSample *table, const RmxSrcLayout *
     }
     hipLaunchKernelGGL(fn, dim3((unsigned)blocks), dim3(wpb * RMX_WAVE), lds, op->ctx->stream, a);
     HIP_TRY(hipGetLastError());
+    if (!op->captured) {
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(op->ctx->stream, &capturing) == hipSuccess && capturing == hipStreamCaptureStatusActive) op->captured = true;
+    }
     return RMX_OK;
 }
 
@@ -607,7 +617,7 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
                      bool per_sample_scale = true, bool channel_reverse = false, int *open_slot = nullptr) {
     RmxSample *t;
     int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
+    if (slot < 0) return slot == -2 ? RMX_ERR_INVALID : RMX_ERR_HIP;
     uint64_t bytes = 0;
     int max_rows = 1;
     for (int i = 0; i < op->n; i++) {
@@ -773,7 +783,7 @@ int rmx_update_transpose(rmx_op *op, const uint32_t *src_roi) {
     if (!op->aux1) return update_k1(op, src_roi, nullptr, nullptr, nullptr, nullptr);  // a layout change of the streaming kernel
     RmxSample *t;
     int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
+    if (slot < 0) return slot == -2 ? RMX_ERR_INVALID : RMX_ERR_HIP;
     uint64_t bytes = 0;
     int max_w = 1, max_h = 1;
     for (int i = 0; i < op->n; i++) {
@@ -1301,7 +1311,7 @@ static int update_resize_common(rmx_op *op, const uint32_t *src_roi, const uint3
     if (!op || op->kind != OP_RESIZE) return fail(RMX_ERR_INVALID, "op is not a Resize node");
     RmxSample *t;
     int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
+    if (slot < 0) return slot == -2 ? RMX_ERR_INVALID : RMX_ERR_HIP;
     int rc = fill_resize_rows(op, t, src_roi, dst_w, dst_h, crop_roi, scale, bias, mean, stddev, mirror, colour);
     if (rc) return rc;
     return commit_slot(op, slot);
@@ -1347,7 +1357,7 @@ static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const 
                         float d0, float d1, float d2, float d3, bool hue_in_p2) {
     RmxSample *t;
     int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
+    if (slot < 0) return slot == -2 ? RMX_ERR_INVALID : RMX_ERR_HIP;
     uint64_t bytes = 0;
     int max_rows = 1;
     for (int i = 0; i < op->n; i++) {
@@ -1482,7 +1492,7 @@ static int create_point(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, cons
 static int update_point(rmx_op *op, const uint32_t *roi, const float *p0, const float *gamma) {
     RmxSample *t;
     int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
+    if (slot < 0) return slot == -2 ? RMX_ERR_INVALID : RMX_ERR_HIP;
     uint64_t bytes = 0;
     int max_rows = 1;
     const int sources = op->kind == OP_BLEND ? 2 : 1;
@@ -1576,7 +1586,7 @@ static int create_warp(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const
 static int update_warp(rmx_op *op, const uint32_t *roi, const float *affine, const float *angle, const uint32_t *dst_w, const uint32_t *dst_h) {
     RmxSample *t;
     int slot = next_slot(op, &t);
-    if (slot < 0) return RMX_ERR_HIP;
+    if (slot < 0) return slot == -2 ? RMX_ERR_INVALID : RMX_ERR_HIP;
     uint64_t bytes = 0;
     int max_dw = 1, max_dh = 1;
     double worst_box = 0;

@@ -268,6 +268,34 @@ int run_pipeline(const std::string &scenario, const std::string &dir) {
         outs.push_back(rocalNormalize(ctx, src, hwc, m3, s3, true, 3.0f, 1.0f, ROCAL_FP16));  // given statistics, scale and shift
         outs.push_back(rocalTranspose(ctx, src, {1, 0, 2}, true, ROCAL_NHWC));                // [N, W, H, C]
         outs.push_back(rocalTranspose(ctx, src, {2, 0, 1}, true, ROCAL_NCHW));                // [N, C, H, W]
+    } else if (scenario == "ref_cases") {
+        // The fixed-parameter cases of the reference's own unit tests (tests/cpp_api/unit_tests/unit_tests.cpp:605-624,730-735,
+        // 745-856), all on one source, with the parameters written there.
+        std::vector<float> mean128{128, 128, 128}, std12{1.2f, 1.2f, 1.2f};
+        RocalIntParam m1 = rocalCreateIntParameter(1);
+        outs.push_back(rocalResize(ctx, src, 400, 400, true, ROCAL_SCALING_MODE_DEFAULT, {}, 0, 0, ROCAL_LINEAR_INTERPOLATION));      // case 0
+        outs.push_back(rocalResize(ctx, src, 400, 400, true, ROCAL_SCALING_MODE_DEFAULT, {}, 0, 0, ROCAL_TRIANGULAR_INTERPOLATION));  // case 0, triangular
+        outs.push_back(rocalCropMirrorNormalize(ctx, src, 224, 224, 0, 0, mean128, std12, true, m1));                                 // case 25
+        outs.push_back(rocalCropMirrorNormalize(ctx, src, 224, 224, 0.5f, 0.5f, mean128, std12, true, m1));                           // case 55
+        outs.push_back(rocalCropResizeFixed(ctx, src, 224, 224, true, 0.25f, 1.2f, 0.6f, 0.4f));                                      // case 30
+        RocalTensor rot = rocalRotateFixed(ctx, src, 45, true);                                                                       // case 31
+        outs.push_back(rot);
+        outs.push_back(rocalBrightnessFixed(ctx, src, 1.90f, 20, true));                                                              // case 32
+        outs.push_back(rocalGammaFixed(ctx, src, 0.5f, true));                                                                        // case 33
+        outs.push_back(rocalContrastFixed(ctx, src, 30, 80, true));                                                                   // case 34
+        outs.push_back(rocalBlendFixed(ctx, src, rot, 0.5f, true));                                                                   // case 36
+        outs.push_back(rocalWarpAffineFixed(ctx, src, 1, 1, 0.5f, 0.5f, 7, 7, true));                                                 // case 37
+        outs.push_back(rocalColorTempFixed(ctx, src, 70, true));                                                                      // case 43
+        outs.push_back(rocalExposureFixed(ctx, src, 1, true));                                                                        // case 46
+        outs.push_back(rocalFlipFixed(ctx, src, 1, 0, true));                                                                         // case 47
+        outs.push_back(rocalHueFixed(ctx, src, 150, true));                                                                           // case 48
+        outs.push_back(rocalSaturationFixed(ctx, src, 0.3f, true));                                                                   // case 49
+        outs.push_back(rocalColorTwistFixed(ctx, src, 0.2f, 10.0f, 100.0f, 0.25f, true));                                             // case 50
+        outs.push_back(rocalCropFixed(ctx, src, 224, 224, 1, true, 0, 0, 0));                                                         // case 51
+        outs.push_back(rocalCropCenterFixed(ctx, src, 224, 224, 2, true));                                                            // case 52
+        outs.push_back(rocalResizeCropMirrorFixed(ctx, src, 400, 400, true, 200, 200, m1));                                           // case 53
+        outs.push_back(rocalResizeMirrorNormalize(ctx, src, 400, 400, mean128, std12, true, ROCAL_SCALING_MODE_DEFAULT, {}, 0, 0,
+                                                  ROCAL_LINEAR_INTERPOLATION, m1));                                                   // case 56
     } else if (scenario == "to_tensor") {
         outs.push_back(rocalResize(ctx, src, 40, 32, true));
     } else if (scenario == "errors") {

@@ -225,7 +225,8 @@ def test_warp_on_an_exact_size_source_and_tiny_windows(ctx, interp, W):
 def test_launches_can_be_captured_in_a_graph_and_replayed(ctx):
     """update() uploads the parameter table outside the capture; the launches of a resize -> colour twist -> flip
     chain are recorded in a HIP graph and replayed several times, with eager work and synchronisation between
-    the replays and a new input each time; every replay must equal the eager result."""
+    the replays and a new input each time; every replay must equal the eager result. An op whose launch was recorded
+    refuses further updates (its replays would read rows that the table ring hands out again)."""
     import torch
     s = torch.cuda.Stream()
     c2 = ops.Context(0, stream=s.cuda_stream)
@@ -252,6 +253,13 @@ def test_launches_can_be_captured_in_a_graph_and_replayed(ctx):
         flip.launch(b, out)
     for rep in range(4):
         img = rng.integers(0, 256, (n, H, W, 3), dtype=np.uint8)
+        if rep == 2:
+            # an update between replays: refused, because the graph's kernel node reads the table slot of the update before
+            # the capture, which the ring would hand out again a few updates later; the replays after it are unchanged
+            from rocal_amd._lib import RmxError
+            for op_, args in ((resize, (roi, dw // 2, dh)), (twist, (mid_roi, one(0.9), one(1.0), one(5.0), one(1.0)))):
+                with pytest.raises(RmxError, match="recorded into a HIP graph"):
+                    op_.update(*args)
         with torch.cuda.stream(s):
             src.copy_(torch.from_numpy(img))
             out.zero_()
