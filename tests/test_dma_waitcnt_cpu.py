@@ -72,3 +72,66 @@ def test_streaming_triangular_kernel_counts_its_stores():
         assert "global_load_lds_dwordx4" in body
         checked += 1
     assert checked == 54  # every instance of the kernel
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="needs hipcc")
+def test_warp_kernel_hand_written_lds_reads_are_awaited_before_use():
+    """The raw bilinear form of the warp kernel writes the LDS reads of a pixel's taps out by hand and waits for them by a
+    count (s_waitcnt lgkmcnt(4): the four reads of the next pixel may still be outstanding). The compiler does not know
+    that those registers are filled later, so the generated code of every instance is checked: in a loop that waits this
+    way there are exactly the 32 read instructions of 8 pixels and nothing else that counts as an LDS / scalar-memory
+    operation; the waits are 7 x lgkmcnt(4) and one lgkmcnt(0); and no instruction between a pixel's reads and the wait
+    that covers them touches a register those reads fill."""
+    from rocal_amd import build as rbuild
+    src = os.path.join(ROOT, "rocal_amd", "csrc", "rmx_kernels_warp.hip")
+    with tempfile.TemporaryDirectory() as tmp:
+        out = os.path.join(tmp, "warp.s")
+        subprocess.run([HIPCC] + list(rbuild.FLAGS) + ["-I" + os.path.join(ROOT, "rocal_amd", "csrc"), "-I" + os.path.join(ROOT, "include"),
+                        "--cuda-device-only", "-S", src, "-o", out], check=True, capture_output=True, timeout=600)
+        text = open(out).read()
+
+    def regs(tok):
+        m = re.match(r"v\[(\d+):(\d+)\]", tok)
+        if m:
+            return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        m = re.match(r"v(\d+)$", tok)
+        return {int(m.group(1))} if m else set()
+
+    funcs = re.split(r"\n(?=_ZN3rmx15rmx_warp_kernel[^\n]*:\s)", text)
+    loops = 0
+    for f in funcs:
+        m = re.match(r"(_ZN3rmx15rmx_warp_kernel\S*):", f)
+        if not m:
+            continue
+        body = f.split("s_endpgm")[0]
+        blocks = re.split(r"\n(?=\.LBB\d+_\d+:)", body)
+        for blk in blocks:
+            if not re.search(r"ds_read2_b32 [^\n]* offset0:4[0-9] offset1:4[0-9]", blk):
+                continue  # (only the hand-written reads take the row below from an offset inside the instruction)
+            ins = [l.strip() for l in blk.splitlines() if l.strip() and not l.strip().startswith((";", "."))]
+            lgkm = [i for i in ins if re.match(r"(ds_|s_load|s_buffer_load|s_memtime|s_memrealtime|s_sendmsg|s_dcache)", i)]
+            assert len(lgkm) == 32 and all(i.startswith(("ds_read2_b32", "ds_read_b32")) for i in lgkm), (m.group(1), lgkm[:3], len(lgkm))
+            waits = [i for i in ins if i.startswith("s_waitcnt")]
+            assert [w.split()[-1] for w in waits] == ["lgkmcnt(4)"] * 7 + ["lgkmcnt(0)"], (m.group(1), waits)
+            # pixel k's four reads are covered by the k-th wait
+            pos_reads = [n for n, i in enumerate(ins) if i.startswith("ds_read")]
+            pos_waits = [n for n, i in enumerate(ins) if i.startswith("s_waitcnt")]
+            for k in range(8):
+                group = pos_reads[4 * k: 4 * k + 4]
+                filled = set()
+                for n in group:
+                    filled |= regs(ins[n].split()[1].rstrip(","))
+                for n in range(group[-1] + 1, pos_waits[k]):
+                    if ins[n].startswith("ds_read"):
+                        continue  # (the next pixel's reads: they fill other registers, checked next)
+                    toks = re.findall(r"v\[\d+:\d+\]|v\d+", ins[n])
+                    touched = set().union(*[regs(t) for t in toks]) if toks else set()
+                    assert not (touched & filled), "%s: '%s' touches a register whose LDS read is not awaited yet" % (m.group(1), ins[n])
+                # the next pixel's reads must not fill a register of this pixel before this pixel's wait
+                if k + 1 < 8 and pos_reads[4 * k + 4] < pos_waits[k]:
+                    nxt = set()
+                    for n in pos_reads[4 * k + 4: 4 * k + 8]:
+                        nxt |= regs(ins[n].split()[1].rstrip(","))
+                    assert not (nxt & filled), m.group(1)
+            loops += 1
+    assert loops >= 12  # two loops (with and without the ROI test) in each of the six formats
