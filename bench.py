@@ -45,6 +45,7 @@ WORKLOADS = {
     9: "N4 Exposure 224x224 u8->u8 NHWC batch 256",
     10: "N4 ColorTemperature 224x224 u8->u8 NHWC batch 256",
     11: "C1 with a ColorTwist node fused between RandomResizedCrop and CropMirrorNormalize (one launch), ->224x224 fp16 NCHW batch 256",
+    12: "C1's RandomResizedCrop windows with triangular (antialiasing) interpolation + normalize + mirror ->224x224 fp16 NCHW batch 256",
 }
 
 
@@ -130,6 +131,18 @@ def build_case(cfg, ctx, n=None):
         def cpu(k):
             from oracle import orc
             return orc.resize(c["img"][:k], c["roi"][:k], dw[:k], dh[:k], 360, 640, interp=orc.TRIANGULAR, mirror=c["mirror"][:k],
+                              scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16)
+    elif cfg == 12:
+        n = n or 256
+        c = wl.config1(n)
+        dw = np.full(n, 224, np.uint32)
+        op = ops.Resize(ctx, ops.desc(n, 640, 640, ops.NHWC, ops.UINT8), ops.desc(n, 224, 224, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+        op.update(c["roi"], dw, dw, c["mirror"], np.tile(wl.MEAN, n), np.tile(wl.STD, n))
+        scale, bias = scale_bias(n)
+
+        def cpu(k):
+            from oracle import orc
+            return orc.resize(c["img"][:k], c["roi"][:k], dw[:k], dw[:k], 224, 224, interp=orc.TRIANGULAR, mirror=c["mirror"][:k],
                               scale=scale[:3 * k], bias=bias[:3 * k], layout=orc.NCHW, dtype=orc.FP16)
     elif cfg == 5:
         n = n or 256
