@@ -10,6 +10,7 @@
 #include <new>
 #include <string>
 #include <limits>
+#include <mutex>
 #include <vector>
 
 #include "rmx_common.h"
@@ -70,8 +71,11 @@ __global__ void __launch_bounds__(256) rmx_table_upload_kernel(const uint4 *__re
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += gridDim.x * blockDim.x) dst[i] = src[i];
 }
 
+static std::mutex g_life_lock;  // creation and destruction of ops against the destruction of their context
+
 struct rmx_ctx {
     int upload_kernel = 1;        // 1: tables are uploaded by rmx_table_upload_kernel, 0: by hipMemcpyAsync
+    // (both under g_life_lock: a garbage collector may destroy ops and their context from different threads)
     int live_ops = 0;             // ops made on this context and not yet destroyed: they use its streams until their own end
     bool closed = false;          // rmx_ctx_destroy was called while ops were alive; the last op's end frees the context
     void *scratch_ptr = nullptr;  // device address of `scratch` on this context's device
@@ -178,7 +182,10 @@ int make_op(rmx_ctx *ctx, int kind, const rmx_tensor_desc *src, const rmx_tensor
     rmx_op *op = new (std::nothrow) rmx_op();
     if (!op) return fail(RMX_ERR_NOMEM, "out of host memory");
     op->ctx = ctx;
-    ctx->live_ops++;
+    {
+        std::lock_guard<std::mutex> life(g_life_lock);
+        ctx->live_ops++;
+    }
     op->kind = kind;
     op->src = *src;
     op->dst = *dst;
@@ -419,9 +426,12 @@ static void ctx_free(rmx_ctx *ctx) {
 
 int rmx_ctx_destroy(rmx_ctx *ctx) {
     if (!ctx) return RMX_OK;
-    if (ctx->live_ops > 0) {  // an op outlives its context (destruction order of a garbage collector): keep the streams for it
-        ctx->closed = true;
-        return RMX_OK;
+    {
+        std::lock_guard<std::mutex> life(g_life_lock);
+        if (ctx->live_ops > 0) {  // an op outlives its context (destruction order of a garbage collector): keep the streams for it
+            ctx->closed = true;
+            return RMX_OK;
+        }
     }
     ctx_free(ctx);
     return RMX_OK;
@@ -446,7 +456,12 @@ int rmx_op_destroy(rmx_op *op) {
     }
     rmx_ctx *ctx = op->ctx;
     delete op;
-    if (--ctx->live_ops == 0 && ctx->closed) ctx_free(ctx);
+    bool last;
+    {
+        std::lock_guard<std::mutex> life(g_life_lock);
+        last = --ctx->live_ops == 0 && ctx->closed;
+    }
+    if (last) ctx_free(ctx);
     return RMX_OK;
 }
 

@@ -39,9 +39,26 @@ def _deleter(p):
     _alive.pop(C.addressof(p.contents), None)
 
 
+# A capsule that is dropped without having been consumed still carries the name "dltensor": its destructor then calls the
+# deleter (the DLPack producer rule); a consumer renames the capsule ("used_dltensor") and calls the deleter itself.
+_CAPSULE_DESTRUCTOR = C.CFUNCTYPE(None, C.c_void_p)
+_capsule_is_valid = C.pythonapi.PyCapsule_IsValid
+_capsule_is_valid.restype = C.c_int
+_capsule_is_valid.argtypes = [C.c_void_p, C.c_char_p]
+_capsule_get_pointer = C.pythonapi.PyCapsule_GetPointer
+_capsule_get_pointer.restype = C.c_void_p
+_capsule_get_pointer.argtypes = [C.c_void_p, C.c_char_p]
+
+
+@_CAPSULE_DESTRUCTOR
+def _capsule_destructor(capsule):
+    if _capsule_is_valid(capsule, b"dltensor"):
+        _alive.pop(_capsule_get_pointer(capsule, b"dltensor"), None)
+
+
 _capsule_new = C.pythonapi.PyCapsule_New
 _capsule_new.restype = C.py_object
-_capsule_new.argtypes = [C.c_void_p, C.c_char_p, C.c_void_p]
+_capsule_new.argtypes = [C.c_void_p, C.c_char_p, _CAPSULE_DESTRUCTOR]
 
 
 def to_dlpack(device_ptr, shape, dtype, device_id=0, keep_alive=None):
@@ -59,4 +76,4 @@ def to_dlpack(device_ptr, shape, dtype, device_id=0, keep_alive=None):
     m.manager_ctx = None
     m.deleter = _deleter
     _alive[C.addressof(m)] = (m, dims, keep_alive)
-    return _capsule_new(C.addressof(m), b"dltensor", None)
+    return _capsule_new(C.addressof(m), b"dltensor", _capsule_destructor)
