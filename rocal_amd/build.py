@@ -8,8 +8,12 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
-OBJDIR = os.path.join(HERE, "lib", "obj")
-LIB = os.path.join(LIBDIR, os.environ.get("RMX_LIB_NAME", "librocal_mi355x.so"))  # override: experiment builds
+# RMX_LIB_NAME / RMX_EXTRA_FLAGS: measurement builds under another name (e.g. the streaming bilinear kernel without its loads,
+# stores or arithmetic: RMX_LIB_NAME=librocal_exp4.so RMX_EXTRA_FLAGS=-DRMX_DMA_EXPERIMENT=4), loaded with RMX_LIB=<path>;
+# such a build keeps its objects apart from the library's.
+_NAME = os.environ.get("RMX_LIB_NAME", "librocal_mi355x.so")
+OBJDIR = os.path.join(HERE, "lib", "obj" if _NAME == "librocal_mi355x.so" else "obj_" + os.path.splitext(_NAME)[0])
+LIB = os.path.join(LIBDIR, _NAME)
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 # -ffp-contract=off: the kernels spell every fused multiply-add out (bit-exact parity with the

@@ -47,6 +47,13 @@ namespace rmx {
 
 extern __shared__ uint32_t rmx_lds_dma[];
 
+// (measurement builds: every word of a group that is not stored still has to be computed)
+template <typename T>
+RMX_DEV void keep_alive(const PackedGroup<T> &g) {
+#pragma unroll
+    for (int i = 0; i < PackedGroup<T>::WORDS; i++) asm volatile("" ::"v"(g.w[i]));
+}
+
 RMX_DEV float src_coord_d(int u, float ratio, float off, float lo) {
     float s = (float)u * ratio;
     s = s + off;
@@ -324,7 +331,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
                 packed_on = full;
                 packed_r = r;
             } else if (full) {
-                if constexpr (RMX_DMA_EXPERIMENT & 2) asm volatile("" ::"v"(packed.w[0]), "v"(packed.w[PackedGroup<T>::WORDS - 1]));
+                if constexpr (RMX_DMA_EXPERIMENT & 2) keep_alive(packed);
                 else store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, r, x0, packed);
             }
         }
@@ -344,7 +351,7 @@ __global__ void __launch_bounds__(256) rmx_resize_dma_kernel(RmxKArgs a) {
         }
         asm volatile("" ::: "memory");  // the held-back stores are issued after those loads, not before
         if (DEFER && packed_on) {
-            if constexpr (RMX_DMA_EXPERIMENT & 2) asm volatile("" ::"v"(packed.w[0]), "v"(packed.w[PackedGroup<T>::WORDS - 1]));
+            if constexpr (RMX_DMA_EXPERIMENT & 2) keep_alive(packed);
             else store_packed<T, LAYOUT, RMX_DMA_NT, !ALIGNED>(dimg, a.dst_h, a.dst_w, packed_r, x0, packed);
         }
         asm volatile("" ::: "memory");
