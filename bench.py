@@ -384,7 +384,8 @@ def rocal_protocol(batches=400, pairs=4):
     pipe.build()
     srcs = [torch.from_numpy(c["img"]).cuda() for _ in range(pairs)]
     dsts = [torch.empty((n, 3, 224, 224), dtype=torch.float16, device="cuda") for _ in range(pairs)]
-    W, H = [int(x) for x in c["W"]], [int(x) for x in c["H"]]
+    import numpy as np
+    W, H = np.ascontiguousarray(c["W"], dtype=np.uint32), np.ascontiguousarray(c["H"], dtype=np.uint32)
 
     def one(i, wait):
         pipe.feed(src, srcs[i % pairs], W, H)

@@ -175,9 +175,16 @@ class Backend:
         return host().rocalDeviceSource(handle, max_width, max_height, is_output)
 
     def deviceSourceFeed(self, handle, source, device_ptr, widths, heights):
-        n = len(widths)
-        w = (C.c_uint * n)(*[int(x) for x in widths])
-        h = (C.c_uint * n)(*[int(x) for x in heights])
+        # contiguous uint32 numpy arrays are handed over as they are (no per-element conversion on the per-batch path)
+        def as_uints(v):
+            if hasattr(v, "ctypes") and getattr(v, "dtype", None) == "uint32" and v.flags["C_CONTIGUOUS"] and v.ndim == 1:
+                return v.ctypes.data_as(C.POINTER(C.c_uint)), v
+            arr = (C.c_uint * len(v))(*[int(x) for x in v])
+            return arr, arr
+        w, keep_w = as_uints(widths)
+        h, keep_h = as_uints(heights)
+        if len(widths) != len(heights):
+            raise ValueError("widths and heights differ in length")
         return host().rocalDeviceSourceFeed(handle, source, device_ptr, w, h)
 
     def packedSource(self, handle, max_width, max_height, is_output, queue_depth, slot_bytes):

@@ -81,11 +81,19 @@ class UniformRand : public Parameter<T> {
     // One engine draw per value even when the range is a single point (the draw happens first).
     void renew_value() {
         std::lock_guard<std::mutex> g(_mutex);
+        renew_value_unlocked();
+    }
+    // For a caller that draws a whole batch from this parameter (the crop-window laws): it takes mutex() once for the batch
+    // and then draws with renew_value_unlocked(), which is renew() + get() of a parameter without an array.
+    std::mutex &mutex() { return _mutex; }
+    bool has_array() const { return !_values.empty(); }
+    T renew_value_unlocked() {
         const auto raw = _engine();
         if (single_value())
             _current = _lo;
         else
             _current = static_cast<T>(((double)raw / (double)_engine.max()) * ((double)_hi - (double)_lo) + (double)_lo);
+        return _current;
     }
     void renew() override {
         if (_values.empty()) {

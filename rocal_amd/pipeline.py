@@ -111,7 +111,8 @@ class Pipeline:
         return b.deviceSource(self._handle, max_width, max_height, is_output)
 
     def feed(self, source, tensor, widths, heights):
-        """tensor: a torch CUDA uint8 tensor [N, max_height, max_width, 3]; widths / heights: the valid size of each image."""
+        """tensor: a torch CUDA uint8 tensor [N, max_height, max_width, 3]; widths / heights: the valid size of each image
+        (sequences of integers, or contiguous uint32 numpy arrays, which are passed on as they are)."""
         assert tensor.is_cuda and tensor.is_contiguous()
         self._fed = tensor  # kept alive until the next batch
         status = b.deviceSourceFeed(self._handle, source, tensor.data_ptr(), widths, heights)

@@ -72,7 +72,8 @@ def test_warp_affine_and_flip_pipeline():
     pipe.bind_output(wa, t_wa)  # both outputs land in the caller's tensors; the flip node reads the first one from there
     pipe.bind_output(fl, t_fl)
     pipe.build()
-    pipe.feed(src, torch.from_numpy(img).cuda(), [w for w, _ in ROIS], [h for _, h in ROIS])
+    # (sizes as uint32 arrays: handed to the library without a per-element conversion)
+    pipe.feed(src, torch.from_numpy(img).cuda(), np.array([w for w, _ in ROIS], np.uint32), np.array([h for _, h in ROIS], np.uint32))
     pipe.rocal_run()
     pipe.get_output_tensors()  # the consumer's wait for the batch
     # matrix [x0, x1, y0, y1, o0, o1] reaches the node as rocAL's fill order x0, y0, x1, y1, o0, o1 (node_warp_affine.cpp:43-48)
