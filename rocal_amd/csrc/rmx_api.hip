@@ -1454,9 +1454,15 @@ static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const 
     bool aligned = op->flat_h ? true : op->dst.w % 8 == 0;
     for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
     op->fn_fast = nullptr;
+    // kernel kind: 0 linear, 1 twist, 2 twist with one comparison for the hue's way back into range (no shift near one sextant)
+    int kkind = 0;
+    if (op->kind == OP_COLOR_TWIST || op->kind == OP_HUE || op->kind == OP_SATURATION) {
+        kkind = 2;
+        for (int i = 0; i < op->n && kkind == 2; i++)
+            if (!(t[i].color[2] < RMX_HUE_SHIFT_LOW || t[i].color[2] >= RMX_HUE_SHIFT_HIGH)) kkind = 1;
+    }
     if (aligned) {
-        const bool twist = (op->kind == OP_COLOR_TWIST || op->kind == OP_HUE || op->kind == OP_SATURATION);
-        op->fn_fast = rmx::select_color_kernel(twist ? 1 : 0, op->dst.dtype, op->dst.layout, 1, &op->fast_name);
+        op->fn_fast = rmx::select_color_kernel(kkind, op->dst.dtype, op->dst.layout, 1, &op->fast_name);
         op->fast_strips = op->strips;
         op->fast_lds = 0;
         op->fast_rows = op->aux0;
@@ -1468,7 +1474,7 @@ static int update_color(rmx_op *op, const uint32_t *roi, const float *p0, const 
     for (int i = 0; i < op->n && wide8; i++) wide8 = t[i].dst_w >= 8 || t[i].dst_w <= 0 || t[i].dst_h <= 0;
     op->fn_mid = nullptr;
     if (wide8) {
-        op->fn_mid = rmx::select_color_kernel((op->kind == OP_COLOR_TWIST || op->kind == OP_HUE || op->kind == OP_SATURATION) ? 1 : 0, op->dst.dtype, op->dst.layout, 2, &op->mid_name);
+        op->fn_mid = rmx::select_color_kernel(kkind, op->dst.dtype, op->dst.layout, 2, &op->mid_name);
         op->mid_strips = op->strips;
         op->mid_lds = 0;
         op->mid_rows = op->aux0;

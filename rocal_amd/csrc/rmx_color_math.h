@@ -27,9 +27,29 @@ constexpr SectorRow sector_row(int hi) {
     return SectorRow{{sg[0], sg[1], sg[2]}, nb[0], nb[1], nb[2], 0.0f, 0.0f};
 }
 
+// How a hue comes back into [0, 6]. The hue of a pixel is num / delta + (0 | 2 | 4) + shift with |num / delta| <= 1 (to within
+// a rounding), so for one sample, whose shift is one number, it lies in [shift - 1, shift + 5]: with shift below 1 it never
+// reaches 6 and only "below 0: + 6" can happen, with shift above 1 it never falls below 0 and only "6 and above: - 6" can.
+// Either is one comparison instead of two: hue >= t ? at : af is added, the same addition the two comparisons choose. A shift
+// within 2e-5 of 1 keeps both comparisons (HUE_WRAP_BOTH): the host looks at the batch's shifts and picks the kernel
+// (RMX_HUE_SHIFT_LOW / RMX_HUE_SHIFT_HIGH in rmx_common.h).
+enum { HUE_WRAP_BOTH = 0, HUE_WRAP_ONE = 1 };
+struct HueWrap {
+    float t, at, af;
+};
+RMX_DEV HueWrap hue_wrap_of(float shift) {
+    const bool low = shift < RMX_HUE_SHIFT_LOW;
+    return HueWrap{low ? 0.0f : 6.0f, low ? 0.0f : -6.0f, low ? 6.0f : 0.0f};
+}
+
 // Branch-free: lanes of a wavefront hold pixels of different hue sectors, so
 // branches would run every case one after the other under changing execution masks.
-RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const SectorRow *sect, float alpha, float beta, float shift, float shift2, float shift4, float satf) {
+template <int WRAP = HUE_WRAP_BOTH>
+RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const SectorRow *sect, float alpha, float beta, float shift, float shift2, float shift4, float satf,
+                      float wrap_t = 0.0f, float wrap_at = 0.0f, float wrap_af = 0.0f) {
+    // (the channel values as plain registers: knowing that they are converted bytes, the compiler subtracts the bytes as integers
+    // for the hue numerator and converts the difference, one instruction more per pixel than subtracting the floats it has)
+    asm("" : "+v"(r), "+v"(g), "+v"(b));
     const float cmax = __builtin_fmaxf(__builtin_fmaxf(r, g), b);
     const float cmin = __builtin_fminf(__builtin_fminf(r, g), b);
     const float delta = cmax - cmin;
@@ -37,13 +57,15 @@ RMX_DEV void twist_px(float &r, float &g, float &b, const float *rcp, const Sect
     float s = delta * rcp[(int)cmax];
     // A grey pixel needs no case of its own: r == g == b makes it a "red is largest" pixel with g - b == 0.
     const bool is_r = cmax == r, is_g = cmax == g;
-    const float num = is_r ? (g - b) : (is_g ? (b - r) : (r - g));
+    const float d_gb = g - b, d_br = b - r, d_rg = r - g;  // (all three, then two selects: no branch)
+    const float num = is_r ? d_gb : (is_g ? d_br : d_rg);
     // sextant offset 0 / 2 / 4 plus the hue shift, the three sums made once per sample
     const float add = is_r ? shift : (is_g ? shift2 : shift4);
     float hh = __builtin_fmaf(num, rd, add);
     // back into [0, 6]: one addition of +6, -6 or 0. A value just below zero can round to exactly 6.0 here; row 6 of the sector
     // table repeats row 0 and fract(6.0) is 0, which is the pixel a second reduction to 0.0 would give.
-    hh = hh + (hh < 0.0f ? 6.0f : (hh >= 6.0f ? -6.0f : 0.0f));
+    if constexpr (WRAP == HUE_WRAP_ONE) hh = hh + (hh >= wrap_t ? wrap_at : wrap_af);
+    else hh = hh + (hh < 0.0f ? 6.0f : (hh >= 6.0f ? -6.0f : 0.0f));
     s = s * satf;
     s = __builtin_fminf(__builtin_fmaxf(s, 0.0f), 1.0f);
     // sector and fraction; hh lies in [0, 6], where hh - floor(hh) is exact and equals hh - trunc(hh)

@@ -65,3 +65,10 @@ struct RmxKArgs {
 };
 
 #define RMX_WAVE 64
+
+// Hue shift of a sample in sextants (ColorTwist, Hue, Saturation). A pixel's hue before it is brought back into [0, 6] lies in
+// [shift - 1.0000002, shift + 5.0000002]; below RMX_HUE_SHIFT_LOW it can never reach 6, from RMX_HUE_SHIFT_HIGH on never fall
+// below 0, and one comparison brings it back. The host picks the twist kernel with the single comparison for batches in
+// which every sample's shift is on one side or the other; the kernel tells the sides apart with the same comparison.
+#define RMX_HUE_SHIFT_LOW 0.99998f
+#define RMX_HUE_SHIFT_HIGH 1.00002f

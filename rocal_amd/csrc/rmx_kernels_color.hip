@@ -11,14 +11,18 @@
 
 namespace rmx {
 
-enum { COLOR_LINEAR = 0, COLOR_TWIST = 1 };
+// COLOR_TWIST1: the twist for batches in which no sample's hue shift lies within 2e-5 of one sextant (one comparison brings
+// the hue back into range, see HueWrap)
+enum { COLOR_LINEAR = 0, COLOR_TWIST = 1, COLOR_TWIST1 = 2 };
 
 
 // MODE: 0 the general form; 1 whole 8-pixel groups and 16-byte aligned destination rows; 2 rows of 8 pixels and more at any
 // alignment: the pipeline of 1, the short last group of a row moved left until it is whole (it recomputes up to seven pixels of
 // its neighbour and stores the same values to the same places), groups stored at the element's own alignment.
-template <typename T, int LAYOUT, int KIND, int MODE>
+template <typename T, int LAYOUT, int KIND_ARG, int MODE>
 __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
+    constexpr int KIND = KIND_ARG == COLOR_TWIST1 ? COLOR_TWIST : KIND_ARG;
+    constexpr int WRAP = KIND_ARG == COLOR_TWIST1 ? HUE_WRAP_ONE : HUE_WRAP_BOTH;
     constexpr bool FAST = MODE != 0;
     constexpr bool ANY = MODE == 2;
     __shared__ ColorTables tabs;
@@ -68,11 +72,14 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     // between them is two selects per pixel (from scalar registers the compiler selects a constant and adds the shift again)
     float sh0 = p2, sh2 = p2 + 2.0f, sh4 = p2 + 4.0f;
     if constexpr (KIND == COLOR_TWIST) asm volatile("" : "+v"(sh0), "+v"(sh2), "+v"(sh4));
+    const HueWrap hw = hue_wrap_of(p2);
+    float wrap_t = hw.t, wrap_at = hw.at, wrap_af = hw.af;
+    if constexpr (WRAP == HUE_WRAP_ONE) asm volatile("" : "+v"(wrap_t), "+v"(wrap_at), "+v"(wrap_af));
     auto colour = [&](float (&v)[3][PX]) {
 #pragma unroll
         for (int k = 0; k < PX; k++) {
             if constexpr (KIND == COLOR_TWIST) {
-                twist_px(v[0][k], v[1][k], v[2][k], rcp, sect, p0, p1, sh0, sh2, sh4, p3);
+                twist_px<WRAP>(v[0][k], v[1][k], v[2][k], rcp, sect, p0, p1, sh0, sh2, sh4, p3, wrap_t, wrap_at, wrap_af);
             } else {
 #pragma unroll
                 for (int c = 0; c < 3; c++) v[c][k] = __builtin_fmaf(v[c][k] - p2, p0, p1);
@@ -174,8 +181,10 @@ static KernelFn pick_mode(int mode, int dtype, int layout) {
     return mode == 1 ? pick<KIND, 1>(dtype, layout) : (mode == 2 ? pick<KIND, 2>(dtype, layout) : pick<KIND, 0>(dtype, layout));
 }
 
+// kind: 0 linear, 1 twist, 2 twist for batches whose hue shifts all allow the single comparison
 KernelFn select_color_kernel(int kind, int dtype, int layout, int mode, const char **name) {
     *name = "rmx_color_kernel";
+    if (kind == COLOR_TWIST1) return pick_mode<COLOR_TWIST1>(mode, dtype, layout);
     return kind == COLOR_TWIST ? pick_mode<COLOR_TWIST>(mode, dtype, layout) : pick_mode<COLOR_LINEAR>(mode, dtype, layout);
 }
 

@@ -289,7 +289,10 @@ def test_color_family_fixed_params(ctx):
            orc.color_twist(img, roi, one(0.2), one(10.0), one(100.0), one(0.25)), ops.UINT8, what="twist fixed")
 
 
-def test_color_twist_all_rgb_values(ctx):
+# hue sets: far from one sextant (60 degrees) on both sides: the kernel that brings the hue back into range with one comparison;
+# at and next to 60 degrees: the kernel with both comparisons; just outside the band around 60 in which both are kept
+@pytest.mark.parametrize("hue", [(0.0, -18.0, 127.3, 359.9), (60.0, 59.9995, 60.0005, 420.0), (59.99, 60.01, 59.0, 61.0), (30.0, 359.99999, -0.00001, 300.0)])
+def test_color_twist_all_rgb_values(ctx, hue):
     """Every (r,g,b) triple on a 64-step lattice plus the extremes, several parameter sets."""
     v = np.unique(np.concatenate([np.arange(0, 256, 5), [1, 2, 254, 255]])).astype(np.uint8)
     r, g, b = np.meshgrid(v, v, v, indexing="ij")
@@ -302,7 +305,7 @@ def test_color_twist_all_rgb_values(ctx):
     roi = np.tile(np.array([0, 0, W, H], np.uint32), (n, 1))
     alpha = np.array([1.0, 0.7, 1.3, 1.95], np.float32)
     beta = np.array([0.0, 12.5, -7.25, 25.0], np.float32)
-    hue = np.array([0.0, -18.0, 127.3, 359.9], np.float32)
+    hue = np.array(hue, np.float32)
     sat = np.array([1.0, 0.0, 1.4, 0.37], np.float32)
     exp = orc.color_twist(img, roi, alpha, beta, hue, sat)
     sd = ops.desc(n, H, W, ops.NHWC, ops.UINT8)
