@@ -95,7 +95,9 @@ RMX_DEV uint32_t elem_bits(float v) {
 // SLOTS: output rows in flight. Four cover every downscale (rows four apart never share a source row); eight cover samples
 // that grow vertically by up to about 3.8 (two taps, several output rows per source row; 113 registers, four wavefronts per
 // SIMD), so that a batch of RandomResizedCrop windows, some of which shrink and some of which grow, stays in this kernel
-// (measured on 256 such windows to 224 x 224: 160 us through the ring kernel). Two are enough when
+// (measured on 256 such windows to 224 x 224: 160 us through the ring kernel; in that kernel a sample that shrinks runs a row
+// loop of its own that adds to the lower four sets only, and windows with two or three horizontal taps have their own
+// unrolled passes: 70.2 -> 67.2 us on those windows). Two are enough when
 // rows two apart never do, which the host establishes for ratios that are whole or half numbers (1080 -> 360 rows, any
 // decimation by 2, 3, 4 or 1.5): every source row then enters two accumulator sets instead of four.
 template <typename T, int LAYOUT, bool NORM, bool QUANT, int SLOTS>
@@ -131,6 +133,10 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
     const int pcx = P.pc_x, pcy = P.pc_y;
     const TriAxis ax = tri_axis(P.rx, P.fsx), ay = tri_axis(P.ry, P.fsy);
     const int kx = to_sgpr(ax.ksize), ky = to_sgpr(ay.ksize);
+    // Accumulator sets this sample uses: output row r lives in set (r - r0) & smask. A sample that shrinks vertically never has
+    // more than four rows in flight (the host has established that for every sample with a vertical ratio of 1 and more), so
+    // in the kernel with eight sets it leaves the upper four alone: half the vertical FMAs per source row.
+    const int smask = SLOTS == 8 ? to_sgpr(P.ry >= 1.0f ? 3 : 7) : SLOTS - 1;
 
     // (a sample is smaller than 4 GiB: the host checks it, so offsets inside a sample are 32-bit)
     uint32_t row_stride_v;
@@ -341,11 +347,11 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
         float cf[TS_SLOTS];
 #pragma unroll
         for (int k = 0; k < TS_SLOTS; k++) cf[k] = 0.0f;
-        for (int rb = r0; rb < r1; rb += TS_SLOTS) {
+        for (int rb = r0; rb < r1; rb += smask + 1) {
 #pragma unroll
             for (int k = 0; k < TS_SLOTS; k++) {
                 const int r = rb + k;
-                if (r < r1) {
+                if (k <= smask && r < r1) {
                     const int j = y - row_loc(r);
                     const float c = tri_coeff(row_w0(r), ay.radius, j, ay.fscale);
                     if ((uint32_t)j < (uint32_t)ky) cf[k] = c;
@@ -402,8 +408,12 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
     // unrolled horizontal pass (4, 5, 6 or 8 >= the taps that are run): taps beyond those carry coefficient 0 (fma(p, 0, a) == a
     // for the finite p an unpacked byte always is), so no bound test is needed inside. A column's 3 NT bytes start at byte
     // tap_ph of dword tap_w: NE + 1 dwords are read and realigned into NE.
-    auto process_row = [&](auto nt, const lds_u8 *srow, int yy) {
+    auto process_row = [&](auto nt, auto lower_only, const lds_u8 *srow, int yy) {
         constexpr int NT = decltype(nt)::value;
+        // LIVE: the accumulator sets this instance of the row loop adds to and stores from (the lower four of eight for a sample
+        // that shrinks: a loop of its own rather than a branch around the upper sets' FMAs, at whose join the accumulators
+        // would be copied)
+        constexpr int LIVE = (TS_SLOTS == 8 && decltype(lower_only)::value) ? 4 : TS_SLOTS;
         constexpr int NE = (3 * NT + 3) / 4;
         // A row inside the window is one tap of every output row that reads it: one pass, coefficients from the table. The
         // first / last row of the window is also read by every tap index that leaves the window: one pass per such tap, in
@@ -415,9 +425,9 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
             npass = 0;
 #pragma unroll
             for (int m = 0; m < TS_SLOTS; m++) {
-                const int r = rq + ((m - (rq - r0)) & (TS_SLOTS - 1));  // the row in flight that lives in slot m
+                const int r = rq + ((m - (rq - r0)) & smask);  // the row in flight that lives in slot m
                 ec[m] = 0.0f;
-                if (r < r1) {
+                if (m <= smask && r < r1) {
                     const int loc = row_loc(r);
                     const int jlo = max((yy == ylo) ? 0 : yy - loc, 0);
                     const int jhi = min((yy == yhi) ? ky - 1 : yy - loc, ky - 1);
@@ -459,7 +469,7 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
         // ---- vertical pass: every pass adds the filtered row to all four slots with that pass's coefficients (0: none)
         for (int p = 0;;) {
 #pragma unroll
-            for (int m = 0; m < TS_SLOTS; m++)
+            for (int m = 0; m < LIVE; m++)
 #pragma unroll
                 for (int ch = 0; ch < 3; ch++)
 #pragma unroll
@@ -472,7 +482,7 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
             if constexpr (TS_SLOTS == 2) {
                 if (rsum_idx & 1) emit(std::integral_constant<int, 1>{});
                 else emit(std::integral_constant<int, 0>{});
-            } else if constexpr (TS_SLOTS == 8) {
+            } else if constexpr (LIVE == 8) {
                 switch (rsum_idx & 7) {
                     case 0: emit(std::integral_constant<int, 0>{}); break;
                     case 1: emit(std::integral_constant<int, 1>{}); break;
@@ -505,7 +515,7 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
     // since those loads (6 per output row, see store_elem), so it never waits for a store. The next step's loads are
     // started right behind the wait (the slots they fill were read for the last time in the step before).
     constexpr int NS = 3 * TPX;  // store instructions per output row
-    auto run = [&](auto nt) {
+    auto run = [&](auto nt, auto lower_only) {
         lds_u8 *half_cur = bufb, *half_nxt = bufb + TS_RPS * pitch;
         bool by_lanes = issue(half_cur);
         build_table();  // (under the round trip of the first loads)
@@ -524,17 +534,24 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
             emitted = 0;
             by_lanes = (y + TS_RPS <= y_last) ? issue(half_nxt) : false;
             replicate(half_cur, nr);
-            for (int q = 0; q < nr; q++) process_row(nt, half_cur + q * pitch, y + q);
+            for (int q = 0; q < nr; q++) process_row(nt, lower_only, half_cur + q * pitch, y + q);
             wave_sync();  // the slots are reused two steps on
             lds_u8 *t = half_cur;
             half_cur = half_nxt;
             half_nxt = t;
         }
     };
-    if (kx_run <= 4) run(std::integral_constant<int, 4>{});
-    else if (kx_run == 5) run(std::integral_constant<int, 5>{});
-    else if (kx_run <= 6) run(std::integral_constant<int, 6>{});
-    else run(std::integral_constant<int, 8>{});
+    // (two and three taps: windows that grow or barely shrink horizontally, which only batches with growing samples hold in numbers)
+    auto run_taps = [&](auto lower_only) {
+        if (SLOTS == 8 && kx_run <= 2) run(std::integral_constant<int, SLOTS == 8 ? 2 : 4>{}, lower_only);
+        else if (SLOTS == 8 && kx_run == 3) run(std::integral_constant<int, SLOTS == 8 ? 3 : 4>{}, lower_only);
+        else if (kx_run <= 4) run(std::integral_constant<int, 4>{}, lower_only);
+        else if (kx_run == 5) run(std::integral_constant<int, 5>{}, lower_only);
+        else if (kx_run <= 6) run(std::integral_constant<int, 6>{}, lower_only);
+        else run(std::integral_constant<int, 8>{}, lower_only);
+    };
+    if (SLOTS == 8 && smask == 3) run_taps(std::integral_constant<bool, SLOTS == 8>{});
+    else run_taps(std::false_type{});
 }
 
 template <typename T, int LAYOUT, int SLOTS>

@@ -69,11 +69,13 @@ def test_streaming_triangular_kernel_counts_its_stores():
             continue
         body = f.split("s_endpgm")[0]
         stores = re.findall(r"^\s*(global_store_\w+|flat_store_\w+|buffer_store_\w+|scratch_\w+)", body, re.M)
-        # four tap-count variants of the row loop x accumulator slots (the kernel's last template argument: 2, 4 or 8 rows in
-        # flight) x (two columns x three channels)
+        # tap-count variants of the row loop x accumulator sets it stores from x (two columns x three channels). The kernel's
+        # last template argument is the number of sets: 2, 4 or 8; the kernel with eight has six tap-count variants instead of
+        # four and every one twice, for samples that use all eight sets and for samples that use the lower four
         slots = int(re.search(r"Li(\d)EEEv8RmxKArgs$", m.group(1)).group(1))
         assert slots in (2, 4, 8)
-        assert len(stores) == 4 * slots * 6, "%s: %d store instructions" % (m.group(1), len(stores))
+        expected = 6 * (8 + 4) * 6 if slots == 8 else 4 * slots * 6
+        assert len(stores) == expected, "%s: %d store instructions" % (m.group(1), len(stores))
         assert len(set(stores)) == 1 and stores[0].startswith("global_store_"), "%s: %s" % (m.group(1), sorted(set(stores)))
         waits = sorted(set(int(x) for x in re.findall(r"s_waitcnt vmcnt\((\d+)\)", body)))
         assert set(waits) <= {0, 6, 12}, "%s: waits %s" % (m.group(1), waits)
