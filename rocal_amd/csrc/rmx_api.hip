@@ -87,7 +87,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 4, k3_rows = 8, k3_flat_rows = 0, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, flat_frames = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_slots = 0, tri_per_cu = 0, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k3_rows = 8, k3_flat_rows = 0, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, flat_frames = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_slots = 0, tri_per_cu = 0, tri_sort = 1, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -409,6 +409,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->tri_tpx = tune_env("RMX_TUNE_TRI_TPX", ctx->tri_tpx, 1, 2);     // output columns per lane of the downscaling kernel
         ctx->tri_slots = tune_env("RMX_TUNE_TRI_SLOTS", ctx->tri_slots, 0, 4);  // 4: the streaming triangular kernel always keeps four rows in flight (batches that need eight go to the ring kernel)
         ctx->deal_xcd = tune_env("RMX_TUNE_DEAL_XCD", ctx->deal_xcd, 0, 1);  // samples dealt round-robin to the XCDs (0: eight runs in batch order)
+        ctx->tri_sort = tune_env("RMX_TUNE_TRI_SORT", ctx->tri_sort, 0, 1);  // rows of batches of uneven cost go largest window first
         ctx->tri_per_cu = tune_env("RMX_TUNE_TRI_PER_CU", ctx->tri_per_cu, 0, 32);  // wavefronts per CU the strip planner counts on (0: by registers and LDS)
     }
     *out = ctx;
@@ -981,6 +982,7 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             }
         }
         int rows = op->ctx->tri_rows > 0 ? op->ctx->tri_rows : 12;
+        bool sort_rows = false;
         // Streaming form of the downscaling variant (source rows straight into LDS as raw bytes): every source row must start
         // at the same byte phase (row stride a multiple of 4), and four LDS rows of the widest tile plus the table of vertical
         // coefficients must leave room for ten wavefronts per CU at least.
@@ -1086,27 +1088,31 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
             // rounds of (wavefront slots) at a time; pick the R with the least rounds x rows-per-strip. Measured on
             // MI355X: a batch of equal strips that march in step runs 10-20 % slower than one whose last strip of each
             // image is a short one, so an R that leaves a remainder of at most R/2 rows is preferred.
+            // A batch whose samples differ in vertical ratio (RandomResizedCrop windows: a strip of one sample filters
+            // several times the source rows of a strip of another)
+            float min_ry = max_ry;
+            for (int i = 0; i < op->n; i++)
+                if (t[i].dst_w > 0 && t[i].dst_h > 0) min_ry = std::min(min_ry, t[i].ry);
+            const bool ragged_cost = max_ry > 1.5f * min_ry;
+            sort_rows = ragged_cost;
             if (op->ctx->tri_rows == 0) {
                 // (wavefronts per CU: 16 by the registers of the kernel that stages through registers, 20 by those of the streaming
                 // one, 24 when it keeps two rows in flight)
                 const int by_regs = tdma ? (op->tri_rows_in_flight == 2 ? 24 : (op->tri_rows_in_flight == 8 ? 16 : 20)) : 16;
                 const int per_cu = op->ctx->tri_per_cu > 0 ? op->ctx->tri_per_cu : std::max(1, std::min(by_regs, (160 * 1024) / op->lds_per_wave));
                 const long slots = (long)op->ctx->num_cus * per_cu;
-                // A batch whose samples differ in vertical ratio (RandomResizedCrop windows: a strip of one sample filters
-                // several times the source rows of a strip of another) is only spread evenly over the device when there
-                // are several strips per wavefront slot for the hardware to deal out as slots fall free. Measured on 256
-                // such windows to 224 x 224: strips of 30 rows (one per slot) 80.9 us, of 8 rows (3.5 per slot) 69.2 us.
-                float min_ry = max_ry;
-                for (int i = 0; i < op->n; i++)
-                    if (t[i].dst_w > 0 && t[i].dst_h > 0) min_ry = std::min(min_ry, t[i].ry);
-                const bool ragged_cost = max_ry > 1.5f * min_ry;
+                // Such a batch is only spread evenly over the device when there are several strips per wavefront slot for the
+                // hardware to deal out as slots fall free. Measured on 256 such windows to 224 x 224: strips of 30 rows (one
+                // per slot) 80.9 us, of 8 rows (3.5 per slot) 69.2 us.
                 double best_cost = 0.0;
                 for (int r = 4; r <= 64; r++) {
                     long waves = 0;
                     for (int i = 0; i < op->n; i++)
                         if (t[i].dst_w > 0 && t[i].dst_h > 0) waves += (long)((t[i].dst_w + tile_w - 1) / tile_w) * ((t[i].dst_h + r - 1) / r);
-                    if (ragged_cost) {  // the tallest strips that still leave three per slot
-                        if (r > 4 && waves < 3 * slots) break;
+                    if (ragged_cost) {
+                        // the tallest strips that still leave three per slot; two when the rows go out largest window first (below),
+                        // which evens the slots out by itself (same windows, sorted: strips of 9 / 14 / 19 rows 62.8 / 57.1 / 62.8 us)
+                        if (r > 4 && waves < (op->ctx->tri_sort ? 2 : 3) * slots) break;
                         rows = r;
                         continue;
                     }
@@ -1129,6 +1135,19 @@ static int plan_resize(rmx_op *op, RmxSample *t, bool norm) {
         const int ystrips = (max_dh + op->strip_rows - 1) / op->strip_rows;
         op->strips = xtiles * ystrips;
         for (int i = 0; i < op->n; i++) t[i].strip_rows = (ring_rows << 16) | kx_cap;
+        // A batch whose samples differ in cost goes to the device largest window first: the hardware deals the strips out in
+        // launch order as wavefront slots fall free, so the launch ends with the small windows instead of waiting for a
+        // large one that started late (measured on 256 RandomResizedCrop windows: 66.4 -> 62.2 us). Only the ROWS change
+        // places; each carries its sample's index (plan[2]), from which the kernels address source and destination.
+        if (sort_rows && op->ctx->tri_sort) {
+            std::vector<int> order(op->n);
+            for (int i = 0; i < op->n; i++) order[i] = i;
+            std::stable_sort(order.begin(), order.end(), [&](int x, int y) {
+                return (int64_t)t[x].src_w * t[x].src_h > (int64_t)t[y].src_w * t[y].src_h;
+            });
+            std::vector<RmxSample> rows(t, t + op->n);
+            for (int i = 0; i < op->n; i++) t[i] = rows[order[i]];
+        }
         return RMX_OK;
     }
     const char *nm = nullptr;
@@ -1336,6 +1355,7 @@ static int fill_resize_rows(rmx_op *op, RmxSample *t, const uint32_t *src_roi, c
         } else {
             s.rx = s.ry = s.fsx = s.fsy = 1.0f;
         }
+        s.plan[2] = i;  // the sample this row belongs to (the triangular kernels take it from here: their rows may be reordered)
         for (int c = 0; c < 3; c++) {
             if (scale) {
                 s.scale[c] = scale[i * 3 + c];

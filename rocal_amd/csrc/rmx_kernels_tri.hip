@@ -43,6 +43,7 @@ __global__ void __launch_bounds__(256) rmx_resize_tri_kernel(RmxKArgs a) {
     const int tiles_x = a.aux1;
     const int strip = part / tiles_x, tx = part - strip * tiles_x;
     const RmxSample &P = a.table[s];
+    s = P.plan[2];  // (the host may have put the rows in another order: the row names its sample)
 
     const int dw = P.dst_w, dh = P.dst_h;
     const int srows = a.aux0;
@@ -312,6 +313,7 @@ __global__ void __launch_bounds__(256, RMX_TRI_DOWN_WAVES(NPX)) rmx_resize_tri_d
     // the whole table row in one round trip
     const RmxSample P = a.table[s];
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.fsx));
+    s = P.plan[2];  // (the host may have put the rows in another order: the row names its sample)
 
     const int dw = P.dst_w, dh = P.dst_h;
     const int srows = a.aux0;

@@ -120,6 +120,7 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
     // the whole table row in one round trip
     const RmxSample P = a.table[s];
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.pc_x), "s"(P.flags), "s"(P.rx), "s"(P.scale[0]), "s"(P.bias[2]), "s"(P.fsx));
+    s = P.plan[2];  // (the host may have put the rows in another order: the row names its sample)
 
     const int dw = P.dst_w, dh = P.dst_h;
     const int srows = a.aux0;

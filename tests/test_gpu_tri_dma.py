@@ -307,10 +307,12 @@ def _packed(rng, widths, heights, gaps):
     return packed, np.array(offsets, np.uint64), strides.astype(np.uint32), padded
 
 
-def test_packed_source_with_rows_at_multiples_of_four(ctx):
+@pytest.mark.parametrize("heights_out", [(50, 40, 31, 60), (60, 60, 60, 20)])
+def test_packed_source_with_rows_at_multiples_of_four(ctx, heights_out):
     """Packed images (a byte offset and a row stride per image, strides multiples of 4, bases at byte phases 0, 1, 2, 3) in an
     exact-size buffer: the last rows of the last image end on the last bytes of the buffer and are staged by the lanes with
-    bounds-checked loads."""
+    bounds-checked loads. The second set of output heights makes the vertical ratios differ by more than 1.5 (2.0 .. 7.5): the
+    table rows of such a batch go to the device largest window first, each naming its sample."""
     rng = np.random.default_rng(8)
     n = 4
     widths = np.array([300, 257, 128, 400], np.uint32)
@@ -320,7 +322,7 @@ def test_packed_source_with_rows_at_multiples_of_four(ctx):
     roi = np.array([[0, 0, widths[i], heights[i]] for i in range(n)], np.uint32)
     roi[1] = (3, 2, 250, 85)
     dw = np.array([140, 100, 64, 180], np.uint32)
-    dh = np.array([50, 40, 31, 60], np.uint32)
+    dh = np.array(heights_out, np.uint32)
     mirror = np.array([0, 1, 1, 0], np.uint32)
     scale, bias = _scale_bias(n)
     exp = orc.resize(padded, roi, dw, dh, 60, 180, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
