@@ -260,6 +260,10 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
         return by_lanes;
     };
 
+    // The first two rows are asked for here, ahead of the coefficient set-up below (some hundred instructions that need no
+    // memory): they travel while it runs.
+    const bool first_by_lanes = issue(bufb);
+
     // ---- per-lane columns: taps, coefficients (registers), column sums, destination column (mirrored if asked)
     // (a lane whose column lies beyond the row takes the last column again and stores the same value to the same place:
     // every store instruction is then issued by every wavefront, which the count in the wait below relies on)
@@ -518,7 +522,7 @@ __global__ void __launch_bounds__(256, SLOTS == 8 ? 4 : RMX_TDMA_WAVES) rmx_resi
     constexpr int NS = 3 * TPX;  // store instructions per output row
     auto run = [&](auto nt, auto lower_only) {
         lds_u8 *half_cur = bufb, *half_nxt = bufb + TS_RPS * pitch;
-        bool by_lanes = issue(half_cur);
+        bool by_lanes = first_by_lanes;
         build_table();  // (under the round trip of the first loads)
         for (int y = y_first; y <= y_last; y += TS_RPS) {
             const int nr = min(TS_RPS, y_last - y + 1);
