@@ -27,11 +27,22 @@ def _newest_header():
     return max(os.path.getmtime(h) for h in glob.glob(os.path.join(CSRC, "*.h")) + [os.path.join(HERE, "..", "include", "rocal_mi355x.h")])
 
 
+# Sources whose generated code the CPU tests read (explicit wait counts that rely on how many instructions the compiler makes):
+# their device assembly is kept next to the object, so that the tests need not compile them a second time.
+KEEP_ASSEMBLY = ("rmx_kernels_resize_dma.hip", "rmx_kernels_tri_dma_2.hip", "rmx_kernels_tri_dma_4.hip", "rmx_kernels_tri_dma_8_nchw.hip",
+                 "rmx_kernels_tri_dma_8_nhwc.hip", "rmx_kernels_warp.hip")
+
+
+def assembly_path(src_name):
+    return os.path.join(OBJDIR, os.path.splitext(src_name)[0] + "-hip-amdgcn-amd-amdhsa-gfx950.s")
+
+
 def _compile(src, incremental=False):
     obj = os.path.join(OBJDIR, os.path.basename(src) + ".o")
     if incremental and os.path.exists(obj) and os.path.getmtime(obj) > max(os.path.getmtime(src), _newest_header()):
         return obj, ""
-    cmd = [HIPCC] + FLAGS + os.environ.get("RMX_EXTRA_FLAGS", "").split() + ["-c", src, "-o", obj]
+    keep = ["-save-temps=obj"] if os.path.basename(src) in KEEP_ASSEMBLY else []
+    cmd = [HIPCC] + FLAGS + keep + os.environ.get("RMX_EXTRA_FLAGS", "").split() + ["-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature name: that warning is expected
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)

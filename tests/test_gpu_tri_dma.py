@@ -189,12 +189,15 @@ def test_random_whole_and_half_ratios_with_a_crop_behind_the_resize(ctx, seed):
     _check_windows(out.cpu().numpy(), exp, crop[:, 2], crop[:, 3], ops.NCHW, 5, "seed %d (%s)" % (seed, op.plan))
 
 
-@pytest.mark.parametrize("rx", [1, 3, 5])
-def test_odd_whole_horizontal_ratios_skip_their_first_tap(ctx, ctx_staged, rx):
+@pytest.mark.parametrize("rx,layout,dtype", [(1, ops.NCHW, ops.FP16), (2, ops.NCHW, ops.FP16), (3, ops.NCHW, ops.FP16), (5, ops.NCHW, ops.FP16),
+                                             (2, ops.NHWC, ops.UINT8), (3, ops.NHWC, ops.FP32)])
+def test_whole_horizontal_ratios(ctx, ctx_staged, rx, layout, dtype):
     """Horizontal ratios 1 and 3: the first tap of every column has coefficient 0 and the streaming kernel runs one tap less
-    (1 and 5 taps: its 4- and 5-tap passes); ratio 5 has ten taps and goes to the ring kernel. Windows at the left and right
-    end of the source (replicas), in the middle, mirrored; a second tile (more than 128 columns); a batch with one window of
-    another ratio, whose wavefronts keep the first tap. Against the oracle, also through the kernel that stages through registers."""
+    (1 and 5 taps: its 4- and 5-tap passes); ratio 5 has ten taps and goes to the ring kernel. Ratios 2 and 3: a lane takes two
+    NEIGHBOURING columns and reads the union of their taps once (rows of even width: 150 = a tile of 128 and one of 22, and 140;
+    the row of 31 columns keeps the columns 64 apart). Windows at the left and right end of the source (replicas), in the
+    middle, mirrored; a second tile (more than 128 columns); a batch with one window of another ratio, whose wavefronts keep
+    the first tap and the columns apart. Against the oracle, also through the kernel that stages through registers."""
     rng = np.random.default_rng(50 + rx)
     n, OH, OW = 4, 24, 150
     dw = np.array([OW, 140, 31, 150], np.uint32)
@@ -207,16 +210,21 @@ def test_odd_whole_horizontal_ratios_skip_their_first_tap(ctx, ctx_staged, rx):
     dh = np.array([OH, 20, 18, 24], np.uint32)
     mirror = np.array([0, 1, 0, 1], np.uint32)
     scale, bias = _scale_bias(n)
-    exp = orc.resize(img, roi, dw, dh, OH, OW, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+    norm = dtype != ops.UINT8
+    kw = dict(interp=orc.TRIANGULAR, mirror=mirror, scale=scale if norm else None, bias=bias if norm else None, layout=layout, dtype=dtype)
+    exp = orc.resize(img, roi, dw, dh, OH, OW, **kw)
     for c in (ctx, ctx_staged):
-        op = ops.Resize(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, ops.NCHW, ops.FP16), ops.TRIANGULAR)
-        op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        op = ops.Resize(c, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, layout, dtype), ops.TRIANGULAR)
+        if norm:
+            op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        else:
+            op.update(roi, dw, dh, mirror)
         if c is ctx:
             assert op.kernel_name == ("rmx_resize_tri_dma_kernel" if rx < 5 else "rmx_resize_tri_kernel"), op.plan
         out = op.alloc_output(fill=9)
         op.launch(_gpu(img), out)
         c.sync()
-        _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 9, "rx=%d %s" % (rx, op.kernel_name))
+        _check_windows(out.cpu().numpy(), exp, dw, dh, layout, 9, "rx=%d %s" % (rx, op.kernel_name))
 
 
 @pytest.mark.parametrize("layout,dtype", [(ops.NCHW, ops.FP16), (ops.NHWC, ops.UINT8), (ops.NCHW, ops.FP32)])
