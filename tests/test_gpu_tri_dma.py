@@ -373,3 +373,28 @@ def test_warp_on_a_packed_source_with_rows_at_multiples_of_four(ctx, interp):
     got = out.cpu().numpy()
     for i in range(n):
         assert np.array_equal(got[i, :dh[i], :dw[i]], exp[i, :dh[i], :dw[i]]), "sample %d: %d values differ" % (i, int((got[i, :dh[i], :dw[i]] != exp[i, :dh[i], :dw[i]]).sum()))
+
+
+def test_rows_in_another_order_with_an_empty_sample(ctx):
+    """A batch of uneven cost (vertical ratios 0.6 .. 3, so its table rows go to the device largest window first) in which one
+    sample has an empty destination: that sample's output stays untouched wherever its row ends up, the others match the
+    oracle, and a second update of the same op with other windows (another order) does too."""
+    rng = np.random.default_rng(77)
+    n, H, W, OH, OW = 5, 96, 100, 32, 32
+    img = wl.smooth_noise(rng, n, H, W, sigma=1.0)
+    scale, bias = _scale_bias(n)
+    op = ops.Resize(ctx, ops.desc(n, H, W, ops.NHWC, ops.UINT8), ops.desc(n, OH, OW, ops.NCHW, ops.FP16), ops.TRIANGULAR)
+    src = _gpu(img)
+    for roi in ([[0, 0, 64, 64], [3, 5, 40, 40], [10, 10, 20, 20], [0, 0, 50, 50], [2, 1, 96, 90]],
+                [[1, 1, 20, 19], [0, 0, 100, 96], [7, 9, 33, 41], [0, 0, 50, 50], [5, 5, 64, 60]]):
+        roi = np.array(roi, np.uint32)
+        dw = np.array([32, 32, 32, 0, 32], np.uint32)
+        dh = np.array([32, 32, 32, 32, 30], np.uint32)
+        mirror = np.array([1, 0, 0, 1, 0], np.uint32)
+        op.update_cmn(roi, dw, dh, scale, bias, mirror)
+        assert op.kernel_name == "rmx_resize_tri_dma_kernel" and "rows_in_flight=8" in op.plan, op.plan
+        out = op.alloc_output(fill=5)
+        op.launch(src, out)
+        ctx.sync()
+        exp = orc.resize(img, roi, np.maximum(dw, 1), dh, OH, OW, interp=orc.TRIANGULAR, mirror=mirror, scale=scale, bias=bias, layout=ops.NCHW, dtype=ops.FP16)
+        _check_windows(out.cpu().numpy(), exp, dw, dh, ops.NCHW, 5, "sorted rows")
