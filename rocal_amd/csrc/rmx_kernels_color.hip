@@ -28,12 +28,15 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     __shared__ ColorTables tabs;
     const float *rcp = tabs.rcp;
     const SectorRow *sect = tabs.sect;
+    // The workgroup copies the two tables of the twist from device memory into LDS, 16 bytes per thread (two for the first
+    // threads of a workgroup of one wavefront). The reads are started here and written to LDS behind the fetch of the table
+    // row below, so that the two round trips overlap.
+    constexpr unsigned TAB_PIECES = sizeof(ColorTables) / 16;
+    uint4 tab0 = {}, tab1 = {};
     if constexpr (KIND == COLOR_TWIST) {
-        // the workgroup copies the two tables of the twist from device memory into LDS, 16 bytes per thread
         const uint4 *rom = reinterpret_cast<const uint4 *>(&rmx_color_tables_rom);
-        uint4 *ram = reinterpret_cast<uint4 *>(&tabs);
-        for (unsigned i = threadIdx.x; i < sizeof(ColorTables) / 16; i += blockDim.x) ram[i] = rom[i];
-        __syncthreads();
+        if (threadIdx.x < TAB_PIECES) tab0 = rom[threadIdx.x];
+        if (threadIdx.x + blockDim.x < TAB_PIECES) tab1 = rom[threadIdx.x + blockDim.x];
     }
     const int lane = threadIdx.x & (RMX_WAVE - 1);
     // fp32 and interleaved fp16 outputs: the lanes of a row exchange their runs through LDS before storing (store_packed_coalesced)
@@ -46,14 +49,21 @@ __global__ void __launch_bounds__(256) rmx_color_kernel(RmxKArgs a) {
     const uint32_t nwaves = (uint32_t)a.n * (uint32_t)a.strips;
     uint32_t wave = blockIdx.x * (uint32_t)a.wpb + (threadIdx.x / RMX_WAVE);
     wave = __builtin_amdgcn_readfirstlane(wave);
-    if (wave >= nwaves) return;
     int s, strip;
     // workgroups in launch order (no XCD renumbering): the whole device walks the batch as one contiguous address stream,
     // and dealing the samples would only break that stream up (measured: 11-16 % slower)
-    wave_to_sample(a, wave, s, strip, false);
-    // whole table row in one round trip (the empty statement keeps the fetch above the early exit)
+    // (a wavefront beyond the batch fetches the last wavefront's row: it stays for the workgroup's barrier and leaves then)
+    wave_to_sample(a, min(wave, nwaves - 1), s, strip, false);
+    // whole table row in one round trip (the empty statement keeps the fetch above the barrier and the early exit)
     const RmxSample P = a.table[s];
     asm volatile("" : : "s"(P.src_x), "s"(P.dst_w), "s"(P.flags), "s"(P.color[0]), "s"(P.color[3]));
+    if constexpr (KIND == COLOR_TWIST) {
+        uint4 *ram = reinterpret_cast<uint4 *>(&tabs);
+        if (threadIdx.x < TAB_PIECES) ram[threadIdx.x] = tab0;
+        if (threadIdx.x + blockDim.x < TAB_PIECES) ram[threadIdx.x + blockDim.x] = tab1;
+        __syncthreads();
+    }
+    if (wave >= nwaves) return;
     const int w = P.dst_w, h = P.dst_h;
     const int srows = a.aux0;
     const int r0 = strip * srows;
