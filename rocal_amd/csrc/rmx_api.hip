@@ -87,7 +87,7 @@ struct rmx_ctx {
     // Launch-plan tunables (rows per wavefront strip, LDS budget of the resize fast path). Defaults are the
     // values measured best on MI355X; RMX_TUNE_* environment variables, read once when the context is
     // created and clamped to safe ranges, override them for sweeps. They change plans, never results.
-    int k1_rows = 4, k3_rows = 8, k3_flat_rows = 0, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, flat_frames = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_slots = 0, tri_per_cu = 0, tri_sort = 1, warp_passes = 2, warp_wpb = 4;
+    int k1_rows = 4, k1_flat_rows = 0, k3_rows = 8, k3_flat_rows = 0, tri_rows = 0, gen_rows = 8, fast_rows = 4, fast_lds = 10 * 1024, fast_wpb = 1, dma = 1, dma_lds = 10 * 1024, dma_group = 1, flat_frames = 1, deal_xcd = 1, tri_wpb = 1, tri_ring = 0, tri_tpx = 2, tri_slots = 0, tri_per_cu = 0, tri_sort = 1, warp_passes = 2, warp_wpb = 4;
 };
 
 static int tune_env(const char *name, int def, int lo, int hi) {
@@ -392,6 +392,7 @@ int rmx_ctx_create(int device, void *stream, int own_stream, rmx_ctx **out) {
         ctx->k1_rows = tune_env("RMX_TUNE_CMN_ROWS", ctx->k1_rows, 1, 64);
         ctx->k3_rows = tune_env("RMX_TUNE_COLOR_ROWS", ctx->k3_rows, 1, 64);
         ctx->k3_flat_rows = tune_env("RMX_TUNE_COLOR_FLAT_ROWS", ctx->k3_flat_rows, 0, 64);  // 0: one row for the twist, two for the linear kinds
+        ctx->k1_flat_rows = tune_env("RMX_TUNE_K1_FLAT_ROWS", ctx->k1_flat_rows, 0, 16);  // rows of 512 pixels per wavefront, whole frames through the K1 kernel (0: by output type)
         ctx->tri_rows = tune_env("RMX_TUNE_TRI_ROWS", ctx->tri_rows, 0, 64);  // 0: chosen per batch
         ctx->gen_rows = tune_env("RMX_TUNE_RESIZE_ROWS", ctx->gen_rows, 1, 64);
         ctx->fast_rows = tune_env("RMX_TUNE_FAST_ROWS", ctx->fast_rows, 1, 64);
@@ -697,10 +698,21 @@ static int update_k1(rmx_op *op, const uint32_t *roi, const float *scale, const 
         max_rows = std::max(max_rows, (int)s.dst_h);
     }
     op->algo_bytes = bytes;
-    const int rows = op->ctx->k1_rows;
+    int rows = op->ctx->k1_rows;
+    // whole frames that are not mirrored (a mirror is a matter of rows): as rows of 512 pixels, like the colour family's
+    bool flipped = false;
+    for (int i = 0; i < op->n && !flipped; i++) flipped = (t[i].flags & (RMX_S_HFLIP | RMX_S_VFLIP)) != 0;
+    if (!flipped && flatten_whole_frames(op, t)) {
+        max_rows = op->flat_h;
+        // (256 frames of 224 x 224, 1 / 2 / 4 / 8 such rows per wavefront against strips of the images' own rows: u8 -> f16 planes
+        // 21.6 / 22.4 / 23.7 / 26.9 against 22.3 us, u8 -> u8 18.7 / 16.75 / 18.6 / 19.9 against 17.35 us)
+        rows = op->ctx->k1_flat_rows ? op->ctx->k1_flat_rows : (op->dst.dtype == RMX_UINT8 ? 2 : 1);
+    } else {
+        op->flat_h = 0;
+    }
     plan_streaming(op, max_rows, rows);
     // aligned specialisation: whole 8-pixel groups everywhere and 16-byte aligned destination rows
-    bool aligned = op->dst.w % 8 == 0;
+    bool aligned = op->flat_h ? true : op->dst.w % 8 == 0;
     for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
     op->fn_fast = nullptr;
     if (aligned) {
@@ -1623,8 +1635,15 @@ static int update_point(rmx_op *op, const uint32_t *roi, const float *p0, const 
         max_rows = std::max(max_rows, (int)s.dst_h);
     }
     op->algo_bytes = bytes;
-    plan_streaming(op, max_rows, op->ctx->k3_rows);
-    bool aligned = op->dst.w % 8 == 0;
+    int rows = op->ctx->k3_rows;
+    if (flatten_whole_frames(op, t)) {  // whole frames as rows of 512 pixels, as the colour family takes them
+        max_rows = op->flat_h;
+        // (256 frames of 224 x 224, 1 / 2 / 4 / 8 such rows per wavefront against the images' own rows: Gamma 16.9 / 17.2 / 18.7 /
+        // 20.6 against 18.1 us, Blend 24.4 / 22.8 / 25.0 / 27.1 against 23.9 us)
+        rows = op->ctx->k3_flat_rows ? op->ctx->k3_flat_rows : (op->kind == OP_GAMMA ? 1 : 2);
+    }
+    plan_streaming(op, max_rows, rows);
+    bool aligned = op->flat_h ? true : op->dst.w % 8 == 0;
     for (int i = 0; i < op->n && aligned; i++) aligned = (t[i].dst_w % 8 == 0);
     op->fn_fast = nullptr;
     if (aligned) {

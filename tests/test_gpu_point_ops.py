@@ -180,3 +180,50 @@ def test_wide_rows_take_several_tiles(ctx, layout, dtype):
     g = rng.uniform(0.3, 7.0, n).astype(np.float32)
     got, _ = _run(ctx, ops.Gamma, n, h, w, layout, dtype, lambda o: o.update(crop, g), [img])
     _same(got, orc.gamma(img, crop, g, layout=layout, dtype=dtype), "gamma")
+
+
+@pytest.mark.parametrize("layout,dtype", COMBOS)
+def test_whole_frames_run_as_rows_of_512_pixels(ctx, layout, dtype):
+    """Batches in which every sample is a whole frame (64 x 96 = 12 rows of 512 pixels) are handed to the streaming kernels as
+    such rows: the colour family, Gamma, Blend, ColorTemperature, CropMirrorNormalize without a mirror and ToTensor, in every
+    output format, against the oracle; a mirrored sample keeps CropMirrorNormalize on the image's own rows."""
+    n, h, w = 5, 64, 96
+    rng = np.random.default_rng(1234 + 10 * layout + dtype)
+    img = rng.integers(0, 256, (n, h, w, 3), dtype=np.uint8)
+    img2 = rng.integers(0, 256, (n, h, w, 3), dtype=np.uint8)
+    roi = np.tile(np.array([0, 0, w, h], np.uint32), (n, 1))
+    f = lambda lo, hi: rng.uniform(lo, hi, n).astype(np.float32)
+    gamma, factor, adj, ratio = f(0.3, 3.0), f(-1.0, 1.5), rng.integers(-60, 61, n).astype(np.int32), f(0.0, 1.0)
+    alpha, beta, hue, sat = f(0.6, 1.4), f(-20, 20), f(-180, 180), f(0.2, 1.8)
+    kw = dict(layout=layout, dtype=dtype)
+    cases = [
+        (ops.Gamma, lambda op: op.update(roi, gamma), (img,), orc.gamma(img, roi, gamma, **kw)),
+        (ops.Blend, lambda op: op.update(roi, ratio), (img, img2), orc.blend(img, img2, roi, ratio, **kw)),
+        (ops.Exposure, lambda op: op.update(roi, factor), (img,), orc.exposure(img, roi, factor, **kw)),
+        (ops.ColorTemperature, lambda op: op.update(roi, adj), (img,), orc.color_temperature(img, roi, adj, **kw)),
+        (ops.Brightness, lambda op: op.update(roi, alpha, beta), (img,), orc.brightness(img, roi, alpha, beta, **kw)),
+        (ops.ColorTwist, lambda op: op.update(roi, alpha, beta, hue, sat), (img,), orc.color_twist(img, roi, alpha, beta, hue, sat, **kw)),
+    ]
+    for cls, upd, srcs, exp in cases:
+        got, op = _run(ctx, cls, n, h, w, layout, dtype, upd, srcs)
+        assert "flat_rows=12" in op.plan, (cls.__name__, op.plan)
+        _same(got, exp, "%s as rows of 512 pixels" % cls.__name__)
+    # CropMirrorNormalize of whole frames: as rows of 512 pixels without a mirror, on the image's rows with one
+    scale = rng.uniform(0.01, 0.03, (n, 3)).astype(np.float32)
+    bias = rng.uniform(-1.0, 1.0, (n, 3)).astype(np.float32)
+    if dtype == ops.UINT8:
+        scale, bias = np.ones((n, 3), np.float32), rng.integers(-20, 20, (n, 3)).astype(np.float32)
+    for mirror in (np.zeros(n, np.uint32), np.array([0, 1, 0, 0, 1], np.uint32)):
+        got, op = _run(ctx, ops.CropMirrorNormalize, n, h, w, layout, dtype, lambda op: op.update(roi, scale, bias, mirror), (img,))
+        assert ("flat_rows=12" in op.plan) == (not mirror.any()), op.plan
+        _same(got, orc.crop_mirror_normalize(img, roi, scale, bias, mirror, h, w, layout, dtype), "CropMirrorNormalize mirror=%s" % mirror.tolist())
+    if dtype != ops.UINT8:
+        mul, add = np.array([0.5, 0.25, 2.0], np.float32), np.array([-3.0, 7.5, 0.125], np.float32)
+        for rev in (False, True):
+            op = ops.ToTensor(ctx, ops.desc(n, h, w, ops.NHWC, ops.UINT8), ops.desc(n, h, w, layout, dtype))
+            op.update(mul, add, rev)
+            assert "flat_rows=12" in op.plan, op.plan
+            out = op.alloc_output()
+            op.launch(_gpu(img), out)
+            ctx.sync()
+            _same(out.cpu().numpy(), orc.to_tensor(img, mul, add, rev, layout, dtype), "ToTensor reverse=%s" % rev)
